@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Benchmark of the GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
+
+A step is one gemm launch over one set of synthetic operands already resident in HBM.  The
+headline workload is bf16 M=N=K=8192, Normal(0,1) operands (the configuration the metric is
+quoted on); fp8 8192^3, bf16 4096^3, fp16 512^3 and the skinny projection shapes are timed with
+fewer steps and reported under "extras".  Prints ONE JSON line.
+
+Protocol follows the reference's benchmark (kernels/tests/gemm_bench.py:285-295, :502-506):
+warm-up, then timed launches, TFLOP/s = 2*M*N*K / t — with HIP events on the launch stream
+instead of wall-clock around each launch, and operand sets rotated for the memory-bound shapes
+so they are not served from the 256 MB Infinity Cache.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "cute-examples_amd"))
+
+METRIC = "GEMM TFLOP/s and % of MI355X dense MFMA peak, bf16 8192^3 and fp8 8192^3"
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "e4m3": 5000.0}   # dense MFMA, MI355X
+PEAK_HBM_GBS = 8000.0
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=50)
+    p.add_argument("--warmup", type=int, default=10)
+    p.add_argument("--workload", default="bf16_8192")
+    p.add_argument("--variant", default="auto")
+    p.add_argument("--no-extras", action="store_true")
+    p.add_argument("--no-cpu", action="store_true")
+    return p.parse_args()
+
+
+def time_calls(call, steps, warmup):
+    """HIP events on the current stream around `steps` back-to-back launches -> ms per launch."""
+    import torch
+    for _ in range(warmup):
+        call()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        call()
+    e1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return e0.elapsed_time(e1) / steps, wall_ms
+
+
+def build_case(name, variant, device="cuda", seed=0):
+    import torch
+    import gemm_kernels
+    from gemm_kernels import workloads as w
+
+    rot = 1
+    if name == "bf16_8192":
+        A, B = w.bf16_8192(seed, device)
+        sets, tag, fp8 = [(A, B)], "bf16", None
+    elif name == "bf16_4096":
+        sets, tag, fp8 = [w.bf16_4096(seed + 10 * i, device) for i in range(4)], "bf16", None
+    elif name == "fp16_512":
+        sets, tag, fp8 = [w.fp16_512(seed, device)], "f16", None
+    elif name == "fp8_8192":
+        A, B, sa, sb = w.fp8_8192(seed, device)
+        sets, tag, fp8 = [(A, B)], "e4m3", (float(sa), float(sb))
+    elif name.startswith("skinny_"):
+        M, N, K = (int(x) for x in name.split("_")[1:])
+        # rotate operand sets so weights come from HBM, not the Infinity Cache (256 MB)
+        rot = max(2, int(600e6 // (N * K * 2)) + 1)
+        sets, tag, fp8 = [w.skinny(M, N, K, seed + 10 * i, device) for i in range(rot)], "bf16", None
+    else:
+        raise SystemExit("unknown workload " + name)
+    M, K = sets[0][0].shape
+    N = sets[0][1].shape[0]
+    out_dt = torch.bfloat16 if fp8 else sets[0][0].dtype
+    C = torch.empty((M, N), dtype=out_dt, device=device)
+    state = {"i": 0}
+
+    def call():
+        A, B = sets[state["i"] % len(sets)]
+        state["i"] += 1
+        if fp8:
+            gemm_kernels.gemm_tn_fp8(A, B, fp8[0], fp8[1], C, variant)
+        else:
+            gemm_kernels.gemm_tn(A, B, C, variant)
+
+    es = sets[0][0].element_size()
+    nbytes = (M * K + N * K) * es + M * N * C.element_size()
+    return call, 2.0 * M * N * K, nbytes, tag, (M, N, K), sets, C, fp8
+
+
+def measure(name, variant, steps, warmup):
+    call, flops, nbytes, tag, mnk, sets, C, fp8 = build_case(name, variant)
+    ms, wall_ms = time_calls(call, steps, warmup)
+    tflops = flops / ms / 1e9
+    row = {"workload": name, "M": mnk[0], "N": mnk[1], "K": mnk[2], "dtype": tag, "steps": steps,
+           "ms": round(ms, 5), "wall_ms": round(wall_ms, 5), "tflops": round(tflops, 2),
+           "pct_mfma_peak": round(100 * tflops / PEAK_TFLOPS[tag], 2),
+           "gbs": round(nbytes / ms / 1e6, 1), "pct_hbm_peak": round(100 * nbytes / ms / 1e6 / PEAK_HBM_GBS, 2)}
+    return row, (sets, C, fp8, flops, nbytes)
+
+
+def cpu_baseline(A, B, budget_s=12.0):
+    """The oracle's fp32 matmul (the reference's ground truth, gemm_test.py:36) timed on the host
+    cores on a bounded sample: as many row blocks of A against all of B as fit the budget."""
+    import torch
+    from oracle import oracle
+    Bc = B.cpu()
+    N, K = Bc.shape
+    rows = min(1024, A.shape[0])
+    Ac = A[:rows].cpu()
+    oracle.gemm_tn_fp32(Ac[:64], Bc)            # warm-up (thread pool, conversions)
+    t0 = time.perf_counter()
+    done = 0
+    while True:
+        oracle.gemm_tn_fp32(Ac, Bc)
+        done += rows
+        el = time.perf_counter() - t0
+        if el > budget_s or done >= 8 * A.shape[0]:
+            break
+    tflops = 2.0 * done * N * K / el / 1e12
+    return {"value": round(tflops, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": "torch.matmul fp32 (incl. bf16->fp32 casts) of %d-row blocks of A against all of B "
+                      "(N=%d, K=%d), %d rows in %.1f s; host has %d logical cpus"
+                      % (rows, N, K, done, el, os.cpu_count())}
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this library is a single-GPU GEMM; --gpus %d is not supported "
+              "(run with --gpus 1)" % a.gpus, file=sys.stderr)
+        raise SystemExit(2)
+    import torch
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    import gemm_kernels
+
+    head, keep = measure(a.workload, a.variant, a.steps, a.warmup)
+    sets, C, fp8, flops, nbytes = keep
+    mfma_bound = not a.workload.startswith("skinny_")
+    if mfma_bound:
+        roof = {"bound": "mfma", "achieved": head["tflops"], "peak": PEAK_TFLOPS[head["dtype"]],
+                "unit": "TFLOP/s", "frac": round(head["tflops"] / PEAK_TFLOPS[head["dtype"]], 4),
+                "traffic": None}
+    else:
+        roof = {"bound": "hbm", "achieved": head["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(head["gbs"] / PEAK_HBM_GBS, 4), "traffic": None}
+    roof["kernel"] = gemm_kernels.select_variant(head["M"], head["N"], head["K"], sets[0][0].dtype) \
+        if a.variant == "auto" else a.variant
+    roof["flops_per_launch"] = flops
+    roof["algorithmic_bytes_per_launch"] = nbytes
+    roof["avg_launch_ms"] = head["ms"]
+
+    cpu = None
+    if not a.no_cpu:
+        cpu = cpu_baseline(sets[0][0], sets[0][1])
+    del sets, C, keep
+    torch.cuda.empty_cache()
+
+    extras = []
+    if not a.no_extras:
+        names = ["bf16_8192", "fp8_8192", "bf16_4096", "fp16_512"] + \
+                ["skinny_%d_%d_%d" % (m, n, k) for (n, k) in ((14336, 4096), (4096, 14336), (6144, 4096))
+                 for m in (16, 64, 256)]
+        for n in names:
+            if n == a.workload:
+                continue
+            steps = 30 if "8192" in n else 100
+            row, keep = measure(n, "auto", steps, 5)
+            extras.append(row)
+            del keep
+            torch.cuda.empty_cache()
+        if a.workload == "bf16_8192" and a.variant == "auto":
+            for v in ("basic", "pingpong"):
+                row, keep = measure("bf16_8192", v, 30, 5)
+                row["variant"] = v
+                extras.append(row)
+                del keep
+                torch.cuda.empty_cache()
+
+    out = {
+        "metric": METRIC, "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": a.steps, "warmup": a.warmup, "ms_per_step": head["ms"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic",
+        "config": {"workload": "%s: M=%d N=%d K=%d, A (M,K) and B (N,K) K-contiguous, fp32 accumulate"
+                               % (a.workload, head["M"], head["N"], head["K"]),
+                   "variant": roof["kernel"], "parallelism": "single GPU"},
+        "pct_of_dense_mfma_peak": head["pct_mfma_peak"],
+        "roofline": roof, "cpu_baseline": cpu, "extras": extras,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,78 @@
+"""Build the gfx950 kernel library and the gemm_kernels._C extension in-tree.
+
+    python cute-examples_amd/build.py            # both
+    python cute-examples_amd/build.py --lib-only  # libmi355gemm.so only (no torch headers needed)
+
+Outputs land in cute-examples_amd/gemm_kernels/: libmi355gemm.so (the C ABI of
+include/mi355_gemm.h) and _C.<abi>.so (the torch binding, linked against it via $ORIGIN).
+Counterpart in the reference: kernels/setup.py:8-28 + build.sh:1-7.
+"""
+import os
+import subprocess
+import sys
+import sysconfig
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OUT = os.path.join(HERE, "gemm_kernels")
+LIB = os.path.join(OUT, "libmi355gemm.so")
+
+HIP_SOURCES = ["gemm_api.hip", "gemm_tn_simple.hip", "gemm_tn_tile256.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
+]
+
+
+def _run(cmd):
+    print("+", " ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    # hipcc's host pass does not know the packed-fp32 target feature and says so once per file.
+    for line in proc.stdout.splitlines():
+        if "packed-fp32-ops" not in line:
+            print(line)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed (%d): %s" % (proc.returncode, " ".join(cmd)))
+
+
+def build_lib():
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    _run([hipcc] + HIPCC_FLAGS + ["-o", LIB] + [os.path.join(CSRC, s) for s in HIP_SOURCES])
+    return LIB
+
+
+def ext_path():
+    return os.path.join(OUT, "_C" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_ext():
+    import pybind11
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_C",
+           "-DTORCH_API_INCLUDE_EXTENSION_H",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           "-Wno-deprecated-declarations"]
+    for inc in ce.include_paths("cuda") + [sysconfig.get_paths()["include"], pybind11.get_include()]:
+        cmd += ["-isystem", inc]
+    cmd += ["-o", ext_path(), os.path.join(CSRC, "torch_binding.cpp"),
+            "-L" + OUT, "-l:libmi355gemm.so", "-L" + tlib, "-L/opt/rocm/lib",
+            "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python", "-lc10", "-lc10_hip", "-lamdhip64",
+            "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + tlib, "-Wl,-rpath,/opt/rocm/lib"]
+    _run(cmd)
+    return ext_path()
+
+
+def main(argv):
+    build_lib()
+    if "--lib-only" not in argv:
+        build_ext()
+
+
+if __name__ == "__main__":
+    main(sys.argv[1:])

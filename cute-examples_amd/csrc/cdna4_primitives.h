@@ -1,0 +1,136 @@
+// Device-side building blocks for gfx950 (CDNA4): buffer resources, direct global->LDS loads,
+// MFMA wrappers per element type, and fp32 -> 16-bit round-to-nearest-even conversion.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi355 {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+
+// Element-type tags.  kBytes = bytes per element; kSliceChunks = 16-byte chunks of one operand
+// row that a single lane feeds into one 32x32 MFMA (1 for 16-bit types: 8 elements; 2 for fp8:
+// 32 elements).
+struct BF16 { static constexpr int kBytes = 2; static constexpr int kSliceChunks = 1; };
+struct F16  { static constexpr int kBytes = 2; static constexpr int kSliceChunks = 1; };
+struct E4M3 { static constexpr int kBytes = 1; static constexpr int kSliceChunks = 2; };
+
+// Raw (unstructured) buffer descriptor over [base, base+bytes): loads beyond `bytes` return 0,
+// which is how ragged tile edges are handled.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_raw_buffer(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+// One wave copies 64 x 16 B from global memory straight into LDS.  Lane l's 16 bytes come from
+// buffer offset voffset(l) + soffset and land at LDS byte address lds_base + 16*l (lds_base is
+// wave-uniform).  Completion is tracked by the wave's vmcnt counter; the compiler does not see
+// the LDS write, so callers order it with wait_vmcnt<N>() and a workgroup barrier.
+__device__ __forceinline__ void dma_16B_to_lds(uint32_t lds_base, uint32_t voffset,
+                                               __amdgpu_buffer_rsrc_t rsrc, uint32_t soffset) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %1, %2, %3 offen lds"
+      :
+      : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
+      : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return (uint32_t)(uintptr_t)p;
+}
+
+// acc += X · Y^T for one 32x32 block.  x holds the block's "row" operand (lane%32 = row index,
+// lane/32 selects which k-chunks), y the "column" operand; result register r of lane l is
+// D[8*(r/4) + 4*(l/32) + r%4][l%32].
+template <class T> struct Mfma32;
+
+template <> struct Mfma32<BF16> {
+  typedef i32x4 Frag;
+  static __device__ __forceinline__ f32x16 run(Frag x, Frag y, f32x16 acc) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x),
+                                                   __builtin_bit_cast(bf16x8, y), acc, 0, 0, 0);
+  }
+};
+template <> struct Mfma32<F16> {
+  typedef i32x4 Frag;
+  static __device__ __forceinline__ f32x16 run(Frag x, Frag y, f32x16 acc) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, x),
+                                                  __builtin_bit_cast(f16x8, y), acc, 0, 0, 0);
+  }
+};
+template <> struct Mfma32<E4M3> {
+  typedef i32x8 Frag;
+  static __device__ __forceinline__ f32x16 run(Frag x, Frag y, f32x16 acc) {
+    // cbsz = blgp = 0 selects e4m3 for both operands; zero scale operands select the unscaled
+    // form of the instruction.
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, acc, 0, 0, 0, 0, 0, 0);
+  }
+};
+
+// Four fp32 -> four 16-bit values (round to nearest even), packed into 8 bytes.
+template <class OutT> struct Pack4;
+template <> struct Pack4<BF16> {
+  static __device__ __forceinline__ u32x2 run(float a, float b, float c, float d) {
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf2;
+    typedef __attribute__((ext_vector_type(2))) float f2;
+    bf2 lo = __builtin_convertvector((f2){a, b}, bf2);
+    bf2 hi = __builtin_convertvector((f2){c, d}, bf2);
+    return (u32x2){__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
+  }
+  static __device__ __forceinline__ uint16_t one(float a) {
+    return __builtin_bit_cast(uint16_t, (__bf16)a);
+  }
+};
+template <> struct Pack4<F16> {
+  static __device__ __forceinline__ u32x2 run(float a, float b, float c, float d) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+    typedef __attribute__((ext_vector_type(2))) float f2;
+    h2 lo = __builtin_convertvector((f2){a, b}, h2);
+    h2 hi = __builtin_convertvector((f2){c, d}, h2);
+    return (u32x2){__builtin_bit_cast(unsigned, lo), __builtin_bit_cast(unsigned, hi)};
+  }
+  static __device__ __forceinline__ uint16_t one(float a) {
+    return __builtin_bit_cast(uint16_t, (_Float16)a);
+  }
+};
+
+// Element -> fp32 for the one-thread-per-output kernel.
+template <class T> struct Decode;
+template <> struct Decode<BF16> {
+  static __device__ __forceinline__ float run(const void* p, int64_t i) {
+    uint32_t u = ((const uint16_t*)p)[i];
+    return __builtin_bit_cast(float, u << 16);
+  }
+};
+template <> struct Decode<F16> {
+  static __device__ __forceinline__ float run(const void* p, int64_t i) {
+    return (float)((const _Float16*)p)[i];
+  }
+};
+template <> struct Decode<E4M3> {
+  // OCP e4m3fn: 1 sign, 4 exponent (bias 7), 3 mantissa bits; no infinities; S.1111.111 = NaN.
+  static __device__ __forceinline__ float run(const void* p, int64_t i) {
+    uint32_t b = ((const uint8_t*)p)[i];
+    uint32_t s = b >> 7, e = (b >> 3) & 15, m = b & 7;
+    float v;
+    if (e == 0) v = (float)m * 0.001953125f;                 // m * 2^-9 (subnormal)
+    else if (e == 15 && m == 7) v = __builtin_nanf("");
+    else v = __builtin_bit_cast(float, ((e + 120u) << 23) | (m << 20));
+    return s ? -v : v;
+  }
+};
+
+}  // namespace mi355

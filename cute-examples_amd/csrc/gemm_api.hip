@@ -1,0 +1,134 @@
+// C ABI of the library (declared in include/mi355_gemm.h): argument validation, variant
+// selection and dispatch.  Validation runs before any HIP call so that it can be exercised on a
+// machine without a GPU.  Counterpart in the reference: the host launcher
+// test::gemm_tn_test, kernels/gemm_kernels/sm90a/gemm_test.cu:12-92.
+#include "../../include/mi355_gemm.h"
+
+#include "gemm_launch.h"
+#include "tile_map.h"
+
+namespace {
+
+int elem_bytes(int dtype) { return dtype == MI355_E4M3 ? 1 : 2; }
+
+bool valid_in(int d) { return d == MI355_BF16 || d == MI355_F16 || d == MI355_E4M3; }
+bool valid_out(int d) { return d == MI355_BF16 || d == MI355_F16; }
+
+// Constraints of the 256x256-tile kernels beyond the generic ones.
+bool tile256_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int in_dtype) {
+  const int64_t es = elem_bytes(in_dtype);
+  if (M <= 0 || N <= 0 || K <= 0) return false;
+  if ((K * es) % 128 != 0) return false;                    // whole k-steps only
+  if ((lda * es) % 16 != 0 || (ldb * es) % 16 != 0) return false;  // 16-byte row chunks
+  if (N % 4 != 0 || ldc % 4 != 0) return false;             // 8-byte output stores
+  if (256 * lda * es >= (int64_t)1 << 32 || 256 * ldb * es >= (int64_t)1 << 32) return false;
+  return true;
+}
+
+int check_common(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                 int in_dtype, int out_dtype, int variant) {
+  if (!valid_in(in_dtype) || !valid_out(out_dtype)) return MI355_ERR_DTYPE;
+  if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_SIMPLE) return MI355_ERR_VARIANT;
+  if (M < 0 || N < 0 || K < 0) return MI355_ERR_SHAPE;
+  if (lda < K || ldb < K || ldc < N) return MI355_ERR_SHAPE;
+  return MI355_OK;
+}
+
+int resolve(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int in_dtype,
+            int variant) {
+  if (variant == MI355_VARIANT_AUTO)
+    return tile256_ok(M, N, K, lda, ldb, ldc, in_dtype) ? MI355_VARIANT_BASIC : MI355_VARIANT_SIMPLE;
+  if (variant == MI355_VARIANT_BASIC || variant == MI355_VARIANT_PINGPONG)
+    return tile256_ok(M, N, K, lda, ldb, ldc, in_dtype) ? variant : MI355_ERR_SHAPE;
+  if (variant == MI355_VARIANT_SKINNY) return MI355_ERR_VARIANT;
+  return variant;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi355_gemm_version(void) { return (0 << 16) | 1; }
+
+const char* mi355_gemm_strerror(int status) {
+  switch (status) {
+    case MI355_OK: return "success";
+    case MI355_ERR_NULL: return "A, B and C must be non-null device pointers";
+    case MI355_ERR_DTYPE: return "unsupported dtype: inputs bf16/fp16/e4m3, output bf16/fp16";
+    case MI355_ERR_SHAPE:
+      return "shape or leading dimension violates a constraint of the requested variant "
+             "(need M,N,K >= 0, lda,ldb >= K, ldc >= N; tiled variants need K*elem_bytes % 128 == 0, "
+             "16-byte aligned rows and N % 4 == 0)";
+    case MI355_ERR_VARIANT: return "unknown variant, or variant not available for this shape/dtype";
+    case MI355_ERR_WORKSPACE: return "workspace is NULL or smaller than mi355_gemm_workspace_bytes()";
+    case MI355_ERR_LAUNCH: return "HIP runtime rejected the kernel launch";
+    case MI355_ERR_ALIGN: return "A and B must be 16-byte aligned and C 8-byte aligned for the tiled variants";
+  }
+  return "unknown status code";
+}
+
+int mi355_gemm_tile_coord(int64_t block, int64_t tiles_m, int64_t tiles_n, int64_t* tile_m,
+                          int64_t* tile_n) {
+  if (!tile_m || !tile_n) return MI355_ERR_NULL;
+  if (tiles_m <= 0 || tiles_n <= 0 || block < 0 || block >= tiles_m * tiles_n) return MI355_ERR_SHAPE;
+  mi355::tile_coord(block, tiles_m, tiles_n, tile_m, tile_n);
+  return MI355_OK;
+}
+
+int mi355_gemm_check(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
+                     int in_dtype, int out_dtype, int variant) {
+  int st = check_common(M, N, K, lda, ldb, ldc, in_dtype, out_dtype, variant);
+  if (st != MI355_OK) return st;
+  int v = resolve(M, N, K, lda, ldb, ldc, in_dtype, variant);
+  return v < 0 ? v : MI355_OK;
+}
+
+int mi355_gemm_select_variant(int64_t M, int64_t N, int64_t K, int in_dtype) {
+  if (!valid_in(in_dtype)) return MI355_ERR_DTYPE;
+  if (M < 0 || N < 0 || K < 0) return MI355_ERR_SHAPE;
+  return resolve(M, N, K, K, K, N, in_dtype, MI355_VARIANT_AUTO);
+}
+
+size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int in_dtype, int variant) {
+  (void)M; (void)N; (void)K; (void)in_dtype; (void)variant;
+  return 0;
+}
+
+int mi355_gemm_tn(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
+                  int64_t lda, int64_t ldb, int64_t ldc, int in_dtype, int out_dtype, float scale,
+                  int variant, void* workspace, size_t workspace_bytes, void* stream) {
+  (void)workspace; (void)workspace_bytes;
+  int st = check_common(M, N, K, lda, ldb, ldc, in_dtype, out_dtype, variant);
+  if (st != MI355_OK) return st;
+  if (M == 0 || N == 0) return MI355_OK;  // nothing to write
+  if (!C || (K > 0 && (!A || !B))) return MI355_ERR_NULL;  // K == 0 reads no operand
+  int v = resolve(M, N, K, lda, ldb, ldc, in_dtype, variant);
+  if (v < 0) return v;
+
+  mi355::GemmArgs g;
+  g.A = A; g.B = B; g.C = C;
+  g.M = M; g.N = N; g.K = K;
+  g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+  g.scale = scale;
+  hipStream_t s = (hipStream_t)stream;
+
+  if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG) {
+    const bool aligned = ((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) && ((uintptr_t)C % 8 == 0);
+    if (!aligned) {
+      if (variant != MI355_VARIANT_AUTO) return MI355_ERR_ALIGN;
+      v = MI355_VARIANT_SIMPLE;
+    }
+  }
+  int rc;
+  if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG) {
+    g.tiles_m = (M + 255) / 256;
+    g.tiles_n = (N + 255) / 256;
+    rc = mi355::launch_tile256(g, in_dtype, out_dtype, v == MI355_VARIANT_PINGPONG, s);
+  } else {
+    g.tiles_m = g.tiles_n = 0;
+    rc = mi355::launch_simple(g, in_dtype, out_dtype, s);
+  }
+  return rc == 0 ? MI355_OK : MI355_ERR_LAUNCH;
+}
+
+}  // extern "C"

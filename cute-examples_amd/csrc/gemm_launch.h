@@ -1,0 +1,24 @@
+// Host-side plumbing shared by the kernel translation units and the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi355 {
+
+// Kernel argument block.  Leading dimensions are in elements.
+struct GemmArgs {
+  const void* A;
+  const void* B;
+  void* C;
+  int64_t M, N, K;
+  int64_t lda, ldb, ldc;
+  int64_t tiles_m, tiles_n;
+  float scale;
+};
+
+// Each returns 0 after a successful enqueue, non-zero if the runtime rejected the launch.
+// in_dtype / out_dtype use the numbering of enum mi355_dtype.
+int launch_tile256(const GemmArgs& g, int in_dtype, int out_dtype, bool pingpong, hipStream_t stream);
+int launch_simple(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
+
+}  // namespace mi355

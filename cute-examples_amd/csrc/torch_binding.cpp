@@ -1,0 +1,151 @@
+// Python module gemm_kernels._C: the thin PyTorch boundary over the C ABI in mi355_gemm.h.
+//
+// Keeps the reference's module name, function name, keyword names and return value
+// (kernels/gemm_kernels/__init__.cpp:4-9: m.def("gemm_tn_test", ..., arg("A"), arg("B"),
+// arg("C")) returning the C tensor) and the argument checks of its host launcher
+// (kernels/gemm_kernels/sm90a/gemm_test.cu:15-41).  Differences, all supersets: fp16 inputs are
+// accepted as well as bf16, C is validated, shapes need not be multiples of the tile, and the
+// launch goes to torch's current stream of A's device instead of the legacy default stream
+// (gemm_test.cu:82-85).  Every check that does not need a GPU runs before the first HIP call.
+#include <torch/extension.h>
+
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include <string>
+
+#include "../../include/mi355_gemm.h"
+
+namespace {
+
+int dtype_code(at::ScalarType t) {
+  switch (t) {
+    case at::kBFloat16: return MI355_BF16;
+    case at::kHalf: return MI355_F16;
+    case at::kFloat8_e4m3fn: return MI355_E4M3;
+    default: return -1;
+  }
+}
+
+int variant_code(const std::string& v) {
+  if (v == "auto") return MI355_VARIANT_AUTO;
+  if (v == "basic") return MI355_VARIANT_BASIC;
+  if (v == "pingpong") return MI355_VARIANT_PINGPONG;
+  if (v == "skinny") return MI355_VARIANT_SKINNY;
+  if (v == "simple") return MI355_VARIANT_SIMPLE;
+  TORCH_CHECK(false, "unknown variant '", v, "' (expected auto, basic, pingpong, skinny or simple)");
+}
+
+const char* variant_name(int v) {
+  switch (v) {
+    case MI355_VARIANT_AUTO: return "auto";
+    case MI355_VARIANT_BASIC: return "basic";
+    case MI355_VARIANT_PINGPONG: return "pingpong";
+    case MI355_VARIANT_SKINNY: return "skinny";
+    case MI355_VARIANT_SIMPLE: return "simple";
+  }
+  return "?";
+}
+
+torch::Tensor run(const torch::Tensor& A, const torch::Tensor& B, torch::Tensor C, float scale,
+                  int variant, bool fp8) {
+  // Same order as the reference's checks (gemm_test.cu:15-28), then the ones it lacks.
+  TORCH_CHECK(A.device() == B.device(), "All tensors must be on the same device");
+  TORCH_CHECK(A.is_contiguous() && B.is_contiguous(), "All tensors must be contiguous");
+  TORCH_CHECK(A.dim() == 2 && B.dim() == 2, "Both tensors must be 2D (matrix) tensors");
+  TORCH_CHECK(A.size(1) == B.size(1), "Inner dimensions of A and B must match (A: ", A.size(1),
+              ", B: ", B.size(1), ")");
+  TORCH_CHECK(A.scalar_type() == B.scalar_type(), "A and B must have the same dtype");
+  const int in_dt = dtype_code(A.scalar_type());
+  if (fp8) {
+    TORCH_CHECK(in_dt == MI355_E4M3, "Both tensors must be of type float8_e4m3fn");
+  } else {
+    TORCH_CHECK(in_dt == MI355_BF16 || in_dt == MI355_F16,
+                "Both tensors must be of type bfloat16 or float16");
+  }
+  const int64_t M = A.size(0), N = B.size(0), K = A.size(1);
+  TORCH_CHECK(C.dim() == 2 && C.size(0) == M && C.size(1) == N, "C must have shape (", M, ", ", N, ")");
+  TORCH_CHECK(C.device() == A.device(), "All tensors must be on the same device");
+  const int out_dt = dtype_code(C.scalar_type());
+  if (fp8) {
+    TORCH_CHECK(out_dt == MI355_BF16 || out_dt == MI355_F16, "C must be bfloat16 or float16");
+  } else {
+    TORCH_CHECK(out_dt == in_dt, "C must have the dtype of A and B");
+  }
+  TORCH_CHECK(N <= 1 || C.stride(1) == 1, "C must be contiguous in its last dimension");
+  const int64_t ldc = M > 1 ? C.stride(0) : N;
+  int st = mi355_gemm_check(M, N, K, K, K, ldc, in_dt, out_dt, variant);
+  TORCH_CHECK(st == MI355_OK, "gemm_kernels: ", mi355_gemm_strerror(st), " [M=", M, " N=", N,
+              " K=", K, " variant=", variant_name(variant), "]");
+  TORCH_CHECK(A.is_cuda(), "gemm_kernels runs on a HIP device only; got tensors on ", A.device());
+
+  if (M == 0 || N == 0) return C;
+  c10::DeviceGuard guard(A.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStream(A.device().index()).stream();
+  const size_t ws_bytes = mi355_gemm_workspace_bytes(M, N, K, in_dt, variant);
+  torch::Tensor ws;
+  void* ws_ptr = nullptr;
+  if (ws_bytes) {
+    // From torch's caching allocator, so the memory is stream-ordered with the launch below.
+    ws = torch::empty({(int64_t)ws_bytes}, A.options().dtype(torch::kUInt8));
+    ws_ptr = ws.data_ptr();
+  }
+  st = mi355_gemm_tn(A.const_data_ptr(), B.const_data_ptr(), C.mutable_data_ptr(), M, N, K, K, K,
+                     ldc, in_dt, out_dt, scale, variant, ws_ptr, ws_bytes, (void*)stream);
+  TORCH_CHECK(st == MI355_OK, "gemm_kernels: ", mi355_gemm_strerror(st));
+  return C;
+}
+
+float scalar_of(const pybind11::object& o) {
+  if (THPVariable_Check(o.ptr())) {
+    const torch::Tensor& t = THPVariable_Unpack(o.ptr());
+    TORCH_CHECK(t.numel() == 1, "a scale tensor must hold exactly one element");
+    return t.item<float>();
+  }
+  return o.cast<float>();
+}
+
+}  // namespace
+
+namespace test {
+
+// C = A · B^T, A (M,K) and B (N,K) contiguous bf16 or fp16, C (M,N) of the same dtype.
+torch::Tensor gemm_tn_test(const torch::Tensor A, const torch::Tensor B, torch::Tensor C) {
+  return run(A, B, C, 1.0f, MI355_VARIANT_AUTO, false);
+}
+
+torch::Tensor gemm_tn(const torch::Tensor A, const torch::Tensor B, torch::Tensor C,
+                      const std::string& variant) {
+  return run(A, B, C, 1.0f, variant_code(variant), false);
+}
+
+// C = (scale_a*scale_b) * A_q · B_q^T for per-tensor-scaled float8_e4m3fn operands.
+torch::Tensor gemm_tn_fp8(const torch::Tensor A_q, const torch::Tensor B_q, pybind11::object scale_a,
+                          pybind11::object scale_b, torch::Tensor C, const std::string& variant) {
+  return run(A_q, B_q, C, scalar_of(scale_a) * scalar_of(scale_b), variant_code(variant), true);
+}
+
+std::string select_variant(int64_t M, int64_t N, int64_t K, at::ScalarType dtype) {
+  const int dt = dtype_code(dtype);
+  TORCH_CHECK(dt >= 0, "dtype must be bfloat16, float16 or float8_e4m3fn");
+  const int v = mi355_gemm_select_variant(M, N, K, dt);
+  TORCH_CHECK(v >= 0, "gemm_kernels: ", mi355_gemm_strerror(v));
+  return variant_name(v);
+}
+
+}  // namespace test
+
+PYBIND11_MODULE(_C, m) {
+  namespace py = pybind11;
+  m.def("gemm_tn_test", &test::gemm_tn_test, "C = A @ B.T (bf16/fp16 in and out, fp32 accumulate)",
+        py::arg("A"), py::arg("B"), py::arg("C"));
+  m.def("gemm_tn", &test::gemm_tn, "gemm_tn_test with an explicit kernel variant", py::arg("A"),
+        py::arg("B"), py::arg("C"), py::arg("variant") = "auto");
+  m.def("gemm_tn_fp8", &test::gemm_tn_fp8,
+        "C = scale_a*scale_b * A_q @ B_q.T for float8_e4m3fn operands, bf16/fp16 out",
+        py::arg("A_q"), py::arg("B_q"), py::arg("scale_a"), py::arg("scale_b"), py::arg("C"),
+        py::arg("variant") = "auto");
+  m.def("select_variant", &test::select_variant, py::arg("M"), py::arg("N"), py::arg("K"),
+        py::arg("dtype"));
+  m.def("version", []() { return mi355_gemm_version(); });
+}

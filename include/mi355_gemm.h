@@ -1,0 +1,116 @@
+/*
+ * mi355_gemm.h — C ABI of the MI355X (gfx950) dense GEMM library.
+ *
+ * Every entry point computes C[M,N] = scale * A[M,K] · B[N,K]^T with both operands
+ * K-contiguous ("TN"), fp32 accumulation on the matrix cores and a round-to-nearest-even
+ * down-conversion of the result.  Pointers are device pointers; nothing here allocates,
+ * synchronises or touches global mutable state, so calls are re-entrant and may be issued
+ * from several host threads on different streams.
+ *
+ * The functions replace the reference's host launcher
+ *   test::gemm_tn_test(const torch::Tensor A, const torch::Tensor B, torch::Tensor C)
+ *   (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92, bound at
+ *    kernels/gemm_kernels/__init__.cpp:7-8)
+ * with plain pointers and sizes so that any host language can bind them.
+ */
+#ifndef MI355_GEMM_H
+#define MI355_GEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types.  Inputs: BF16, F16, E4M3 (OCP e4m3fn, max 448).  Outputs: BF16, F16. */
+enum mi355_dtype {
+  MI355_BF16 = 0,
+  MI355_F16 = 1,
+  MI355_E4M3 = 2
+};
+
+/* Kernel families.  AUTO picks by shape; the others force one family (and fail with
+ * MI355_ERR_SHAPE when the shape does not meet that family's constraints). */
+enum mi355_variant {
+  MI355_VARIANT_AUTO = 0,
+  MI355_VARIANT_BASIC = 1,    /* 256x256 tile, one wave group in lock step, LDS double buffer */
+  MI355_VARIANT_PINGPONG = 2, /* same tile, two wave groups alternating MFMA and load phases   */
+  MI355_VARIANT_SKINNY = 3,   /* small-M weight-streaming kernel with split-K                  */
+  MI355_VARIANT_SIMPLE = 4    /* one thread per output element; any shape; slow; self-check    */
+};
+
+/* Status codes (0 = success, negative = error; see mi355_gemm_strerror). */
+enum mi355_status {
+  MI355_OK = 0,
+  MI355_ERR_NULL = -1,      /* a required pointer is NULL                                   */
+  MI355_ERR_DTYPE = -2,     /* unsupported input/output dtype combination                   */
+  MI355_ERR_SHAPE = -3,     /* M, N, K or a leading dimension violates a constraint         */
+  MI355_ERR_VARIANT = -4,   /* unknown variant, or variant cannot run this shape/dtype      */
+  MI355_ERR_WORKSPACE = -5, /* workspace missing or smaller than mi355_gemm_workspace_bytes */
+  MI355_ERR_LAUNCH = -6,    /* the HIP runtime refused the launch                           */
+  MI355_ERR_ALIGN = -7      /* a pointer or leading dimension is not 16-byte aligned        */
+};
+
+/*
+ * C = scale * A · B^T.
+ *
+ *   A         device pointer, M rows of K elements, row stride lda (elements)
+ *   B         device pointer, N rows of K elements, row stride ldb (elements)
+ *   C         device pointer, M rows of N elements, row stride ldc (elements)
+ *   in_dtype  element type of A and B (enum mi355_dtype)
+ *   out_dtype element type of C: MI355_BF16 or MI355_F16
+ *   scale     fp32 factor applied to the fp32 accumulator before the down-conversion
+ *             (1.0f for bf16/fp16; scale_a*scale_b for per-tensor-scaled fp8)
+ *   variant   enum mi355_variant
+ *   workspace device scratch of at least mi355_gemm_workspace_bytes(...) bytes, or NULL when
+ *             that function returns 0; contents need not be initialised
+ *   stream    hipStream_t on which the kernels are enqueued (NULL = the null stream)
+ *
+ * Replaces test::gemm_tn_test (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92): same operand
+ * layout and the argument checks of :15-41, plus checks of C the reference omits; divisibility
+ * by the tile is not required.  Asynchronous: returns after enqueueing.
+ */
+int mi355_gemm_tn(const void *A, const void *B, void *C,
+                  int64_t M, int64_t N, int64_t K,
+                  int64_t lda, int64_t ldb, int64_t ldc,
+                  int in_dtype, int out_dtype, float scale, int variant,
+                  void *workspace, size_t workspace_bytes, void *stream);
+
+/* Scratch bytes mi355_gemm_tn needs for this problem and variant (0 for most shapes).
+ * Counterpart: none in the reference (it has no split-K); sizes the split-K partials that
+ * replace the reference's single-pass accumulation (gemm.cuh:352-367) on skinny shapes. */
+size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K,
+                                  int in_dtype, int variant);
+
+/* The variant MI355_VARIANT_AUTO resolves to for this problem (an enum mi355_variant value),
+ * or a negative mi355_status.  Replaces the compile-time choice of kernel header at
+ * kernels/gemm_kernels/sm90a/gemm_test.cu:7 / kernels/setup.py:12-15. */
+int mi355_gemm_select_variant(int64_t M, int64_t N, int64_t K, int in_dtype);
+
+/* Argument validation only, no HIP call: returns what mi355_gemm_tn would return before it
+ * touches the device.  Mirrors the TORCH_CHECK block at gemm_test.cu:15-41. */
+int mi355_gemm_check(int64_t M, int64_t N, int64_t K,
+                     int64_t lda, int64_t ldb, int64_t ldc,
+                     int in_dtype, int out_dtype, int variant);
+
+/* Output tile a workgroup computes: block index -> (tile_m, tile_n) for a tiles_m x tiles_n
+ * grid.  Pure integer function, callable without a GPU.  Replaces Scheduler::
+ * get_swizzled_block_idx (kernels/gemm_kernels/sm90a/gemm.cuh:184-197): same contract
+ * (a bijection onto the tile grid that keeps co-resident workgroups on neighbouring tiles),
+ * re-derived for 8 XCDs with private L2s.  Returns 0, or MI355_ERR_SHAPE if block is out of
+ * range. */
+int mi355_gemm_tile_coord(int64_t block, int64_t tiles_m, int64_t tiles_n,
+                          int64_t *tile_m, int64_t *tile_n);
+
+/* Human-readable text for a status code; never NULL.  Replaces the TORCH_CHECK messages of
+ * gemm_test.cu:15-41 and the stderr print of :88-90. */
+const char *mi355_gemm_strerror(int status);
+
+/* Library version, (major << 16) | minor. */
+int mi355_gemm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_GEMM_H */

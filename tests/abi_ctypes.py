@@ -1,0 +1,62 @@
+"""ctypes view of include/mi355_gemm.h for the tests (and a model of the stub a non-Python host
+would write).  Loads the in-tree library; raises if it has not been built."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "cute-examples_amd", "gemm_kernels", "libmi355gemm.so")
+HEADER = os.path.join(ROOT, "include", "mi355_gemm.h")
+
+BF16, F16, E4M3 = 0, 1, 2
+AUTO, BASIC, PINGPONG, SKINNY, SIMPLE = 0, 1, 2, 3, 4
+OK, ERR_NULL, ERR_DTYPE, ERR_SHAPE, ERR_VARIANT, ERR_WORKSPACE, ERR_LAUNCH, ERR_ALIGN = 0, -1, -2, -3, -4, -5, -6, -7
+
+
+def declared_symbols():
+    """Function names declared in the public header."""
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355_gemm\w*)\s*\(", text)))
+
+
+def load():
+    if not os.path.exists(LIB):
+        raise RuntimeError("libmi355gemm.so is not built; run python cute-examples_amd/build.py")
+    L = ctypes.CDLL(LIB)
+    i64, vp, ci, f32, sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
+    L.mi355_gemm_tn.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, f32, ci, vp, sz, vp]
+    L.mi355_gemm_tn.restype = ci
+    L.mi355_gemm_workspace_bytes.argtypes = [i64, i64, i64, ci, ci]
+    L.mi355_gemm_workspace_bytes.restype = sz
+    L.mi355_gemm_select_variant.argtypes = [i64, i64, i64, ci]
+    L.mi355_gemm_select_variant.restype = ci
+    L.mi355_gemm_check.argtypes = [i64, i64, i64, i64, i64, i64, ci, ci, ci]
+    L.mi355_gemm_check.restype = ci
+    L.mi355_gemm_tile_coord.argtypes = [i64, i64, i64, ctypes.POINTER(i64), ctypes.POINTER(i64)]
+    L.mi355_gemm_tile_coord.restype = ci
+    L.mi355_gemm_strerror.argtypes = [ci]
+    L.mi355_gemm_strerror.restype = ctypes.c_char_p
+    L.mi355_gemm_version.argtypes = []
+    L.mi355_gemm_version.restype = ci
+    return L
+
+
+def torch_code(dtype):
+    import torch
+    return {torch.bfloat16: BF16, torch.float16: F16, torch.float8_e4m3fn: E4M3}[dtype]
+
+
+def gemm_tn(L, A, B, C, scale=1.0, variant=AUTO, stream=None):
+    """Call mi355_gemm_tn on torch device tensors through the C ABI (no torch types cross it)."""
+    import torch
+    M, K = A.shape
+    N = B.shape[0]
+    in_dt, out_dt = torch_code(A.dtype), torch_code(C.dtype)
+    ws_bytes = L.mi355_gemm_workspace_bytes(M, N, K, in_dt, variant)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=A.device) if ws_bytes else None
+    s = stream if stream is not None else torch.cuda.current_stream().cuda_stream
+    rc = L.mi355_gemm_tn(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0),
+                         C.stride(0), in_dt, out_dt, scale, variant,
+                         ws.data_ptr() if ws is not None else None, ws_bytes, s)
+    return rc

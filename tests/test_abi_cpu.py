@@ -1,0 +1,87 @@
+"""The C-ABI library on a machine without a GPU: it loads, exports every symbol the public
+header declares, validates arguments before touching the device, and its tile map is a
+bijection (the invariant of the reference's Scheduler, kernels/gemm_kernels/sm90a/gemm.cuh:184-211)."""
+import ctypes
+import subprocess
+
+import pytest
+
+from tests import abi_ctypes as ac
+
+
+def test_exports_every_declared_symbol(abi):
+    names = ac.declared_symbols()
+    assert "mi355_gemm_tn" in names and len(names) >= 7
+    for n in names:
+        assert hasattr(abi, n), n
+    dyn = subprocess.run(["nm", "-D", "--defined-only", ac.LIB], capture_output=True, text=True).stdout
+    for n in names:
+        assert f" T {n}" in dyn, n
+
+
+def test_version_and_strerror(abi):
+    assert abi.mi355_gemm_version() >= 1
+    for code in range(0, -8, -1):
+        msg = abi.mi355_gemm_strerror(code)
+        assert msg and b"unknown status" not in msg
+    assert b"unknown status" in abi.mi355_gemm_strerror(-99)
+
+
+@pytest.mark.parametrize("args,want", [
+    ((256, 256, 64, 64, 64, 256, ac.BF16, ac.BF16, ac.AUTO), ac.OK),
+    ((256, 256, 64, 64, 64, 256, 7, ac.BF16, ac.AUTO), ac.ERR_DTYPE),
+    ((256, 256, 64, 64, 64, 256, ac.BF16, ac.E4M3, ac.AUTO), ac.ERR_DTYPE),
+    ((256, 256, 64, 64, 64, 256, ac.BF16, ac.BF16, 9), ac.ERR_VARIANT),
+    ((-1, 256, 64, 64, 64, 256, ac.BF16, ac.BF16, ac.AUTO), ac.ERR_SHAPE),
+    ((256, 256, 64, 32, 64, 256, ac.BF16, ac.BF16, ac.AUTO), ac.ERR_SHAPE),   # lda < K
+    ((256, 256, 64, 64, 64, 128, ac.BF16, ac.BF16, ac.AUTO), ac.ERR_SHAPE),   # ldc < N
+    ((256, 256, 72, 72, 72, 256, ac.BF16, ac.BF16, ac.BASIC), ac.ERR_SHAPE),  # K bytes % 128
+    ((256, 256, 72, 72, 72, 256, ac.BF16, ac.BF16, ac.AUTO), ac.OK),          # AUTO falls back
+    ((16, 30, 7, 7, 7, 30, ac.F16, ac.F16, ac.SIMPLE), ac.OK),
+    ((256, 256, 128, 128, 128, 256, ac.E4M3, ac.BF16, ac.BASIC), ac.OK),
+    ((256, 256, 64, 64, 64, 256, ac.E4M3, ac.BF16, ac.BASIC), ac.ERR_SHAPE),  # 64 fp8 bytes < k-step
+    ((0, 0, 0, 0, 0, 0, ac.BF16, ac.BF16, ac.AUTO), ac.OK),
+])
+def test_check(abi, args, want):
+    assert abi.mi355_gemm_check(*args) == want
+
+
+def test_gemm_tn_rejects_before_any_device_access(abi):
+    """Bad arguments and NULL pointers come back as codes without a GPU present."""
+    f = abi.mi355_gemm_tn
+    assert f(None, None, None, 256, 256, 64, 64, 64, 256, 0, 0, 1.0, 0, None, 0, None) == ac.ERR_NULL
+    assert f(None, None, None, 256, 256, 64, 64, 64, 256, 5, 0, 1.0, 0, None, 0, None) == ac.ERR_DTYPE
+    assert f(None, None, None, 256, 256, 64, 8, 64, 256, 0, 0, 1.0, 0, None, 0, None) == ac.ERR_SHAPE
+    assert f(None, None, None, 0, 256, 64, 64, 64, 256, 0, 0, 1.0, 0, None, 0, None) == ac.OK  # empty
+
+
+def test_select_variant(abi):
+    assert abi.mi355_gemm_select_variant(8192, 8192, 8192, ac.BF16) in (ac.BASIC, ac.PINGPONG)
+    assert abi.mi355_gemm_select_variant(100, 30, 77, ac.BF16) == ac.SIMPLE
+    assert abi.mi355_gemm_select_variant(8192, 8192, 8192, 9) == ac.ERR_DTYPE
+
+
+@pytest.mark.parametrize("tm,tn", [(32, 32), (16, 16), (1, 1), (1, 56), (3, 5), (7, 9), (33, 31), (2, 24), (17, 1)])
+def test_tile_map_is_a_bijection(abi, tm, tn):
+    seen = set()
+    a, b = ctypes.c_int64(), ctypes.c_int64()
+    for blk in range(tm * tn):
+        assert abi.mi355_gemm_tile_coord(blk, tm, tn, ctypes.byref(a), ctypes.byref(b)) == 0
+        assert 0 <= a.value < tm and 0 <= b.value < tn
+        seen.add((a.value, b.value))
+    assert len(seen) == tm * tn
+    assert abi.mi355_gemm_tile_coord(tm * tn, tm, tn, ctypes.byref(a), ctypes.byref(b)) == ac.ERR_SHAPE
+
+
+def test_tile_map_keeps_an_xcd_compact(abi):
+    """Blocks b, b+8, b+16, ... run on one XCD.  The 32 that are co-resident at the start must
+    touch few distinct A and B panels so they share them through that XCD's L2."""
+    tm = tn = 32
+    a, b = ctypes.c_int64(), ctypes.c_int64()
+    for xcd in range(8):
+        rows, cols = set(), set()
+        for i in range(32):
+            abi.mi355_gemm_tile_coord(xcd + 8 * i, tm, tn, ctypes.byref(a), ctypes.byref(b))
+            rows.add(a.value)
+            cols.add(b.value)
+        assert len(rows) + len(cols) <= 12, (xcd, rows, cols)
