@@ -24,7 +24,14 @@ struct E4M3 { static constexpr int kBytes = 1; static constexpr int kSliceChunks
 // Raw (unstructured) buffer descriptor over [base, base+bytes): loads beyond `bytes` return 0,
 // which is how ragged tile edges are handled.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_raw_buffer(const void* base, uint32_t bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+  // The descriptor must live in scalar registers.  The operands are wave-uniform by
+  // construction; readfirstlane makes that visible to the compiler (64-bit address arithmetic
+  // is done on the vector ALU and would otherwise drag the descriptor into vector registers).
+  const uint64_t p = (uint64_t)base;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)p);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(p >> 32));
+  void* q = (void*)(((uint64_t)hi << 32) | lo);
+  return __builtin_amdgcn_make_buffer_rsrc(q, 0, (int)__builtin_amdgcn_readfirstlane(bytes), 0x00020000);
 }
 
 // One wave copies 64 x 16 B from global memory straight into LDS.  Lane l's 16 bytes come from
@@ -40,6 +47,16 @@ __device__ __forceinline__ void dma_16B_to_lds(uint32_t lds_base, uint32_t voffs
       :
       : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
       : "memory");
+}
+
+// Same copy through the compiler's own intrinsic: the compiler then sets M0, tracks the copy in
+// vmcnt against reads of the destination LDS object, and can schedule it like any VMEM load.
+// imm is added to both the buffer offset and the LDS address.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+template <int kImm = 0>
+__device__ __forceinline__ void dma_16B_to_lds_tracked(void* lds_dst, uint32_t voffset,
+                                                       __amdgpu_buffer_rsrc_t rsrc, uint32_t soffset) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)lds_dst, 16, voffset, soffset, kImm, 0);
 }
 
 template <int N>
