@@ -45,7 +45,8 @@ __device__ __forceinline__ void dma_16B_to_lds(uint32_t lds_base, uint32_t voffs
       "s_nop 0\n\t"
       "buffer_load_dwordx4 %1, %2, %3 offen lds"
       :
-      : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset)
+      : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(voffset), "s"(rsrc),
+        "s"(__builtin_amdgcn_readfirstlane(soffset))
       : "memory");
 }
 

@@ -170,6 +170,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
 
 #ifdef MI355_CLOCK_PROBE
   const uint64_t probe_c0 = __builtin_readcyclecounter(), probe_r0 = __builtin_amdgcn_s_memrealtime();
+  uint64_t probe_r_loop = 0;
 #endif
   Acc acc[kNb][kNb];
 #pragma unroll
@@ -215,6 +216,9 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
   for (int q = 0; q < kReadsPerSlice; ++q)
     read_q(0, q, ring + a_lane, ring + kSlotBytes + b_lane, 0);
 
+#ifdef MI355_CLOCK_PROBE
+  probe_r_loop = __builtin_amdgcn_s_memrealtime();
+#endif
   uint32_t slot_a = 0;  // slot of A(t); B(t) is in slot_a+1, A(t+1) in slot_a+2, B(t+1) in slot_a+3 (mod 5)
   for (uint32_t kt = 0; kt < k_steps; ++kt) {
     const uint32_t slot_b = slot_a + 1 >= kSlots ? slot_a + 1 - kSlots : slot_a + 1;
@@ -292,11 +296,18 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
     }
   }
 #ifdef MI355_CLOCK_PROBE
-  // Timing experiments only: the last block overwrites the start of C with cycle counts.
+  // Timing experiments only: every block overwrites 64 bytes of C with time stamps.
   __builtin_amdgcn_s_barrier();
-  if (blockIdx.x == gridDim.x - 1 && tid == 0) {
-    ((uint64_t*)g.C)[0] = probe_c1 - probe_c0;
-    ((uint64_t*)g.C)[1] = probe_r1 - probe_r0;
+  if (tid == 0) {
+    uint64_t* rec = (uint64_t*)g.C + 8 * (uint64_t)blockIdx.x;
+    rec[0] = probe_c1 - probe_c0;
+    rec[1] = probe_r1 - probe_r0;
+    rec[2] = probe_r0;
+    rec[3] = probe_r_loop;
+    rec[4] = probe_r1;
+    rec[5] = __builtin_amdgcn_s_memrealtime();
+    rec[6] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
+    rec[7] = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11));  // XCC_ID
   }
 #endif
 }
