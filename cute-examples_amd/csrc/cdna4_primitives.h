@@ -13,6 +13,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) int i32x4;
 typedef __attribute__((ext_vector_type(8))) int i32x8;
 typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
 
 // Element-type tags.  kBytes = bytes per element; kSliceChunks = 16-byte chunks of one operand
 // row that a single lane feeds into one 32x32 MFMA (1 for 16-bit types: 8 elements; 2 for fp8:

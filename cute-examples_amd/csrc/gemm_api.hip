@@ -123,7 +123,7 @@ int mi355_gemm_tn(const void* A, const void* B, void* C, int64_t M, int64_t N, i
   if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG) {
     g.tiles_m = (M + 255) / 256;
     g.tiles_n = (N + 255) / 256;
-    rc = v == MI355_VARIANT_PINGPONG ? mi355::launch_tile256(g, in_dtype, out_dtype, true, s)
+    rc = v == MI355_VARIANT_PINGPONG ? mi355::launch_tile256_pingpong(g, in_dtype, out_dtype, s)
                                      : mi355::launch_tile256_ring(g, in_dtype, out_dtype, s);
   } else {
     g.tiles_m = g.tiles_n = 0;

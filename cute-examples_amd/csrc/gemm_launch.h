@@ -18,7 +18,7 @@ struct GemmArgs {
 
 // Each returns 0 after a successful enqueue, non-zero if the runtime rejected the launch.
 // in_dtype / out_dtype use the numbering of enum mi355_dtype.
-int launch_tile256(const GemmArgs& g, int in_dtype, int out_dtype, bool pingpong, hipStream_t stream);
+int launch_tile256_pingpong(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
 int launch_tile256_ring(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
 int launch_simple(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
 

@@ -1,0 +1,286 @@
+// "pingpong" variant: 256x256 output tile, TWO wave groups of 4 waves (8 waves, two per SIMD, one
+// of each group).  Group g owns the 128 output columns [128g, 128g+128); inside a group the four
+// waves own 128x64 sub-tiles (128 fp32 accumulator registers per lane).
+//
+// The two groups run the same program one phase apart, so that on every SIMD one wave is in an
+// MFMA phase while the other is in a load phase, and they swap at every workgroup barrier:
+//
+//   phase  group 0                              group 1
+//   4t+0   M0: MFMAs of slice 0, k-step t       L1: LDS reads of slice 0 of t   + copies
+//   4t+1   L0: LDS reads of slice 1 of t        M0: MFMAs of slice 0 of t
+//   4t+2   M1: MFMAs of slice 1 of t            L0: LDS reads of slice 1 of t
+//   4t+3   L1: LDS reads of slice 0 of t+1      M1: MFMAs of slice 1 of t
+//          + copies of B(t+2), A(t+3)
+//
+// A wave's MFMA and load phases never overlap, so its operand fragments are single-buffered: a
+// load phase refills the registers the preceding MFMA phase has just finished with, and the other
+// group's MFMA phase (32 MFMAs, ~512 cycles) hides the LDS latency.  MFMA phases run at raised
+// wave priority.  LDS ring, swizzle, copy geometry and tile walk are those of the single-group
+// kernel (ring_common.h, gemm_tn_ring.hip): five 32 KiB slots, operand-steps queued as
+// A0 B0 A1 B1 A2 ..., the two slots of k-step t refilled with B(t+2), A(t+3) once both groups
+// have read them (end of phase 4t+2).
+//
+// Counterpart in the reference: kernels/gemm_kernels/sm90a/gemm_pingpong.cuh:121-349, where two
+// consumer warpgroups alternate whole output tiles under an ordering barrier (:244-286) so that
+// one's epilogue overlaps the other's MMA.  gfx950 has no asynchronous MMA to overlap with, so
+// here the alternation is between the MFMA and the LDS/global load phases inside the k-loop.
+#include "gemm_launch.h"
+#include "ring_common.h"
+#include "tile_map.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int kThreads = 512;
+
+template <class T, class OutT>
+__global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_pingpong(GemmArgs g) {
+  __shared__ __attribute__((aligned(1024))) uint8_t ring[kSlots * kSlotBytes];
+  typedef Geo<T> G;
+  typedef typename G::Frag Frag;
+  typedef typename G::Acc Acc;
+  constexpr int kBlk = G::kBlk;
+  constexpr int kNbA = 128 / kBlk;                      // A blocks per wave (128 rows)
+  constexpr int kNbB = 64 / kBlk;                       // B blocks per wave (64 columns)
+  constexpr int kSliceChunks = G::kGroups * G::kCpl;
+  constexpr int kSlices = 8 / kSliceChunks;
+  constexpr int kAccLen = kBlk * kBlk / 64;
+  static_assert(kSlices == 2, "the phase table assumes two slices per k-step");
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t group = wave >> 2;            // waves 0-3 and 4-7 land on SIMDs 0-3 each
+  const uint32_t wm = (wave >> 1) & 1u;        // which 128 rows
+  const uint32_t wn = group * 2 + (wave & 1u); // which 64 columns
+
+  const uint32_t lda_b = (uint32_t)(g.lda * T::kBytes), ldb_b = (uint32_t)(g.ldb * T::kBytes);
+  const uint32_t k_bytes = (uint32_t)(g.K * T::kBytes);
+  const uint32_t k_steps = __builtin_amdgcn_readfirstlane(k_bytes / kRowBytes);
+  const int64_t total_tiles = g.tiles_m * g.tiles_n;
+
+  auto panel_a = [&](int64_t m0) __attribute__((always_inline)) {
+    const int64_t rows = g.M - m0 < kTile ? g.M - m0 : kTile;
+    return make_raw_buffer((const uint8_t*)g.A + m0 * (int64_t)lda_b, (uint32_t)((rows - 1) * lda_b + k_bytes));
+  };
+  auto panel_b = [&](int64_t n0) __attribute__((always_inline)) {
+    const int64_t rows = g.N - n0 < kTile ? g.N - n0 : kTile;
+    return make_raw_buffer((const uint8_t*)g.B + n0 * (int64_t)ldb_b, (uint32_t)((rows - 1) * ldb_b + k_bytes));
+  };
+
+  // Copy geometry as in the single-group kernel, but each of the 8 waves moves 32 rows of an
+  // operand per k-step: copies 4w..4w+3 of 8 rows x 128 B.
+  const uint32_t r8 = lane >> 3, c8 = lane & 7u;
+  uint32_t voff_a[2], voff_b[2];
+#pragma unroll
+  for (int par = 0; par < 2; ++par) {
+    const uint32_t chunk = c8 ^ swizzle(par * 8 + r8);
+    voff_a[par] = (wave * 32 + r8) * lda_b + chunk * 16;
+    voff_b[par] = (wave * 32 + r8) * ldb_b + chunk * 16;
+  }
+  const uint32_t a_step = __builtin_amdgcn_readfirstlane(8 * lda_b);
+  const uint32_t b_step = __builtin_amdgcn_readfirstlane(8 * ldb_b);
+  const uint32_t ring0 = __builtin_amdgcn_readfirstlane(lds_address(ring));
+  const uint32_t dma_wave = ring0 + wave * 4096;
+
+  auto copy_a = [&](__amdgpu_buffer_rsrc_t rsrc, int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
+    const uint32_t soff = (kt < k_steps ? kt : k_steps - 1) * kRowBytes;
+    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff_a[j & 1] + j * a_step, rsrc, soff);
+  };
+  auto copy_b = [&](__amdgpu_buffer_rsrc_t rsrc, int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
+    const uint32_t soff = (kt < k_steps ? kt : k_steps - 1) * kRowBytes;
+    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff_b[j & 1] + j * b_step, rsrc, soff);
+  };
+  auto open_tile = [&](__amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) copy_a(ra, j, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) copy_b(rb, j, 1, 0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) copy_a(ra, j, 2, 1);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) copy_b(rb, j, 3, 1);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) copy_a(ra, j, 4, 2);
+  };
+
+  const uint32_t rblk = lane & (kBlk - 1), grp = lane / kBlk;
+  const uint32_t swz = swizzle(rblk);
+  const uint32_t a_lane = (wm * 128 + rblk) * kRowBytes;
+  const uint32_t b_lane = (wn * 64 + rblk) * kRowBytes;
+  auto chunk_off = [&](int s, int e) __attribute__((always_inline)) -> uint32_t {
+    return ((uint32_t)(s * kSliceChunks + grp * G::kCpl + e) ^ swz) << 4;
+  };
+  auto load_frag = [&](const uint8_t* slot_rows, int blk, int s) __attribute__((always_inline)) -> Frag {
+    const uint8_t* p = slot_rows + blk * kBlk * kRowBytes;
+    if constexpr (G::kCpl == 1) {
+      return *(const i32x4*)(p + chunk_off(s, 0));
+    } else {
+      i32x4 lo = *(const i32x4*)(p + chunk_off(s, 0));
+      i32x4 hi = *(const i32x4*)(p + chunk_off(s, 1));
+      return (i32x8){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+  };
+
+  Acc acc[kNbA][kNbB];
+  Frag fa[kNbA], fb[kNbB];
+
+  auto load_phase_reads = [&](const uint8_t* a_rows, const uint8_t* b_rows, int s) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < kNbB; ++j) fb[j] = load_frag(b_rows, j, s);
+#pragma unroll
+    for (int i = 0; i < kNbA; ++i) fa[i] = load_frag(a_rows, i, s);
+  };
+  auto mfma_phase = [&]() __attribute__((always_inline)) {
+    __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+    for (int i = 0; i < kNbA; ++i)
+#pragma unroll
+      for (int j = 0; j < kNbB; ++j) acc[i][j] = G::mfma(fb[j], fa[i], acc[i][j]);
+    __builtin_amdgcn_s_setprio(0);
+  };
+  // Phase boundary: nothing may move across it.
+  auto phase_barrier = [&]() __attribute__((always_inline)) {
+    MI355_FENCE();
+    __builtin_amdgcn_s_barrier();
+    MI355_FENCE();
+  };
+
+  const float scale = g.scale;
+  const int64_t ldc = g.ldc;
+  uint16_t* const C = (uint16_t*)g.C;
+  auto store8 = [&](int64_t m, int64_t n, u32x2 x, u32x2 y) __attribute__((always_inline)) {
+    if (m >= g.M) return;
+    uint16_t* p = C + m * ldc + n;
+    if constexpr (kBlk == 16) {
+      if (n + 8 <= g.N) __builtin_nontemporal_store((u32x4){x[0], x[1], y[0], y[1]}, (u32x4*)p);
+      else if (n + 4 <= g.N) __builtin_nontemporal_store(x, (u32x2*)p);
+    } else {
+      if (n + 8 <= g.N) *(u32x4*)p = (u32x4){x[0], x[1], y[0], y[1]};
+      else if (n + 4 <= g.N) *(u32x2*)p = x;
+    }
+  };
+  auto pack_quad = [&](const Acc& a, int q) __attribute__((always_inline)) -> u32x2 {
+    return Pack4<OutT>::run(a[4 * q] * scale, a[4 * q + 1] * scale, a[4 * q + 2] * scale, a[4 * q + 3] * scale);
+  };
+  // Same register-to-element map and lane-group swaps as the single-group kernel's epilogue.
+  auto epilogue = [&](int64_t m0, int64_t n0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < kNbA; ++i) {
+      const int64_t m = m0 + wm * 128 + i * kBlk + rblk;
+      if constexpr (kBlk == 16) {
+#pragma unroll
+        for (int j = 0; j < kNbB; j += 2) {
+          u32x2 x = pack_quad(acc[i][j], 0), y = pack_quad(acc[i][j + 1], 0);
+          u32x2 lo = __builtin_amdgcn_permlane16_swap(x[0], y[0], false, false);
+          u32x2 hi = __builtin_amdgcn_permlane16_swap(x[1], y[1], false, false);
+          const int64_t n = n0 + wn * 64 + (j + (grp & 1)) * 16 + (grp >> 1) * 8;
+          store8(m, n, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < kNbB; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; q += 2) {
+            u32x2 x = pack_quad(acc[i][j], q), y = pack_quad(acc[i][j], q + 1);
+            u32x2 lo = __builtin_amdgcn_permlane32_swap(x[0], y[0], false, false);
+            u32x2 hi = __builtin_amdgcn_permlane32_swap(x[1], y[1], false, false);
+            const int64_t n = n0 + wn * 64 + j * 32 + (q >> 1) * 16 + grp * 8;
+            store8(m, n, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
+          }
+        }
+      }
+    }
+  };
+
+  int64_t tile = blockIdx.x;
+  int64_t tile_m, tile_n;
+  tile_coord(tile, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+  __amdgpu_buffer_rsrc_t rsrc_a = panel_a(tile_m * kTile), rsrc_b = panel_b(tile_n * kTile);
+  open_tile(rsrc_a, rsrc_b);
+
+  for (;;) {
+#pragma unroll
+    for (int i = 0; i < kNbA; ++i)
+#pragma unroll
+      for (int j = 0; j < kNbB; ++j)
+#pragma unroll
+        for (int r = 0; r < kAccLen; ++r) acc[i][j][r] = 0.f;
+
+    wait_vmcnt<12>();  // A0 and B0 have landed (A1, B1, A2 may be in flight: 3 x 4 copies)
+    phase_barrier();
+    load_phase_reads(ring + a_lane, ring + kSlotBytes + b_lane, 0);
+    wait_lgkmcnt0();
+    if (group == 1) phase_barrier();  // group 1 runs one phase behind group 0
+
+    uint32_t slot_a = 0;
+    for (uint32_t kt = 0; kt < k_steps; ++kt) {
+      const uint32_t slot_b = slot_a + 1 >= kSlots ? slot_a + 1 - kSlots : slot_a + 1;
+      const uint32_t slot_a1 = slot_a + 2 >= kSlots ? slot_a + 2 - kSlots : slot_a + 2;
+      const uint32_t slot_b1 = slot_a + 3 >= kSlots ? slot_a + 3 - kSlots : slot_a + 3;
+
+      // M0: slice 0 of this k-step.
+      mfma_phase();
+      phase_barrier();
+      // L0: slice 1 of this k-step.  For group 1 this phase ends at global phase 4t+2, the point
+      // by which B(t+1) must have landed everywhere (only the 4 copies of A(t+2) may be in flight).
+      load_phase_reads(ring + slot_a * kSlotBytes + a_lane, ring + slot_b * kSlotBytes + b_lane, 1);
+      wait_lgkmcnt0();
+      if (group == 1) wait_vmcnt<4>();
+      phase_barrier();
+      // M1: slice 1.  For group 0 this phase ends at global phase 4t+2.
+      mfma_phase();
+      if (group == 0) wait_vmcnt<4>();
+      phase_barrier();
+      // L1: slice 0 of the next k-step, and this wave's share of the refill.  Both groups have
+      // finished reading the slots of k-step t by now (group 1 did so in its L0, one phase ago
+      // from group 0's point of view, three phases ago from its own).
+      load_phase_reads(ring + slot_a1 * kSlotBytes + a_lane, ring + slot_b1 * kSlotBytes + b_lane, 0);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) copy_b(rsrc_b, j, slot_a, kt + 2);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) copy_a(rsrc_a, j, slot_b, kt + 3);
+      wait_lgkmcnt0();
+      phase_barrier();
+      slot_a = slot_a1;
+    }
+    if (group == 0) phase_barrier();  // let group 1 finish its last phase; barrier counts now match
+    wait_vmcnt<0>();
+    phase_barrier();
+
+    const int64_t done_m0 = tile_m * kTile, done_n0 = tile_n * kTile;
+    tile += gridDim.x;
+    const bool more = tile < total_tiles;
+    if (more) {
+      tile_coord(tile, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+      rsrc_a = panel_a(tile_m * kTile);
+      rsrc_b = panel_b(tile_n * kTile);
+      open_tile(rsrc_a, rsrc_b);
+    }
+    epilogue(done_m0, done_n0);
+    if (!more) break;
+  }
+}
+
+template <class T, class OutT>
+int launch(const GemmArgs& g, hipStream_t stream) {
+  const int64_t tiles = g.tiles_m * g.tiles_n;
+  const int64_t cus = compute_units();
+  const int64_t blocks = tiles < cus ? tiles : cus;
+  hipLaunchKernelGGL((gemm_tn_tile256_pingpong<T, OutT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, g);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+}  // namespace
+
+int launch_tile256_pingpong(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream) {
+  const bool out_bf16 = out_dtype == 0;
+  switch (in_dtype) {
+    case 0: return out_bf16 ? launch<BF16, BF16>(g, stream) : launch<BF16, F16>(g, stream);
+    case 1: return out_bf16 ? launch<F16, BF16>(g, stream) : launch<F16, F16>(g, stream);
+    case 2: return out_bf16 ? launch<E4M3, BF16>(g, stream) : launch<E4M3, F16>(g, stream);
+  }
+  return -1;
+}
+
+}  // namespace mi355

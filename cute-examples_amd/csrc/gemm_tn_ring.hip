@@ -23,6 +23,14 @@
 // One workgroup barrier per k-step; the loop body is branch-free (loads past the end of K re-read the
 // last k-step into a slot nobody reads).
 //
+// Tiles.  The grid is persistent: one workgroup per CU walks tiles blockIdx.x, +gridDim.x, ...
+// After the last k-step of a tile the workgroup first queues the five opening copies of its next
+// tile and only then converts and stores the finished accumulators, so the store phase of one
+// tile hides the load latency of the next.  Stores: two lanes' 4-element quads are exchanged with
+// v_permlane16_swap / v_permlane32_swap so that every lane writes 8 consecutive outputs (16 B),
+// with the non-temporal hint where a store covers whole 64-byte runs (C is written once and
+// should not evict operand panels from L2).
+//
 // MFMA shape: bf16/fp16 use v_mfma_f32_16x16x32 (8x8 blocks per wave); on random data it sustains
 // a higher clock under the board power limit than 32x32x16.  fp8 uses v_mfma_f32_32x32x64_f8f6f4
 // (4x4 blocks), which keeps the fragment registers within budget.
@@ -30,59 +38,14 @@
 // Counterpart in the reference: the cooperative kernel, kernels/gemm_kernels/sm90a/gemm.cuh:246-418
 // (TMA producer warpgroup, mbarrier full/empty ring of 3 stages, two consumer warpgroups); here
 // every wave is loader and math at once because direct-to-LDS loads need no registers.
-#include "cdna4_primitives.h"
 #include "gemm_launch.h"
+#include "ring_common.h"
 #include "tile_map.h"
 
 namespace mi355 {
 namespace {
 
-constexpr int kTile = 256;
-constexpr int kRowBytes = 128;
-constexpr int kSlotBytes = kTile * kRowBytes;  // 32 KiB: one operand, one k-step
-constexpr int kSlots = 5;
 constexpr int kThreads = 256;
-
-__device__ __forceinline__ uint32_t swizzle(uint32_t row) { return (row >> 1) & 7u; }
-
-#define MI355_FENCE() __builtin_amdgcn_sched_barrier(0)
-#ifndef MI355_DEBUG_MODE
-// Timing experiments only (results are wrong when non-zero):
-//   1 no MFMA, 2 no copies in the main loop, 3 = 2 + no barrier, 4 = 3 + no LDS reads, 5 no LDS reads only
-#define MI355_DEBUG_MODE 0
-#endif
-
-// Per-dtype MFMA geometry.
-//   kBlk      rows (and columns) of one MFMA block
-//   kGroups   lane groups of kBlk lanes; group g feeds k-chunks g*kCpl .. g*kCpl+kCpl-1 of a slice
-//   kCpl      16-byte chunks per lane per MFMA
-template <class T> struct Geo;
-template <> struct Geo<BF16> {
-  static constexpr int kBlk = 16, kGroups = 4, kCpl = 1;
-  typedef i32x4 Frag;
-  typedef f32x4 Acc;
-  static __device__ __forceinline__ Acc mfma(Frag x, Frag y, Acc c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x),
-                                                   __builtin_bit_cast(bf16x8, y), c, 0, 0, 0);
-  }
-};
-template <> struct Geo<F16> {
-  static constexpr int kBlk = 16, kGroups = 4, kCpl = 1;
-  typedef i32x4 Frag;
-  typedef f32x4 Acc;
-  static __device__ __forceinline__ Acc mfma(Frag x, Frag y, Acc c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, x),
-                                                  __builtin_bit_cast(f16x8, y), c, 0, 0, 0);
-  }
-};
-template <> struct Geo<E4M3> {
-  static constexpr int kBlk = 32, kGroups = 2, kCpl = 2;
-  typedef i32x8 Frag;
-  typedef f32x16 Acc;
-  static __device__ __forceinline__ Acc mfma(Frag x, Frag y, Acc c) {
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, c, 0, 0, 0, 0, 0, 0);
-  }
-};
 
 template <class T, class OutT>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) {
@@ -104,19 +67,20 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t wm = wave >> 1, wn = wave & 1u;
 
-  int64_t tile_m, tile_n;
-  tile_coord(blockIdx.x, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-  const int64_t m0 = tile_m * kTile, n0 = tile_n * kTile;
-
   const uint32_t lda_b = (uint32_t)(g.lda * T::kBytes), ldb_b = (uint32_t)(g.ldb * T::kBytes);
   const uint32_t k_bytes = (uint32_t)(g.K * T::kBytes);
-  const int64_t rows_a = g.M - m0 < kTile ? g.M - m0 : kTile;
-  const int64_t rows_b = g.N - n0 < kTile ? g.N - n0 : kTile;
-  const __amdgpu_buffer_rsrc_t rsrc_a = make_raw_buffer(
-      (const uint8_t*)g.A + m0 * (int64_t)lda_b, (uint32_t)((rows_a - 1) * lda_b + k_bytes));
-  const __amdgpu_buffer_rsrc_t rsrc_b = make_raw_buffer(
-      (const uint8_t*)g.B + n0 * (int64_t)ldb_b, (uint32_t)((rows_b - 1) * ldb_b + k_bytes));
   const uint32_t k_steps = __builtin_amdgcn_readfirstlane(k_bytes / kRowBytes);
+  const int64_t total_tiles = g.tiles_m * g.tiles_n;
+
+  // Descriptors of the A and B row panels of a tile; rows past the matrix edge are out of range.
+  auto panel_a = [&](int64_t m0) __attribute__((always_inline)) {
+    const int64_t rows = g.M - m0 < kTile ? g.M - m0 : kTile;
+    return make_raw_buffer((const uint8_t*)g.A + m0 * (int64_t)lda_b, (uint32_t)((rows - 1) * lda_b + k_bytes));
+  };
+  auto panel_b = [&](int64_t n0) __attribute__((always_inline)) {
+    const int64_t rows = g.N - n0 < kTile ? g.N - n0 : kTile;
+    return make_raw_buffer((const uint8_t*)g.B + n0 * (int64_t)ldb_b, (uint32_t)((rows - 1) * ldb_b + k_bytes));
+  };
 
   // Copy geometry: one wave instruction moves 8 rows x 128 B.  Wave w issues copies 8w..8w+7 of
   // an operand (rows 64w .. 64w+63).  Lane l fills LDS chunk l%8 of row l/8 with the global
@@ -139,13 +103,26 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
   // in the vector offset, the only part the hardware range-checks against the descriptor (rows
   // past the edge of the matrix read zeros); the scalar offset carries the k-step and is kept
   // inside the row by re-reading the last k-step for kt past the end (the slot is never used).
-  auto copy_a = [&](int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
+  auto copy_a = [&](__amdgpu_buffer_rsrc_t rsrc, int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
     const uint32_t soff = (kt < k_steps ? kt : k_steps - 1) * kRowBytes;
-    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff_a[j & 1] + j * a_step, rsrc_a, soff);
+    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff_a[j & 1] + j * a_step, rsrc, soff);
   };
-  auto copy_b = [&](int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
+  auto copy_b = [&](__amdgpu_buffer_rsrc_t rsrc, int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
     const uint32_t soff = (kt < k_steps ? kt : k_steps - 1) * kRowBytes;
-    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff_b[j & 1] + j * b_step, rsrc_b, soff);
+    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff_b[j & 1] + j * b_step, rsrc, soff);
+  };
+  // Opening copies of a tile: A0 B0 A1 B1 A2 into slots 0..4.
+  auto open_tile = [&](__amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb) __attribute__((always_inline)) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) copy_a(ra, j, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) copy_b(rb, j, 1, 0);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) copy_a(ra, j, 2, 1);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) copy_b(rb, j, 3, 1);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) copy_a(ra, j, 4, 2);
   };
 
   // Fragment geometry: lane l supplies row l%kBlk of a block; group l/kBlk picks the chunks.
@@ -168,153 +145,173 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
     }
   };
 
-#ifdef MI355_CLOCK_PROBE
-  const uint64_t probe_c0 = __builtin_readcyclecounter(), probe_r0 = __builtin_amdgcn_s_memrealtime();
-  uint64_t probe_r_loop = 0;
-#endif
   Acc acc[kNb][kNb];
-#pragma unroll
-  for (int i = 0; i < kNb; ++i)
-#pragma unroll
-    for (int j = 0; j < kNb; ++j)
-#pragma unroll
-      for (int r = 0; r < kAccLen; ++r) acc[i][j][r] = 0.f;
-
   Frag fa[2][kNb], fb[2][kNb];  // [fragment buffer][block]
 
   // Load number q (0..kReadsPerSlice-1) of a slice: B blocks first (every MFMA row needs them all).
   auto read_q = [&](int buf, int q, const uint8_t* a_rows, const uint8_t* b_rows, int s)
       __attribute__((always_inline)) {
-    if (MI355_DEBUG_MODE >= 4) return;
     if (q < kNb) fb[buf][q] = load_frag(b_rows, q, s);
     else fa[buf][q - kNb] = load_frag(a_rows, q - kNb, s);
   };
   auto mfma_u = [&](int buf, int u) __attribute__((always_inline)) {
     const int i = u / kNb, j = u % kNb;
     // B supplies the MFMA "rows" so each lane ends up with consecutive n of one m.
-#if MI355_DEBUG_MODE == 1
-    acc[i][j][0] += __builtin_bit_cast(float, fb[buf][j][0] ^ fa[buf][i][0]);
-#else
     acc[i][j] = G::mfma(fb[buf][j], fa[buf][i], acc[i][j]);
-#endif
   };
 
-  // Prologue: A0 B0 A1 B1 A2 into slots 0..4.
-#pragma unroll
-  for (int j = 0; j < 8; ++j) copy_a(j, 0, 0);
-#pragma unroll
-  for (int j = 0; j < 8; ++j) copy_b(j, 1, 0);
-#pragma unroll
-  for (int j = 0; j < 8; ++j) copy_a(j, 2, 1);
-#pragma unroll
-  for (int j = 0; j < 8; ++j) copy_b(j, 3, 1);
-#pragma unroll
-  for (int j = 0; j < 8; ++j) copy_a(j, 4, 2);
-  wait_vmcnt<24>();  // A0 and B0 have landed
-  __builtin_amdgcn_s_barrier();
-#pragma unroll
-  for (int q = 0; q < kReadsPerSlice; ++q)
-    read_q(0, q, ring + a_lane, ring + kSlotBytes + b_lane, 0);
-
-#ifdef MI355_CLOCK_PROBE
-  probe_r_loop = __builtin_amdgcn_s_memrealtime();
-#endif
-  uint32_t slot_a = 0;  // slot of A(t); B(t) is in slot_a+1, A(t+1) in slot_a+2, B(t+1) in slot_a+3 (mod 5)
-  for (uint32_t kt = 0; kt < k_steps; ++kt) {
-    const uint32_t slot_b = slot_a + 1 >= kSlots ? slot_a + 1 - kSlots : slot_a + 1;
-    const uint32_t slot_a1 = slot_a + 2 >= kSlots ? slot_a + 2 - kSlots : slot_a + 2;
-    const uint32_t slot_b1 = slot_a + 3 >= kSlots ? slot_a + 3 - kSlots : slot_a + 3;
-    const uint8_t* a_rows = ring + slot_a * kSlotBytes + a_lane;
-    const uint8_t* b_rows = ring + slot_b * kSlotBytes + b_lane;
-    const uint8_t* a1_rows = ring + slot_a1 * kSlotBytes + a_lane;
-    const uint8_t* b1_rows = ring + slot_b1 * kSlotBytes + b_lane;
-
-    // Event schedule of one k-step, in MFMA positions p = slice * kMfmaPerSlice + u:
-    //   reads    one fragment load per MFMA at the start of each slice (for the following slice)
-    //   barrier  in slice 0, a few MFMAs after the last read so its data is back
-    //   copies   one every kCopyEvery MFMAs after the barrier, B(t+2) first.  They must not be
-    //            issued faster than the texture-address unit retires them (one 1 KiB copy takes
-    //            it ~23 cycles and it serves all four waves): a wave whose copy finds the unit's
-    //            queue full stalls at issue and its MFMA stream stops with it.
-    constexpr int kBarrierAt = kReadsPerSlice + kMfmaPerSlice / 8;
-    constexpr int kFirstCopy = kBarrierAt + 1;
-    constexpr int kCopyEvery = (2 * kMfmaPerSlice - kFirstCopy) / 16 > 0 ? (2 * kMfmaPerSlice - kFirstCopy) / 16 : 1;
-    static_assert(kFirstCopy + 15 * kCopyEvery < 2 * kMfmaPerSlice, "copies must fit in the k-step");
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-#pragma unroll
-      for (int u = 0; u < kMfmaPerSlice; ++u) {
-        const int p = s * kMfmaPerSlice + u;
-        if (u < kReadsPerSlice) {
-          if (s == 0) read_q(1, u, a_rows, b_rows, 1);        // slice 1 of this k-step
-          else read_q(0, u, a1_rows, b1_rows, 0);            // slice 0 of the next k-step
-        }
-        if (s == 0 && u == kBarrierAt) {
-          // My reads of this k-step's slots are back; B(t+1) (and A(t+1) before it) have landed;
-          // only the 8 copies of A(t+2) may still be in flight.
-          wait_lgkmcnt0();
-          wait_vmcnt<8>();
-          if (MI355_DEBUG_MODE != 3 && MI355_DEBUG_MODE != 4) __builtin_amdgcn_s_barrier();
-        }
-        if (p >= kFirstCopy && (p - kFirstCopy) % kCopyEvery == 0 && (p - kFirstCopy) / kCopyEvery < 16 &&
-            (MI355_DEBUG_MODE < 2 || MI355_DEBUG_MODE == 5)) {
-          const int c = (p - kFirstCopy) / kCopyEvery;
-          if (c < 8) copy_b(c, slot_a, kt + 2);
-          else copy_a(c - 8, slot_b, kt + 3);
-        }
-        mfma_u(s, u);
-        MI355_FENCE();
-      }
-    }
-    slot_a = slot_a1;
-  }
-  wait_vmcnt<0>();  // drain the unused tail copies before the wave ends
-#ifdef MI355_CLOCK_PROBE
-  const uint64_t probe_c1 = __builtin_readcyclecounter(), probe_r1 = __builtin_amdgcn_s_memrealtime();
-#endif
-
-  // Epilogue.  Accumulator register 4q+e of block (i,j) in lane l is C[m][n] with
+  // Epilogue of the tile at (m0, n0).  Accumulator register 4q+e of block (i,j) in lane l is C[m][n],
   //   m = m0 + wm*128 + i*kBlk + l%kBlk,   n = n0 + wn*128 + j*kBlk + q*4*kGroups + 4*(l/kBlk) + e.
+  // Two quads that sit 4 columns apart in neighbouring lane groups are swapped so that each lane
+  // holds 8 consecutive columns.
   const float scale = g.scale;
   const int64_t ldc = g.ldc;
-  uint16_t* C = (uint16_t*)g.C;
+  uint16_t* const C = (uint16_t*)g.C;
+  auto store8 = [&](int64_t m, int64_t n, u32x2 x, u32x2 y) __attribute__((always_inline)) {
+    if (m >= g.M) return;
+    uint16_t* p = C + m * ldc + n;
+    // Non-temporal stores keep C out of L2 (it is written once and would evict operand panels).
+    // They only pay when a store instruction covers at least 64 contiguous bytes per row, which
+    // the 16-wide blocks do (two blocks side by side) and the 32-wide blocks do not (32 bytes).
+    if constexpr (kBlk == 16) {
+      if (n + 8 <= g.N) __builtin_nontemporal_store((u32x4){x[0], x[1], y[0], y[1]}, (u32x4*)p);
+      else if (n + 4 <= g.N) __builtin_nontemporal_store(x, (u32x2*)p);
+    } else {
+      if (n + 8 <= g.N) *(u32x4*)p = (u32x4){x[0], x[1], y[0], y[1]};
+      else if (n + 4 <= g.N) *(u32x2*)p = x;
+    }
+  };
+  auto pack_quad = [&](const Acc& a, int q) __attribute__((always_inline)) -> u32x2 {
+    return Pack4<OutT>::run(a[4 * q] * scale, a[4 * q + 1] * scale, a[4 * q + 2] * scale, a[4 * q + 3] * scale);
+  };
+  auto epilogue = [&](int64_t m0, int64_t n0) __attribute__((always_inline)) {
 #pragma unroll
-  for (int i = 0; i < kNb; ++i) {
-    const int64_t m = m0 + wm * 128 + i * kBlk + rblk;
-    if (m >= g.M) continue;
+    for (int i = 0; i < kNb; ++i) {
+      const int64_t m = m0 + wm * 128 + i * kBlk + rblk;
+      if constexpr (kBlk == 16) {
+        // lane group g = l/16 holds columns 4g..4g+3 of every 16-wide block.  After swapping the
+        // odd groups of block j with the even groups of block j+1, groups 0,2 hold columns
+        // 0..7 / 8..15 of block j and groups 1,3 the same of block j+1.
 #pragma unroll
-    for (int j = 0; j < kNb; ++j) {
+        for (int j = 0; j < kNb; j += 2) {
+          u32x2 x = pack_quad(acc[i][j], 0), y = pack_quad(acc[i][j + 1], 0);
+          u32x2 lo = __builtin_amdgcn_permlane16_swap(x[0], y[0], false, false);
+          u32x2 hi = __builtin_amdgcn_permlane16_swap(x[1], y[1], false, false);
+          const int64_t n = n0 + wn * 128 + (j + (grp & 1)) * 16 + (grp >> 1) * 8;
+          store8(m, n, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
+        }
+      } else {
+        // lane group g = l/32 holds columns 8q+4g..8q+4g+3 (q = 0..3) of every 32-wide block.
+        // After swapping the upper half of quad q with the lower half of quad q+1, group 0 holds
+        // columns 16(q/2)..+7 and group 1 columns 16(q/2)+8..+15.
 #pragma unroll
-      for (int q = 0; q < kAccLen / 4; ++q) {
-        const int64_t n = n0 + wn * 128 + j * kBlk + q * 4 * G::kGroups + grp * 4;
-        if (n < g.N) {
-          u32x2 v = Pack4<OutT>::run(acc[i][j][4 * q] * scale, acc[i][j][4 * q + 1] * scale,
-                                     acc[i][j][4 * q + 2] * scale, acc[i][j][4 * q + 3] * scale);
-          *(u32x2*)(C + m * ldc + n) = v;
+        for (int j = 0; j < kNb; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; q += 2) {
+            u32x2 x = pack_quad(acc[i][j], q), y = pack_quad(acc[i][j], q + 1);
+            u32x2 lo = __builtin_amdgcn_permlane32_swap(x[0], y[0], false, false);
+            u32x2 hi = __builtin_amdgcn_permlane32_swap(x[1], y[1], false, false);
+            const int64_t n = n0 + wn * 128 + j * 32 + (q >> 1) * 16 + grp * 8;
+            store8(m, n, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
+          }
         }
       }
     }
+  };
+
+  int64_t tile = blockIdx.x;
+  int64_t tile_m, tile_n;
+  tile_coord(tile, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+  __amdgpu_buffer_rsrc_t rsrc_a = panel_a(tile_m * kTile), rsrc_b = panel_b(tile_n * kTile);
+  open_tile(rsrc_a, rsrc_b);
+
+  for (;;) {
+#pragma unroll
+    for (int i = 0; i < kNb; ++i)
+#pragma unroll
+      for (int j = 0; j < kNb; ++j)
+#pragma unroll
+        for (int r = 0; r < kAccLen; ++r) acc[i][j][r] = 0.f;
+
+    wait_vmcnt<24>();  // A0 and B0 have landed
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int q = 0; q < kReadsPerSlice; ++q)
+      read_q(0, q, ring + a_lane, ring + kSlotBytes + b_lane, 0);
+
+    uint32_t slot_a = 0;  // slot of A(t); B(t), A(t+1), B(t+1) follow in slot_a+1..+3 (mod 5)
+    for (uint32_t kt = 0; kt < k_steps; ++kt) {
+      const uint32_t slot_b = slot_a + 1 >= kSlots ? slot_a + 1 - kSlots : slot_a + 1;
+      const uint32_t slot_a1 = slot_a + 2 >= kSlots ? slot_a + 2 - kSlots : slot_a + 2;
+      const uint32_t slot_b1 = slot_a + 3 >= kSlots ? slot_a + 3 - kSlots : slot_a + 3;
+      const uint8_t* a_rows = ring + slot_a * kSlotBytes + a_lane;
+      const uint8_t* b_rows = ring + slot_b * kSlotBytes + b_lane;
+      const uint8_t* a1_rows = ring + slot_a1 * kSlotBytes + a_lane;
+      const uint8_t* b1_rows = ring + slot_b1 * kSlotBytes + b_lane;
+
+      // Event schedule of one k-step, in MFMA positions p = slice * kMfmaPerSlice + u:
+      //   reads    one fragment load per MFMA at the start of each slice (for the following slice)
+      //   barrier  in slice 0, a few MFMAs after the last read so its data is back
+      //   copies   one every kCopyEvery MFMAs after the barrier, B(t+2) first.  They must not be
+      //            issued faster than the texture-address unit retires them (one 1 KiB copy takes
+      //            it ~23 cycles and it serves all four waves): a wave whose copy finds the unit's
+      //            queue full stalls at issue and its MFMA stream stops with it.
+      constexpr int kBarrierAt = kReadsPerSlice + kMfmaPerSlice / 8;
+      constexpr int kFirstCopy = kBarrierAt + 1;
+      constexpr int kCopyEvery = (2 * kMfmaPerSlice - kFirstCopy) / 16 > 0 ? (2 * kMfmaPerSlice - kFirstCopy) / 16 : 1;
+      static_assert(kFirstCopy + 15 * kCopyEvery < 2 * kMfmaPerSlice, "copies must fit in the k-step");
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+#pragma unroll
+        for (int u = 0; u < kMfmaPerSlice; ++u) {
+          const int p = s * kMfmaPerSlice + u;
+          if (u < kReadsPerSlice) {
+            if (s == 0) read_q(1, u, a_rows, b_rows, 1);       // slice 1 of this k-step
+            else read_q(0, u, a1_rows, b1_rows, 0);           // slice 0 of the next k-step
+          }
+          if (s == 0 && u == kBarrierAt) {
+            // My reads of this k-step's slots are back; B(t+1) (and A(t+1) before it) have
+            // landed; only the 8 copies of A(t+2) may still be in flight.
+            wait_lgkmcnt0();
+            wait_vmcnt<8>();
+            __builtin_amdgcn_s_barrier();
+          }
+          if (p >= kFirstCopy && (p - kFirstCopy) % kCopyEvery == 0 && (p - kFirstCopy) / kCopyEvery < 16) {
+            const int c = (p - kFirstCopy) / kCopyEvery;
+            if (c < 8) copy_b(rsrc_b, c, slot_a, kt + 2);
+            else copy_a(rsrc_a, c - 8, slot_b, kt + 3);
+          }
+          mfma_u(s, u);
+          MI355_FENCE();
+        }
+      }
+      slot_a = slot_a1;
+    }
+    // The tail copies (past the end of K) must have landed, and every wave must be past its last
+    // LDS read, before the ring is refilled for the next tile.
+    wait_vmcnt<0>();
+    wait_lgkmcnt0();
+    __builtin_amdgcn_s_barrier();
+
+    const int64_t done_m0 = tile_m * kTile, done_n0 = tile_n * kTile;
+    tile += gridDim.x;
+    const bool more = tile < total_tiles;
+    if (more) {
+      tile_coord(tile, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+      rsrc_a = panel_a(tile_m * kTile);
+      rsrc_b = panel_b(tile_n * kTile);
+      open_tile(rsrc_a, rsrc_b);  // in flight while the finished tile is stored
+    }
+    epilogue(done_m0, done_n0);
+    if (!more) break;
   }
-#ifdef MI355_CLOCK_PROBE
-  // Timing experiments only: every block overwrites 64 bytes of C with time stamps.
-  __builtin_amdgcn_s_barrier();
-  if (tid == 0) {
-    uint64_t* rec = (uint64_t*)g.C + 8 * (uint64_t)blockIdx.x;
-    rec[0] = probe_c1 - probe_c0;
-    rec[1] = probe_r1 - probe_r0;
-    rec[2] = probe_r0;
-    rec[3] = probe_r_loop;
-    rec[4] = probe_r1;
-    rec[5] = __builtin_amdgcn_s_memrealtime();
-    rec[6] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
-    rec[7] = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11));  // XCC_ID
-  }
-#endif
 }
 
 template <class T, class OutT>
 int launch(const GemmArgs& g, hipStream_t stream) {
-  const int64_t blocks = g.tiles_m * g.tiles_n;
+  const int64_t tiles = g.tiles_m * g.tiles_n;
+  const int64_t cus = compute_units();
+  const int64_t blocks = tiles < cus ? tiles : cus;  // one resident workgroup per CU (LDS-bound)
   hipLaunchKernelGGL((gemm_tn_tile256_ring<T, OutT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, g);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }

@@ -1,0 +1,65 @@
+// Pieces shared by the ring-buffered 256x256-tile kernels (single wave group and ping-pong):
+// LDS ring geometry, the bank-conflict-free chunk swizzle, and the per-dtype MFMA geometry.
+#pragma once
+#include "cdna4_primitives.h"
+
+#include <atomic>
+
+namespace mi355 {
+
+constexpr int kTile = 256;
+constexpr int kRowBytes = 128;
+constexpr int kSlotBytes = kTile * kRowBytes;  // 32 KiB: one operand, one k-step
+constexpr int kSlots = 5;
+
+__device__ __forceinline__ uint32_t swizzle(uint32_t row) { return (row >> 1) & 7u; }
+
+#define MI355_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// Per-dtype MFMA geometry.
+//   kBlk      rows (and columns) of one MFMA block
+//   kGroups   lane groups of kBlk lanes; group g feeds k-chunks g*kCpl .. g*kCpl+kCpl-1 of a slice
+//   kCpl      16-byte chunks per lane per MFMA
+template <class T> struct Geo;
+template <> struct Geo<BF16> {
+  static constexpr int kBlk = 16, kGroups = 4, kCpl = 1;
+  typedef i32x4 Frag;
+  typedef f32x4 Acc;
+  static __device__ __forceinline__ Acc mfma(Frag x, Frag y, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x),
+                                                   __builtin_bit_cast(bf16x8, y), c, 0, 0, 0);
+  }
+};
+template <> struct Geo<F16> {
+  static constexpr int kBlk = 16, kGroups = 4, kCpl = 1;
+  typedef i32x4 Frag;
+  typedef f32x4 Acc;
+  static __device__ __forceinline__ Acc mfma(Frag x, Frag y, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, x),
+                                                  __builtin_bit_cast(f16x8, y), c, 0, 0, 0);
+  }
+};
+template <> struct Geo<E4M3> {
+  static constexpr int kBlk = 32, kGroups = 2, kCpl = 2;
+  typedef i32x8 Frag;
+  typedef f32x16 Acc;
+  static __device__ __forceinline__ Acc mfma(Frag x, Frag y, Acc c) {
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, c, 0, 0, 0, 0, 0, 0);
+  }
+};
+
+
+// Compute units of the current device (256 on MI355X); queried once per device.
+inline int compute_units() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
+}  // namespace mi355
