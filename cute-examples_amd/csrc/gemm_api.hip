@@ -25,6 +25,13 @@ bool tile256_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64
   return true;
 }
 
+// Constraints of the small-M streaming kernel.
+bool skinny_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int in_dtype) {
+  if (in_dtype == MI355_E4M3) return false;
+  if (M > 256) return false;
+  return tile256_ok(M, N, K, lda, ldb, ldc, in_dtype);
+}
+
 int check_common(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                  int in_dtype, int out_dtype, int variant) {
   if (!valid_in(in_dtype) || !valid_out(out_dtype)) return MI355_ERR_DTYPE;
@@ -36,11 +43,16 @@ int check_common(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int6
 
 int resolve(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int in_dtype,
             int variant) {
-  if (variant == MI355_VARIANT_AUTO)
-    return tile256_ok(M, N, K, lda, ldb, ldc, in_dtype) ? MI355_VARIANT_BASIC : MI355_VARIANT_SIMPLE;
+  if (variant == MI355_VARIANT_AUTO) {
+    if (!tile256_ok(M, N, K, lda, ldb, ldc, in_dtype)) return MI355_VARIANT_SIMPLE;
+    // One row of 256x256 tiles cannot fill the machine; stream the weights instead.
+    if (skinny_ok(M, N, K, lda, ldb, ldc, in_dtype)) return MI355_VARIANT_SKINNY;
+    return MI355_VARIANT_BASIC;
+  }
   if (variant == MI355_VARIANT_BASIC || variant == MI355_VARIANT_PINGPONG)
     return tile256_ok(M, N, K, lda, ldb, ldc, in_dtype) ? variant : MI355_ERR_SHAPE;
-  if (variant == MI355_VARIANT_SKINNY) return MI355_ERR_VARIANT;
+  if (variant == MI355_VARIANT_SKINNY)
+    return skinny_ok(M, N, K, lda, ldb, ldc, in_dtype) ? variant : MI355_ERR_SHAPE;
   return variant;
 }
 
@@ -90,14 +102,16 @@ int mi355_gemm_select_variant(int64_t M, int64_t N, int64_t K, int in_dtype) {
 }
 
 size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int in_dtype, int variant) {
-  (void)M; (void)N; (void)K; (void)in_dtype; (void)variant;
-  return 0;
+  if (!valid_in(in_dtype) || M <= 0 || N <= 0 || K <= 0) return 0;
+  if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_SIMPLE) return 0;
+  if (resolve(M, N, K, K, K, N, in_dtype, variant) != MI355_VARIANT_SKINNY) return 0;
+  const int splits = mi355::stream_splits(M, N, K, elem_bytes(in_dtype));
+  return splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 
 int mi355_gemm_tn(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                   int64_t lda, int64_t ldb, int64_t ldc, int in_dtype, int out_dtype, float scale,
                   int variant, void* workspace, size_t workspace_bytes, void* stream) {
-  (void)workspace; (void)workspace_bytes;
   int st = check_common(M, N, K, lda, ldb, ldc, in_dtype, out_dtype, variant);
   if (st != MI355_OK) return st;
   if (M == 0 || N == 0) return MI355_OK;  // nothing to write
@@ -112,7 +126,7 @@ int mi355_gemm_tn(const void* A, const void* B, void* C, int64_t M, int64_t N, i
   g.scale = scale;
   hipStream_t s = (hipStream_t)stream;
 
-  if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG) {
+  if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG || v == MI355_VARIANT_SKINNY) {
     const bool aligned = ((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) && ((uintptr_t)C % 8 == 0);
     if (!aligned) {
       if (variant != MI355_VARIANT_AUTO) return MI355_ERR_ALIGN;
@@ -120,7 +134,15 @@ int mi355_gemm_tn(const void* A, const void* B, void* C, int64_t M, int64_t N, i
     }
   }
   int rc;
-  if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG) {
+  if (v == MI355_VARIANT_SKINNY) {
+    // The split count depends on the shape only, never on the leading dimensions, so it matches
+    // what mi355_gemm_workspace_bytes reported.
+    const int splits = mi355::stream_splits(M, N, K, elem_bytes(in_dtype));
+    const size_t need = splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0;
+    if (need && (!workspace || workspace_bytes < need || (uintptr_t)workspace % 16 != 0)) return MI355_ERR_WORKSPACE;
+    g.tiles_m = g.tiles_n = 0;
+    rc = mi355::launch_stream(g, in_dtype, out_dtype, splits, workspace, s);
+  } else if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG) {
     g.tiles_m = (M + 255) / 256;
     g.tiles_n = (N + 255) / 256;
     rc = v == MI355_VARIANT_PINGPONG ? mi355::launch_tile256_pingpong(g, in_dtype, out_dtype, s)

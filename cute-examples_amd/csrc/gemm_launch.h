@@ -20,6 +20,9 @@ struct GemmArgs {
 // in_dtype / out_dtype use the numbering of enum mi355_dtype.
 int launch_tile256_pingpong(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
 int launch_tile256_ring(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
+// Skinny (small-M) weight-streaming kernel.  stream_splits is a pure host function.
+int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes);
+int launch_stream(const GemmArgs& g, int in_dtype, int out_dtype, int splits, void* workspace, hipStream_t stream);
 int launch_simple(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
 
 }  // namespace mi355

@@ -1,0 +1,214 @@
+// "skinny" variant: weight-streaming GEMM for small M (LLM projections with a few tokens).
+//
+// C[M,N] = scale * X[M,K] · W[N,K]^T with M <= 256 is bound by reading W once from HBM, so the
+// kernel is built around keeping many bytes of W in flight per CU rather than around MFMA issue:
+//
+//   * output tile TM x 64 with TM = 16/32/64/128/256 >= M; the grid is (N/64 tiles) x (K splits),
+//     several workgroups resident per CU (the LDS ring of one workgroup is 30-120 KiB);
+//   * per k-step (128 B of K per row) the TM rows of X and 64 rows of W go global -> LDS with
+//     full-cache-line direct-to-LDS loads into a ring of kDepth stages, kDepth-1 k-steps ahead;
+//   * the four waves read MFMA fragments from LDS (same 16-byte-chunk swizzle as the big-tile
+//     kernels) and run v_mfma_f32_16x16x32; W blocks are the MFMA rows, so every lane ends up
+//     with four consecutive n of one m;
+//   * with K split S ways the partial tiles go to an fp32 workspace [S][M][N] and a second kernel
+//     adds them in a fixed order (deterministic), scales and rounds; with S = 1 the tile is
+//     rounded and stored directly.
+//
+// Counterpart in the reference: none — its launcher rejects M not divisible by 256
+// (kernels/gemm_kernels/sm90a/gemm_test.cu:33-35); the arithmetic contract is the same one
+// (gemm.cuh:352-377: fp32 accumulation of exact products, round-to-nearest-even output).
+#include "gemm_launch.h"
+#include "ring_common.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kTileN = 64;
+
+// kMB x kNB 16x16 blocks per wave, kWM x kWN waves (kWM * kWN == 4).
+template <class T, class OutT, int kMB, int kNB, int kWM, int kWN, int kDepth>
+__global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* partial, int splits) {
+  typedef Geo<T> G;
+  static_assert(G::kBlk == 16 && kWM * kWN == 4, "16x16x32 MFMA, four waves");
+  constexpr int kTm = 16 * kMB * kWM, kTn = 16 * kNB * kWN;
+  static_assert(kTn == kTileN, "grid assumes 64-row W tiles");
+  constexpr int kStageBytes = (kTm + kTn) * kRowBytes;
+  constexpr int kCopies = (kTm + kTn) / 8;          // 8-row copies per k-step
+  constexpr int kCpw = (kCopies + 3) / 4;           // per wave (padded with repeats)
+  constexpr int kXCopies = kTm / 8;
+  static_assert(kCpw * (kDepth - 1) < 64, "vmcnt is a 6-bit counter");
+  __shared__ __attribute__((aligned(1024))) uint8_t ring[kDepth * kStageBytes];
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t lane = tid & 63u;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t wm = wave / kWN, wn = wave % kWN;
+
+  const int64_t tiles_m = (g.M + kTm - 1) / kTm;
+  const int64_t tile_m = blockIdx.x % tiles_m, tile_n = blockIdx.x / tiles_m;
+  const int64_t m0 = tile_m * kTm, n0 = tile_n * kTn;
+  const uint32_t split = blockIdx.y;
+
+  const uint32_t ldx_b = (uint32_t)(g.lda * T::kBytes), ldw_b = (uint32_t)(g.ldb * T::kBytes);
+  const uint32_t k_bytes = (uint32_t)(g.K * T::kBytes);
+  const uint32_t steps_total = k_bytes / kRowBytes;
+  const uint32_t steps = __builtin_amdgcn_readfirstlane(steps_total / (uint32_t)splits);
+  const uint32_t step0 = __builtin_amdgcn_readfirstlane(split * steps);
+  const int64_t rows_x = g.M - m0 < kTm ? g.M - m0 : kTm;
+  const int64_t rows_w = g.N - n0 < kTn ? g.N - n0 : kTn;
+  const __amdgpu_buffer_rsrc_t rsrc_x = make_raw_buffer(
+      (const uint8_t*)g.A + m0 * (int64_t)ldx_b, (uint32_t)((rows_x - 1) * ldx_b + k_bytes));
+  const __amdgpu_buffer_rsrc_t rsrc_w = make_raw_buffer(
+      (const uint8_t*)g.B + n0 * (int64_t)ldw_b, (uint32_t)((rows_w - 1) * ldw_b + k_bytes));
+
+  // Copy c (0..kCopies-1) of a k-step moves 8 rows x 128 B: X rows first, then W rows; wave w
+  // issues copies w, w+4, ...  (indices past the end repeat earlier copies so that every wave
+  // issues the same number and one vmcnt value fits all).  Rows past the matrix edge are out of
+  // the descriptor's range and read as zeros.
+  const uint32_t r8 = lane >> 3, c8 = lane & 7u;
+  const uint32_t ring0 = __builtin_amdgcn_readfirstlane(lds_address(ring));
+  auto issue_step = [&](uint32_t stage, uint32_t kt) __attribute__((always_inline)) {
+    const uint32_t soff = (kt < steps ? step0 + kt : step0 + steps - 1) * kRowBytes;
+#pragma unroll
+    for (int i = 0; i < kCpw; ++i) {
+      const uint32_t c = (wave + 4 * i) % kCopies;
+      const uint32_t row = c * 8 + r8;                   // row inside the stage: X rows, then W rows
+      const uint32_t chunk = c8 ^ swizzle(row);
+      const uint32_t dst = ring0 + stage * kStageBytes + c * 1024;
+      if (c < kXCopies) dma_16B_to_lds(dst, row * ldx_b + chunk * 16, rsrc_x, soff);   // c is wave-uniform
+      else dma_16B_to_lds(dst, (row - kTm) * ldw_b + chunk * 16, rsrc_w, soff);
+    }
+  };
+
+  // Fragment geometry: lane l supplies row l%16 of a block, lane group l/16 picks the chunk.
+  const uint32_t rblk = lane & 15u, grp = lane >> 4;
+  const uint32_t swz = swizzle(rblk);
+  const uint32_t x_lane = (wm * kMB * 16 + rblk) * kRowBytes;
+  const uint32_t w_lane = (kTm + wn * kNB * 16 + rblk) * kRowBytes;
+  auto frag = [&](const uint8_t* rows, int blk, int s) __attribute__((always_inline)) -> i32x4 {
+    return *(const i32x4*)(rows + blk * 16 * kRowBytes + (((uint32_t)(s * 4) + grp) ^ swz) * 16);
+  };
+
+  f32x4 acc[kMB][kNB];
+#pragma unroll
+  for (int i = 0; i < kMB; ++i)
+#pragma unroll
+    for (int j = 0; j < kNB; ++j) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int st = 0; st < kDepth - 1; ++st) issue_step(st, st);
+
+  uint32_t stage = 0;
+  for (uint32_t kt = 0; kt < steps; ++kt) {
+    wait_vmcnt<kCpw * (kDepth - 2)>();  // my copies of k-step kt have landed
+    wait_lgkmcnt0();                    // my LDS reads of k-step kt-1 are back
+    __builtin_amdgcn_s_barrier();       // everybody's are: stage of kt is full, stage of kt-1 is free
+    const uint32_t refill = stage == 0 ? kDepth - 1 : stage - 1;
+    issue_step(refill, kt + kDepth - 1);
+    const uint8_t* st_base = ring + stage * kStageBytes;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      i32x4 fx[kMB], fw[kNB];
+#pragma unroll
+      for (int j = 0; j < kNB; ++j) fw[j] = frag(st_base + w_lane, j, s);
+#pragma unroll
+      for (int i = 0; i < kMB; ++i) fx[i] = frag(st_base + x_lane, i, s);
+#pragma unroll
+      for (int i = 0; i < kMB; ++i)
+#pragma unroll
+        for (int j = 0; j < kNB; ++j) acc[i][j] = G::mfma(fw[j], fx[i], acc[i][j]);
+    }
+    stage = stage + 1 == kDepth ? 0 : stage + 1;
+  }
+  wait_vmcnt<0>();
+
+  // acc[i][j][r] of lane l is the (partial) sum for
+  //   m = m0 + (wm*kMB + i)*16 + l%16,   n = n0 + (wn*kNB + j)*16 + 4*(l/16) + r.
+#pragma unroll
+  for (int i = 0; i < kMB; ++i) {
+    const int64_t m = m0 + (wm * kMB + i) * 16 + rblk;
+    if (m >= g.M) continue;
+#pragma unroll
+    for (int j = 0; j < kNB; ++j) {
+      const int64_t n = n0 + (wn * kNB + j) * 16 + grp * 4;
+      if (n + 4 > g.N) continue;
+      if (partial) {
+        *(f32x4*)(partial + ((int64_t)split * g.M + m) * g.N + n) = acc[i][j];
+      } else {
+        const float sc = g.scale;
+        *(u32x2*)((uint16_t*)g.C + m * g.ldc + n) =
+            Pack4<OutT>::run(acc[i][j][0] * sc, acc[i][j][1] * sc, acc[i][j][2] * sc, acc[i][j][3] * sc);
+      }
+    }
+  }
+}
+
+// C[m][n..n+3] = rne(scale * (partial[0] + partial[1] + ... + partial[S-1])), summed in that order.
+template <class OutT>
+__global__ __launch_bounds__(256) void splitk_reduce(const float* partial, uint16_t* C, int64_t M, int64_t N,
+                                                     int64_t ldc, int splits, float scale) {
+  const int64_t quads_per_row = N / 4;
+  const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (q >= M * quads_per_row) return;
+  const int64_t m = q / quads_per_row, n = (q % quads_per_row) * 4;
+  f32x4 sum = *(const f32x4*)(partial + m * N + n);
+  for (int s = 1; s < splits; ++s) sum += *(const f32x4*)(partial + ((int64_t)s * M + m) * N + n);
+  *(u32x2*)(C + m * ldc + n) = Pack4<OutT>::run(sum[0] * scale, sum[1] * scale, sum[2] * scale, sum[3] * scale);
+}
+
+template <class T, class OutT, int kMB, int kNB, int kWM, int kWN, int kDepth>
+int launch_cfg(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
+  constexpr int kTm = 16 * kMB * kWM;
+  const int64_t tiles = ((g.M + kTm - 1) / kTm) * ((g.N + kTileN - 1) / kTileN);
+  float* partial = splits > 1 ? ws : nullptr;
+  hipLaunchKernelGGL((gemm_tn_stream<T, OutT, kMB, kNB, kWM, kWN, kDepth>), dim3((unsigned)tiles, (unsigned)splits),
+                     dim3(kThreads), 0, stream, g, partial, splits);
+  if (hipGetLastError() != hipSuccess) return -1;
+  if (splits > 1) {
+    const int64_t quads = g.M * (g.N / 4);
+    hipLaunchKernelGGL((splitk_reduce<OutT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, ws,
+                       (uint16_t*)g.C, g.M, g.N, g.ldc, splits, g.scale);
+    if (hipGetLastError() != hipSuccess) return -1;
+  }
+  return 0;
+}
+
+template <class T, class OutT>
+int launch_m(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
+  if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, 6>(g, splits, ws, stream);   //  16x64, 10 KiB/step
+  if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, 5>(g, splits, ws, stream);   //  32x64, 12 KiB/step
+  if (g.M <= 64) return launch_cfg<T, OutT, 4, 1, 1, 4, 4>(g, splits, ws, stream);   //  64x64, 16 KiB/step
+  if (g.M <= 128) return launch_cfg<T, OutT, 4, 2, 2, 2, 4>(g, splits, ws, stream);  // 128x64, 24 KiB/step
+  return launch_cfg<T, OutT, 4, 4, 4, 1, 3>(g, splits, ws, stream);                  // 256x64, 40 KiB/step
+}
+
+}  // namespace
+
+// K splits for a skinny problem: enough workgroups to put about two on every CU, each with at
+// least 8 k-steps, and the k-steps must divide evenly.
+int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
+  const int64_t tm = M <= 16 ? 16 : M <= 32 ? 32 : M <= 64 ? 64 : M <= 128 ? 128 : 256;
+  const int64_t tiles = ((M + tm - 1) / tm) * ((N + kTileN - 1) / kTileN);
+  const int64_t steps = K * elem_bytes / kRowBytes;
+  const int64_t want = 2 * 256;  // MI355X has 256 CUs; a heuristic only, so no device query here
+  int best = 1;
+  for (int s = 1; s <= 16; ++s) {
+    if (steps % s != 0 || steps / s < 8) continue;
+    best = s;
+    if (tiles * s >= want) break;
+  }
+  return best;
+}
+
+int launch_stream(const GemmArgs& g, int in_dtype, int out_dtype, int splits, void* workspace, hipStream_t stream) {
+  float* ws = (float*)workspace;
+  const bool out_bf16 = out_dtype == 0;
+  switch (in_dtype) {
+    case 0: return out_bf16 ? launch_m<BF16, BF16>(g, splits, ws, stream) : launch_m<BF16, F16>(g, splits, ws, stream);
+    case 1: return out_bf16 ? launch_m<F16, BF16>(g, splits, ws, stream) : launch_m<F16, F16>(g, splits, ws, stream);
+  }
+  return -1;
+}
+
+}  // namespace mi355

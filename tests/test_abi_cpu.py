@@ -40,6 +40,9 @@ def test_version_and_strerror(abi):
     ((16, 30, 7, 7, 7, 30, ac.F16, ac.F16, ac.SIMPLE), ac.OK),
     ((256, 256, 128, 128, 128, 256, ac.E4M3, ac.BF16, ac.BASIC), ac.OK),
     ((256, 256, 64, 64, 64, 256, ac.E4M3, ac.BF16, ac.BASIC), ac.ERR_SHAPE),  # 64 fp8 bytes < k-step
+    ((64, 256, 128, 128, 128, 256, ac.BF16, ac.BF16, ac.SKINNY), ac.OK),
+    ((257, 256, 128, 128, 128, 256, ac.BF16, ac.BF16, ac.SKINNY), ac.ERR_SHAPE),     # M > 256
+    ((64, 256, 128, 128, 128, 256, ac.E4M3, ac.BF16, ac.SKINNY), ac.ERR_SHAPE),      # fp8
     ((0, 0, 0, 0, 0, 0, ac.BF16, ac.BF16, ac.AUTO), ac.OK),
 ])
 def test_check(abi, args, want):
@@ -55,8 +58,23 @@ def test_gemm_tn_rejects_before_any_device_access(abi):
     assert f(None, None, None, 0, 256, 64, 64, 64, 256, 0, 0, 1.0, 0, None, 0, None) == ac.OK  # empty
 
 
+def test_workspace_bytes(abi):
+    f = abi.mi355_gemm_workspace_bytes
+    assert f(8192, 8192, 8192, ac.BF16, ac.AUTO) == 0
+    assert f(8192, 8192, 8192, ac.BF16, ac.BASIC) == 0
+    assert f(16, 512, 128, ac.BF16, ac.SKINNY) == 0              # too few k-steps to split
+    need = f(16, 4096, 14336, ac.BF16, ac.AUTO)
+    assert need > 0 and need % (16 * 4096 * 4) == 0 and need // (16 * 4096 * 4) <= 16
+    assert f(16, 4096, 14336, ac.BF16, ac.BASIC) == 0
+    assert f(16, 4096, 14336, ac.E4M3, ac.AUTO) == 0             # fp8 has no streaming kernel
+    assert f(-1, 4096, 14336, ac.BF16, ac.AUTO) == 0 and f(16, 4096, 14336, 9, ac.AUTO) == 0
+
+
 def test_select_variant(abi):
     assert abi.mi355_gemm_select_variant(8192, 8192, 8192, ac.BF16) in (ac.BASIC, ac.PINGPONG)
+    assert abi.mi355_gemm_select_variant(16, 14336, 4096, ac.BF16) == ac.SKINNY
+    assert abi.mi355_gemm_select_variant(256, 4096, 14336, ac.F16) == ac.SKINNY
+    assert abi.mi355_gemm_select_variant(16, 14336, 4096, ac.E4M3) == ac.BASIC
     assert abi.mi355_gemm_select_variant(100, 30, 77, ac.BF16) == ac.SIMPLE
     assert abi.mi355_gemm_select_variant(8192, 8192, 8192, 9) == ac.ERR_DTYPE
 

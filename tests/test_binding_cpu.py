@@ -51,6 +51,9 @@ def test_variant_argument():
         gemm_kernels.gemm_tn(A, B, C, variant="basic")
     with pytest.raises(RuntimeError, match="HIP device"):  # auto falls back to the simple kernel
         gemm_kernels.gemm_tn(A, B, C)
+    A, B, C = _abc(M=512)
+    with pytest.raises(RuntimeError, match="constraint"):
+        gemm_kernels.gemm_tn(A, B, C, variant="skinny")
 
 
 def test_fp8_contract():
@@ -69,6 +72,7 @@ def test_fp8_contract():
 def test_select_variant():
     assert gemm_kernels.select_variant(8192, 8192, 8192, torch.bfloat16) in ("basic", "pingpong")
     assert gemm_kernels.select_variant(100, 30, 77, torch.float16) == "simple"
+    assert gemm_kernels.select_variant(64, 14336, 4096, torch.bfloat16) == "skinny"
     with pytest.raises(RuntimeError):
         gemm_kernels.select_variant(1, 1, 1, torch.float32)
 

@@ -134,7 +134,7 @@ def test_fp8_per_tensor_scaled(abi, size, variant):
 
 
 @pytest.mark.parametrize("variant", [ac.AUTO] + TILED + [ac.SIMPLE])
-@pytest.mark.parametrize("M,N,K", [(300, 260, 256), (16, 512, 128), (1, 4, 64), (257, 1028, 192),
+@pytest.mark.parametrize("M,N,K", [(300, 260, 256), (16, 512, 128), (1, 4, 64), (257, 1028, 192), (5000, 4100, 512),
                                    (256, 256, 64), (511, 252, 640)])
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
 def test_ragged_shapes(abi, dt, M, N, K, variant):
@@ -224,8 +224,47 @@ def test_config5_fp8_8192_full_size(abi, variant):
 def test_config4_skinny_projections(abi, M, N, K):
     from gemm_kernels import workloads
     X, W = workloads.skinny(M, N, K, seed=60)
+    assert abi.mi355_gemm_select_variant(M, N, K, ac.BF16) == ac.SKINNY
     C = run_abi(abi, X, W, ac.AUTO)
-    check(C, X, W)
+    err, ref = check(C, X, W)
+    assert err < 4e-3
+    # the big-tile kernel must agree on the same inputs
+    assert oracle.rel_frobenius(run_abi(abi, X, W, ac.BASIC), ref) < 4e-3
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 512, 128), (10, 260, 256), (17, 64, 1024), (33, 512, 4096),
+                                   (64, 1024, 2048), (100, 640, 1024), (129, 72, 512), (256, 768, 2048)])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_skinny_kernel_every_tile_height_and_split(abi, dt, M, N, K):
+    """Each TM configuration (16/32/64/128/256), with and without K splits, ragged M and N."""
+    A, B = rand((M, K), M + 1, dt), rand((N, K), N + 2, dt)
+    C = run_abi(abi, A, B, ac.SKINNY)
+    check(C, A, B)
+    assert oracle.rel_frobenius(C, oracle.c_gemm_tn_f32(A, B)) <= TOL[dt]
+
+
+def test_skinny_split_k_is_deterministic_and_needs_its_workspace(abi):
+    M, N, K = 16, 256, 4096
+    A, B = rand((M, K), 1, torch.bfloat16).cuda(), rand((N, K), 2, torch.bfloat16).cuda()
+    need = abi.mi355_gemm_workspace_bytes(M, N, K, ac.BF16, ac.SKINNY)
+    assert need > 0 and need % (M * N * 4) == 0
+    C1 = torch.empty(M, N, dtype=torch.bfloat16, device="cuda")
+    C2 = torch.empty_like(C1)
+    assert ac.gemm_tn(abi, A, B, C1, 1.0, ac.SKINNY) == 0
+    assert ac.gemm_tn(abi, A, B, C2, 1.0, ac.SKINNY) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(C1, C2)
+    s = torch.cuda.current_stream().cuda_stream
+    rc = abi.mi355_gemm_tn(A.data_ptr(), B.data_ptr(), C1.data_ptr(), M, N, K, K, K, N, ac.BF16, ac.BF16, 1.0,
+                           ac.SKINNY, None, 0, s)
+    assert rc == ac.ERR_WORKSPACE
+    small = torch.empty(need - 16, dtype=torch.uint8, device="cuda")
+    rc = abi.mi355_gemm_tn(A.data_ptr(), B.data_ptr(), C1.data_ptr(), M, N, K, K, K, N, ac.BF16, ac.BF16, 1.0,
+                           ac.SKINNY, small.data_ptr(), need - 16, s)
+    assert rc == ac.ERR_WORKSPACE
+    big = torch.empty(300, 64, dtype=torch.bfloat16, device="cuda")
+    assert ac.gemm_tn(abi, big, torch.empty(64, 64, dtype=torch.bfloat16, device="cuda"),
+                      torch.empty(300, 64, dtype=torch.bfloat16, device="cuda"), 1.0, ac.SKINNY) == ac.ERR_SHAPE
 
 
 # ---------------------------------------------------------------- Python module
@@ -246,11 +285,11 @@ def test_python_module_is_the_reference_call(abi):
 def test_python_module_variants_streams_and_fp8():
     import gemm_kernels
     from gemm_kernels.quant import quantize_e4m3
-    A, B = rand((512, 256), 70, torch.bfloat16).cuda(), rand((768, 256), 71, torch.bfloat16).cuda()
+    A, B = rand((192, 1024), 70, torch.bfloat16).cuda(), rand((768, 1024), 71, torch.bfloat16).cuda()
     want = oracle.gemm_tn_fp32(A, B)
     side = torch.cuda.Stream()
-    for v in ["auto", "basic", "pingpong", "simple"]:
-        C = torch.full((512, 768), float("nan"), dtype=torch.bfloat16, device="cuda")
+    for v in ["auto", "basic", "pingpong", "skinny", "simple"]:
+        C = torch.full((192, 768), float("nan"), dtype=torch.bfloat16, device="cuda")
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             gemm_kernels.gemm_tn(A, B, C, variant=v)
