@@ -36,6 +36,10 @@ def parse():
     p.add_argument("--variant", default="auto")
     p.add_argument("--no-extras", action="store_true")
     p.add_argument("--no-cpu", action="store_true")
+    p.add_argument("--copy-calibration", action="store_true",
+                   help="also run three 1 GiB device-to-device copies (known traffic: 1 GiB read + 1 GiB "
+                        "written each) so that a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this "
+                        "command can be scaled by what the same counter reads for a plain copy")
     return p.parse_args()
 
 
@@ -145,6 +149,15 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU")
     import gemm_kernels
+
+    if a.copy_calibration:
+        src = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+        torch.cuda.empty_cache()
 
     head, keep = measure(a.workload, a.variant, a.steps, a.warmup)
     sets, C, fp8, flops, nbytes = keep
