@@ -25,6 +25,10 @@ sys.path.insert(0, os.path.join(ROOT, "cute-examples_amd"))
 METRIC = "GEMM TFLOP/s and % of MI355X dense MFMA peak, bf16 8192^3 and fp8 8192^3"
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "e4m3": 5000.0}   # dense MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
+# HBM-side bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs of this script
+# (FETCH_SIZE, then WRITE_SIZE, each with --copy-calibration and scaled by what the same counter
+# reads for the 1 GiB copy: x2.000 and x1.000).  Workloads without a counter run report null.
+MEASURED_TRAFFIC_BYTES = {"bf16_8192": 1.895e9, "fp8_8192": 1.63e9, "skinny_16_14336_4096": 1.266e8}
 
 
 def parse():
@@ -165,10 +169,10 @@ def main():
     if mfma_bound:
         roof = {"bound": "mfma", "achieved": head["tflops"], "peak": PEAK_TFLOPS[head["dtype"]],
                 "unit": "TFLOP/s", "frac": round(head["tflops"] / PEAK_TFLOPS[head["dtype"]], 4),
-                "traffic": None}
+                "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload)}
     else:
         roof = {"bound": "hbm", "achieved": head["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": round(head["gbs"] / PEAK_HBM_GBS, 4), "traffic": None}
+                "frac": round(head["gbs"] / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload)}
     roof["kernel"] = gemm_kernels.select_variant(head["M"], head["N"], head["K"], sets[0][0].dtype) \
         if a.variant == "auto" else a.variant
     roof["flops_per_launch"] = flops
