@@ -18,10 +18,11 @@ bool valid_out(int d) { return d == MI355_BF16 || d == MI355_F16; }
 bool tile256_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int in_dtype) {
   const int64_t es = elem_bytes(in_dtype);
   if (M <= 0 || N <= 0 || K <= 0) return false;
-  if ((K * es) % 128 != 0) return false;                    // whole k-steps only
-  if ((lda * es) % 16 != 0 || (ldb * es) % 16 != 0) return false;  // 16-byte row chunks
+  if ((K * es) % 16 != 0) return false;                     // rows are moved in 16-byte chunks
+  if ((lda * es) % 16 != 0 || (ldb * es) % 16 != 0) return false;
   if (N % 4 != 0 || ldc % 4 != 0) return false;             // 8-byte output stores
-  if (256 * lda * es >= (int64_t)1 << 32 || 256 * ldb * es >= (int64_t)1 << 32) return false;
+  // A 256-row panel must stay below 2 GiB: offsets from 2^31 up mark chunks to be dropped.
+  if (256 * lda * es >= (int64_t)1 << 31 || 256 * ldb * es >= (int64_t)1 << 31) return false;
   return true;
 }
 
@@ -69,8 +70,8 @@ const char* mi355_gemm_strerror(int status) {
     case MI355_ERR_DTYPE: return "unsupported dtype: inputs bf16/fp16/e4m3, output bf16/fp16";
     case MI355_ERR_SHAPE:
       return "shape or leading dimension violates a constraint of the requested variant "
-             "(need M,N,K >= 0, lda,ldb >= K, ldc >= N; tiled variants need K*elem_bytes % 128 == 0, "
-             "16-byte aligned rows and N % 4 == 0)";
+             "(need M,N,K >= 0, lda,ldb >= K, ldc >= N; tiled variants need K*elem_bytes % 16 == 0, "
+             "16-byte aligned rows and N % 4 == 0; skinny needs M <= 256 and 16-bit inputs)";
     case MI355_ERR_VARIANT: return "unknown variant, or variant not available for this shape/dtype";
     case MI355_ERR_WORKSPACE: return "workspace is NULL or smaller than mi355_gemm_workspace_bytes()";
     case MI355_ERR_LAUNCH: return "HIP runtime rejected the kernel launch";

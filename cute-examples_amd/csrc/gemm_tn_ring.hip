@@ -47,7 +47,10 @@ namespace {
 
 constexpr int kThreads = 256;
 
-template <class T, class OutT>
+// kRaggedK: K*elem_bytes is not a multiple of the 128-byte k-step.  Kept out of the common
+// instantiation because selecting the per-lane offset inside the loop puts a dependent VALU
+// chain in front of every copy and costs ~8 % at 8192^3.
+template <class T, class OutT, bool kRaggedK>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) {
   __shared__ __attribute__((aligned(1024))) uint8_t ring[kSlots * kSlotBytes];
   typedef Geo<T> G;
@@ -69,7 +72,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
 
   const uint32_t lda_b = (uint32_t)(g.lda * T::kBytes), ldb_b = (uint32_t)(g.ldb * T::kBytes);
   const uint32_t k_bytes = (uint32_t)(g.K * T::kBytes);
-  const uint32_t k_steps = __builtin_amdgcn_readfirstlane(k_bytes / kRowBytes);
+  // K need not be a whole number of k-steps: in the last one, chunks past the end of the row are
+  // fetched from an out-of-range offset (the hardware returns zeros), see tail_or_oob below.
+  const uint32_t k_steps = __builtin_amdgcn_readfirstlane((k_bytes + kRowBytes - 1) / kRowBytes);
+  const uint32_t tail_bytes = __builtin_amdgcn_readfirstlane(k_bytes % kRowBytes);
   const int64_t total_tiles = g.tiles_m * g.tiles_n;
 
   // Descriptors of the A and B row panels of a tile; rows past the matrix edge are out of range.
@@ -87,12 +93,16 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
   // chunk (l%8) ^ swizzle(row); swizzle(row) depends only on the copy's parity and l/16, so two
   // per-lane offsets per operand suffice; copy j adds j*8 rows to them.
   const uint32_t r8 = lane >> 3, c8 = lane & 7u;
-  uint32_t voff_a[2], voff_b[2];
+  constexpr uint32_t kOutOfRange = 0x80000000u;  // row panels are smaller than 2 GiB (host check)
+  uint32_t voff_a[2], voff_b[2], tail_a[2], tail_b[2];
 #pragma unroll
   for (int par = 0; par < 2; ++par) {
     const uint32_t chunk = c8 ^ swizzle(par * 8 + r8);
     voff_a[par] = (wave * 64 + r8) * lda_b + chunk * 16;
     voff_b[par] = (wave * 64 + r8) * ldb_b + chunk * 16;
+    const bool tail_or_oob = tail_bytes != 0 && chunk * 16 >= tail_bytes;
+    tail_a[par] = tail_or_oob ? kOutOfRange : voff_a[par];
+    tail_b[par] = tail_or_oob ? kOutOfRange : voff_b[par];
   }
   const uint32_t a_step = __builtin_amdgcn_readfirstlane(8 * lda_b);
   const uint32_t b_step = __builtin_amdgcn_readfirstlane(8 * ldb_b);
@@ -104,12 +114,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
   // past the edge of the matrix read zeros); the scalar offset carries the k-step and is kept
   // inside the row by re-reading the last k-step for kt past the end (the slot is never used).
   auto copy_a = [&](__amdgpu_buffer_rsrc_t rsrc, int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
-    const uint32_t soff = (kt < k_steps ? kt : k_steps - 1) * kRowBytes;
-    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff_a[j & 1] + j * a_step, rsrc, soff);
+    const uint32_t kk = kt < k_steps ? kt : k_steps - 1;
+    const uint32_t voff = kRaggedK && kk == k_steps - 1 ? tail_a[j & 1] : voff_a[j & 1];
+    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff + j * a_step, rsrc, kk * kRowBytes);
   };
   auto copy_b = [&](__amdgpu_buffer_rsrc_t rsrc, int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
-    const uint32_t soff = (kt < k_steps ? kt : k_steps - 1) * kRowBytes;
-    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff_b[j & 1] + j * b_step, rsrc, soff);
+    const uint32_t kk = kt < k_steps ? kt : k_steps - 1;
+    const uint32_t voff = kRaggedK && kk == k_steps - 1 ? tail_b[j & 1] : voff_b[j & 1];
+    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff + j * b_step, rsrc, kk * kRowBytes);
   };
   // Opening copies of a tile: A0 B0 A1 B1 A2 into slots 0..4.
   auto open_tile = [&](__amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb) __attribute__((always_inline)) {
@@ -312,7 +324,10 @@ int launch(const GemmArgs& g, hipStream_t stream) {
   const int64_t tiles = g.tiles_m * g.tiles_n;
   const int64_t cus = compute_units();
   const int64_t blocks = tiles < cus ? tiles : cus;  // one resident workgroup per CU (LDS-bound)
-  hipLaunchKernelGGL((gemm_tn_tile256_ring<T, OutT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, g);
+  if ((g.K * T::kBytes) % kRowBytes == 0)
+    hipLaunchKernelGGL((gemm_tn_tile256_ring<T, OutT, false>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, g);
+  else
+    hipLaunchKernelGGL((gemm_tn_tile256_ring<T, OutT, true>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, g);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

@@ -52,7 +52,10 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
 
   const uint32_t ldx_b = (uint32_t)(g.lda * T::kBytes), ldw_b = (uint32_t)(g.ldb * T::kBytes);
   const uint32_t k_bytes = (uint32_t)(g.K * T::kBytes);
-  const uint32_t steps_total = k_bytes / kRowBytes;
+  // The host only splits K when the k-steps divide evenly; a ragged last k-step (K*elem_bytes not
+  // a multiple of 128) is handled by fetching its missing chunks from an out-of-range offset.
+  const uint32_t steps_total = (k_bytes + kRowBytes - 1) / kRowBytes;
+  const uint32_t tail_bytes = __builtin_amdgcn_readfirstlane(k_bytes % kRowBytes);
   const uint32_t steps = __builtin_amdgcn_readfirstlane(steps_total / (uint32_t)splits);
   const uint32_t step0 = __builtin_amdgcn_readfirstlane(split * steps);
   const int64_t rows_x = g.M - m0 < kTm ? g.M - m0 : kTm;
@@ -69,15 +72,18 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
   const uint32_t r8 = lane >> 3, c8 = lane & 7u;
   const uint32_t ring0 = __builtin_amdgcn_readfirstlane(lds_address(ring));
   auto issue_step = [&](uint32_t stage, uint32_t kt) __attribute__((always_inline)) {
-    const uint32_t soff = (kt < steps ? step0 + kt : step0 + steps - 1) * kRowBytes;
+    const uint32_t kk = kt < steps ? step0 + kt : step0 + steps - 1;
+    const uint32_t soff = kk * kRowBytes;
+    const bool ragged = tail_bytes != 0 && kk == steps_total - 1;
 #pragma unroll
     for (int i = 0; i < kCpw; ++i) {
       const uint32_t c = (wave + 4 * i) % kCopies;
       const uint32_t row = c * 8 + r8;                   // row inside the stage: X rows, then W rows
       const uint32_t chunk = c8 ^ swizzle(row);
       const uint32_t dst = ring0 + stage * kStageBytes + c * 1024;
-      if (c < kXCopies) dma_16B_to_lds(dst, row * ldx_b + chunk * 16, rsrc_x, soff);   // c is wave-uniform
-      else dma_16B_to_lds(dst, (row - kTm) * ldw_b + chunk * 16, rsrc_w, soff);
+      const uint32_t drop = ragged && chunk * 16 >= tail_bytes ? 0x80000000u : 0u;  // panels are < 2 GiB
+      if (c < kXCopies) dma_16B_to_lds(dst, (row * ldx_b + chunk * 16) | drop, rsrc_x, soff);   // c is wave-uniform
+      else dma_16B_to_lds(dst, ((row - kTm) * ldw_b + chunk * 16) | drop, rsrc_w, soff);
     }
   };
 
@@ -190,7 +196,7 @@ int launch_m(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
 int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
   const int64_t tm = M <= 16 ? 16 : M <= 32 ? 32 : M <= 64 ? 64 : M <= 128 ? 128 : 256;
   const int64_t tiles = ((M + tm - 1) / tm) * ((N + kTileN - 1) / kTileN);
-  const int64_t steps = K * elem_bytes / kRowBytes;
+  const int64_t steps = (K * elem_bytes + kRowBytes - 1) / kRowBytes;
   const int64_t want = 2 * 256;  // MI355X has 256 CUs; a heuristic only, so no device query here
   int best = 1;
   for (int s = 1; s <= 16; ++s) {

@@ -69,7 +69,9 @@ enum mi355_status {
  *
  * Replaces test::gemm_tn_test (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92): same operand
  * layout and the argument checks of :15-41, plus checks of C the reference omits; divisibility
- * by the tile is not required.  Asynchronous: returns after enqueueing.
+ * by the tile is not required (the tiled variants need K*elem_bytes % 16 == 0, row strides that
+ * are multiples of 16 bytes, N % 4 == 0 and ldc % 4 == 0; MI355_VARIANT_AUTO routes anything else
+ * to the generic kernel).  Asynchronous: returns after enqueueing.
  */
 int mi355_gemm_tn(const void *A, const void *B, void *C,
                   int64_t M, int64_t N, int64_t K,

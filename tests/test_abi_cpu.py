@@ -35,11 +35,13 @@ def test_version_and_strerror(abi):
     ((-1, 256, 64, 64, 64, 256, ac.BF16, ac.BF16, ac.AUTO), ac.ERR_SHAPE),
     ((256, 256, 64, 32, 64, 256, ac.BF16, ac.BF16, ac.AUTO), ac.ERR_SHAPE),   # lda < K
     ((256, 256, 64, 64, 64, 128, ac.BF16, ac.BF16, ac.AUTO), ac.ERR_SHAPE),   # ldc < N
-    ((256, 256, 72, 72, 72, 256, ac.BF16, ac.BF16, ac.BASIC), ac.ERR_SHAPE),  # K bytes % 128
-    ((256, 256, 72, 72, 72, 256, ac.BF16, ac.BF16, ac.AUTO), ac.OK),          # AUTO falls back
+    ((256, 256, 72, 72, 72, 256, ac.BF16, ac.BF16, ac.BASIC), ac.OK),         # ragged last k-step
+    ((256, 256, 68, 72, 72, 256, ac.BF16, ac.BF16, ac.BASIC), ac.ERR_SHAPE),  # K bytes % 16
+    ((256, 256, 68, 72, 72, 256, ac.BF16, ac.BF16, ac.AUTO), ac.OK),          # AUTO falls back
     ((16, 30, 7, 7, 7, 30, ac.F16, ac.F16, ac.SIMPLE), ac.OK),
     ((256, 256, 128, 128, 128, 256, ac.E4M3, ac.BF16, ac.BASIC), ac.OK),
-    ((256, 256, 64, 64, 64, 256, ac.E4M3, ac.BF16, ac.BASIC), ac.ERR_SHAPE),  # 64 fp8 bytes < k-step
+    ((256, 256, 64, 64, 64, 256, ac.E4M3, ac.BF16, ac.BASIC), ac.OK),         # half a k-step of fp8
+    ((256, 256, 24, 32, 32, 256, ac.E4M3, ac.BF16, ac.BASIC), ac.ERR_SHAPE),  # 24 fp8 bytes % 16
     ((64, 256, 128, 128, 128, 256, ac.BF16, ac.BF16, ac.SKINNY), ac.OK),
     ((257, 256, 128, 128, 128, 256, ac.BF16, ac.BF16, ac.SKINNY), ac.ERR_SHAPE),     # M > 256
     ((64, 256, 128, 128, 128, 256, ac.E4M3, ac.BF16, ac.SKINNY), ac.ERR_SHAPE),      # fp8

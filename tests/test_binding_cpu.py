@@ -46,7 +46,7 @@ def test_variant_argument():
     A, B, C = _abc()
     with pytest.raises(RuntimeError, match="unknown variant"):
         gemm_kernels.gemm_tn(A, B, C, "fastest")
-    A, B, C = _abc(K=72)
+    A, B, C = _abc(K=68)
     with pytest.raises(RuntimeError, match="constraint"):
         gemm_kernels.gemm_tn(A, B, C, variant="basic")
     with pytest.raises(RuntimeError, match="HIP device"):  # auto falls back to the simple kernel

@@ -135,6 +135,7 @@ def test_fp8_per_tensor_scaled(abi, size, variant):
 
 @pytest.mark.parametrize("variant", [ac.AUTO] + TILED + [ac.SIMPLE])
 @pytest.mark.parametrize("M,N,K", [(300, 260, 256), (16, 512, 128), (1, 4, 64), (257, 1028, 192), (5000, 4100, 512),
+                                   (512, 512, 8), (300, 516, 72), (768, 260, 1000), (520, 256, 328),
                                    (256, 256, 64), (511, 252, 640)])
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
 def test_ragged_shapes(abi, dt, M, N, K, variant):
@@ -144,7 +145,7 @@ def test_ragged_shapes(abi, dt, M, N, K, variant):
     assert oracle.rel_frobenius(C, oracle.c_gemm_tn_f32(A, B)) <= TOL[dt]
 
 
-@pytest.mark.parametrize("M,N,K", [(5, 7, 3), (33, 17, 50), (100, 30, 77), (64, 64, 8)])
+@pytest.mark.parametrize("M,N,K", [(5, 7, 3), (33, 17, 50), (100, 30, 77), (64, 64, 4)])
 @pytest.mark.parametrize("dt", list(DTYPES.values()))
 def test_shapes_only_the_simple_kernel_takes(abi, dt, M, N, K):
     A, B = rand((M, K), 3, torch.float32).clamp_(-100, 100).to(dt), rand((N, K), 4, torch.float32).clamp_(-100, 100).to(dt)
@@ -154,6 +155,16 @@ def test_shapes_only_the_simple_kernel_takes(abi, dt, M, N, K):
     assert oracle.rel_frobenius(C, ref) <= TOL[dt]
     rc = ac.gemm_tn(abi, A.cuda(), B.cuda(), torch.empty(M, N, dtype=out_dtype_of(dt), device="cuda"), 1.0, ac.BASIC)
     assert rc == ac.ERR_SHAPE
+
+
+@pytest.mark.parametrize("variant", TILED)
+@pytest.mark.parametrize("K", [16, 48, 144, 400])
+def test_fp8_ragged_last_k_step(abi, K, variant):
+    """K*1 byte not a multiple of 128: the missing chunks of the last k-step must read as zeros."""
+    A = rand((300, K), 1, torch.float32).clamp_(-100, 100).to(torch.float8_e4m3fn)
+    B = rand((264, K), 2, torch.float32).clamp_(-100, 100).to(torch.float8_e4m3fn)
+    C = run_abi(abi, A, B, variant, 0.5)
+    check(C, A, B, 0.5)
 
 
 def test_k_zero_and_empty(abi):
@@ -232,7 +243,7 @@ def test_config4_skinny_projections(abi, M, N, K):
     assert oracle.rel_frobenius(run_abi(abi, X, W, ac.BASIC), ref) < 4e-3
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 512, 128), (10, 260, 256), (17, 64, 1024), (33, 512, 4096),
+@pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 512, 128), (16, 128, 8), (48, 260, 1096), (256, 64, 4104), (10, 260, 256), (17, 64, 1024), (33, 512, 4096),
                                    (64, 1024, 2048), (100, 640, 1024), (129, 72, 512), (256, 768, 2048)])
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
 def test_skinny_kernel_every_tile_height_and_split(abi, dt, M, N, K):
