@@ -26,7 +26,9 @@ bool tile256_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64
   return true;
 }
 
-// Constraints of the small-M streaming kernel.
+// Constraints of the small-M streaming kernel.  It wins up to M = 64; from there on the
+// 128x128-tile kernel with K splits is faster (measured on the LLM projection shapes).
+constexpr int64_t kSkinnyAutoMaxM = 64;
 bool skinny_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int in_dtype) {
   if (in_dtype == MI355_E4M3) return false;
   if (M > 256) return false;
@@ -46,8 +48,8 @@ int resolve(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t l
             int variant) {
   if (variant == MI355_VARIANT_AUTO) {
     if (!tile256_ok(M, N, K, lda, ldb, ldc, in_dtype)) return MI355_VARIANT_SIMPLE;
-    // One row of 256x256 tiles cannot fill the machine; stream the weights instead.
-    if (skinny_ok(M, N, K, lda, ldb, ldc, in_dtype)) return MI355_VARIANT_SKINNY;
+    // A few rows of activations against a large weight matrix: stream the weights.
+    if (M <= kSkinnyAutoMaxM && skinny_ok(M, N, K, lda, ldb, ldc, in_dtype)) return MI355_VARIANT_SKINNY;
     return MI355_VARIANT_BASIC;
   }
   if (variant == MI355_VARIANT_BASIC || variant == MI355_VARIANT_PINGPONG)
@@ -105,8 +107,10 @@ int mi355_gemm_select_variant(int64_t M, int64_t N, int64_t K, int in_dtype) {
 size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int in_dtype, int variant) {
   if (!valid_in(in_dtype) || M <= 0 || N <= 0 || K <= 0) return 0;
   if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_SIMPLE) return 0;
-  if (resolve(M, N, K, K, K, N, in_dtype, variant) != MI355_VARIANT_SKINNY) return 0;
-  const int splits = mi355::stream_splits(M, N, K, elem_bytes(in_dtype));
+  const int v = resolve(M, N, K, K, K, N, in_dtype, variant);
+  int splits = 1;
+  if (v == MI355_VARIANT_SKINNY) splits = mi355::stream_splits(M, N, K, elem_bytes(in_dtype));
+  else if (v == MI355_VARIANT_BASIC) splits = mi355::ring_splits(M, N, K, elem_bytes(in_dtype));
   return splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 
@@ -125,6 +129,8 @@ int mi355_gemm_tn(const void* A, const void* B, void* C, int64_t M, int64_t N, i
   g.M = M; g.N = N; g.K = K;
   g.lda = lda; g.ldb = ldb; g.ldc = ldc;
   g.scale = scale;
+  g.splits = 1;
+  g.partial = nullptr;
   hipStream_t s = (hipStream_t)stream;
 
   if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG || v == MI355_VARIANT_SKINNY) {
@@ -144,10 +150,18 @@ int mi355_gemm_tn(const void* A, const void* B, void* C, int64_t M, int64_t N, i
     g.tiles_m = g.tiles_n = 0;
     rc = mi355::launch_stream(g, in_dtype, out_dtype, splits, workspace, s);
   } else if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG) {
-    g.tiles_m = (M + 255) / 256;
-    g.tiles_n = (N + 255) / 256;
+    const int tile = v == MI355_VARIANT_PINGPONG ? 256 : mi355::ring_tile_edge(M, N);
+    if (v == MI355_VARIANT_BASIC) {
+      const int splits = mi355::ring_splits(M, N, K, elem_bytes(in_dtype));
+      const size_t need = splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0;
+      if (need && (!workspace || workspace_bytes < need || (uintptr_t)workspace % 16 != 0)) return MI355_ERR_WORKSPACE;
+      g.splits = splits;
+      g.partial = (float*)workspace;
+    }
+    g.tiles_m = (M + tile - 1) / tile;
+    g.tiles_n = (N + tile - 1) / tile;
     rc = v == MI355_VARIANT_PINGPONG ? mi355::launch_tile256_pingpong(g, in_dtype, out_dtype, s)
-                                     : mi355::launch_tile256_ring(g, in_dtype, out_dtype, s);
+                                     : mi355::launch_tile_ring(g, in_dtype, out_dtype, tile, s);
   } else {
     g.tiles_m = g.tiles_n = 0;
     rc = mi355::launch_simple(g, in_dtype, out_dtype, s);

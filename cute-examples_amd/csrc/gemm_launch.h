@@ -14,12 +14,24 @@ struct GemmArgs {
   int64_t lda, ldb, ldc;
   int64_t tiles_m, tiles_n;
   float scale;
+  // K split: with splits > 1 every (tile, split) pair is a work item that covers k-steps
+  // [split*steps/splits, (split+1)*steps/splits) and writes its unscaled fp32 partial tile to
+  // partial[split][M][N]; launch_splitk_reduce then adds the splits in order, scales and rounds.
+  int32_t splits;
+  float* partial;
 };
 
 // Each returns 0 after a successful enqueue, non-zero if the runtime rejected the launch.
 // in_dtype / out_dtype use the numbering of enum mi355_dtype.
 int launch_tile256_pingpong(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
-int launch_tile256_ring(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
+// Single-wave-group ring kernel; tile is 256 or 128 (ring_tile_edge and ring_splits are pure host
+// heuristics).
+int ring_tile_edge(int64_t M, int64_t N);
+int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes);
+// C = rne(scale * sum_s partial[s]) for partial laid out [splits][M][N] in fp32.
+int launch_splitk_reduce(const float* partial, void* C, int64_t M, int64_t N, int64_t ldc, int splits,
+                         float scale, int out_dtype, hipStream_t stream);
+int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, hipStream_t stream);
 // Skinny (small-M) weight-streaming kernel.  stream_splits is a pure host function.
 int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes);
 int launch_stream(const GemmArgs& g, int in_dtype, int out_dtype, int splits, void* workspace, hipStream_t stream);

@@ -32,6 +32,7 @@ namespace mi355 {
 namespace {
 
 constexpr int kThreads = 512;
+constexpr int kSlotBytes = kTile * kRowBytes;  // 32 KiB: one operand, one k-step
 
 // kRaggedK: K*elem_bytes is not a multiple of the 128-byte k-step.  Kept out of the common
 // instantiation because selecting the per-lane offset inside the loop puts a dependent VALU

@@ -1,5 +1,6 @@
-// "basic" variant: 256x256 output tile, ONE wave group of 4 waves (one per SIMD), each wave owning
-// a 128x128 sub-tile held in 256 fp32 accumulator registers per lane.
+// "basic" variant: 256x256 (or 128x128) output tile, ONE wave group of 4 waves (one per SIMD), each
+// wave owning a quarter of it (128x128 held in 256 fp32 accumulator registers per lane for the
+// 256 tile, which the description below uses).
 //
 // Data path per k-step (128 bytes of K per row: 64 bf16/fp16 or 128 fp8 elements):
 //
@@ -42,6 +43,8 @@
 #include "ring_common.h"
 #include "tile_map.h"
 
+#include <type_traits>
+
 namespace mi355 {
 namespace {
 
@@ -50,14 +53,21 @@ constexpr int kThreads = 256;
 // kRaggedK: K*elem_bytes is not a multiple of the 128-byte k-step.  Kept out of the common
 // instantiation because selecting the per-lane offset inside the loop puts a dependent VALU
 // chain in front of every copy and costs ~8 % at 8192^3.
-template <class T, class OutT, bool kRaggedK>
-__global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) {
+// kTileT: rows of A and of B per workgroup, 256 or 128.  The 128 variant (64x64 per wave, 80 KiB
+// ring, two workgroups per CU) is for problems with too few 256x256 tiles to occupy the CUs; it
+// moves twice the bytes per flop, so it is copy-bound at about two thirds of the MFMA rate.
+template <class T, class OutT, bool kRaggedK, int kTileT>
+__global__ __launch_bounds__(kThreads, kTileT == 256 ? 1 : 2) void gemm_tn_tile_ring(GemmArgs g) {
+  constexpr int kTile = kTileT;
+  constexpr int kSlotBytes = kTile * kRowBytes;   // one operand, one k-step
+  constexpr int kWaveTile = kTile / 2;            // rows and columns per wave
+  constexpr int kCph = kTile / 32;                // copies (8 rows each) per operand per k-step per wave
   __shared__ __attribute__((aligned(1024))) uint8_t ring[kSlots * kSlotBytes];
   typedef Geo<T> G;
   typedef typename G::Frag Frag;
   typedef typename G::Acc Acc;
   constexpr int kBlk = G::kBlk;
-  constexpr int kNb = 128 / kBlk;                       // blocks per wave per dimension
+  constexpr int kNb = kWaveTile / kBlk;                 // blocks per wave per dimension
   constexpr int kSliceChunks = G::kGroups * G::kCpl;    // chunks of a row consumed per slice
   constexpr int kSlices = 8 / kSliceChunks;
   constexpr int kAccLen = kBlk * kBlk / 64;
@@ -77,6 +87,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
   const uint32_t k_steps = __builtin_amdgcn_readfirstlane((k_bytes + kRowBytes - 1) / kRowBytes);
   const uint32_t tail_bytes = __builtin_amdgcn_readfirstlane(k_bytes % kRowBytes);
   const int64_t total_tiles = g.tiles_m * g.tiles_n;
+  // Work items are (tile, split) pairs, split-major, so that workgroups running together read the
+  // same range of K.  steps is the number of k-steps of one item.
+  const int64_t total_items = total_tiles * g.splits;
+  const uint32_t steps = __builtin_amdgcn_readfirstlane(k_steps / (uint32_t)g.splits);
 
   // Descriptors of the A and B row panels of a tile; rows past the matrix edge are out of range.
   auto panel_a = [&](int64_t m0) __attribute__((always_inline)) {
@@ -98,8 +112,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
 #pragma unroll
   for (int par = 0; par < 2; ++par) {
     const uint32_t chunk = c8 ^ swizzle(par * 8 + r8);
-    voff_a[par] = (wave * 64 + r8) * lda_b + chunk * 16;
-    voff_b[par] = (wave * 64 + r8) * ldb_b + chunk * 16;
+    voff_a[par] = (wave * (kCph * 8) + r8) * lda_b + chunk * 16;
+    voff_b[par] = (wave * (kCph * 8) + r8) * ldb_b + chunk * 16;
     const bool tail_or_oob = tail_bytes != 0 && chunk * 16 >= tail_bytes;
     tail_a[par] = tail_or_oob ? kOutOfRange : voff_a[par];
     tail_b[par] = tail_or_oob ? kOutOfRange : voff_b[par];
@@ -107,41 +121,42 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
   const uint32_t a_step = __builtin_amdgcn_readfirstlane(8 * lda_b);
   const uint32_t b_step = __builtin_amdgcn_readfirstlane(8 * ldb_b);
   const uint32_t ring0 = __builtin_amdgcn_readfirstlane(lds_address(ring));
-  const uint32_t dma_wave = ring0 + wave * 8192;  // this wave's 8 KiB inside a slot
+  const uint32_t dma_wave = ring0 + wave * (kCph * 1024);  // this wave's share of a slot
 
   // Copy j (0..7) of an operand's k-step kt into slot `slot`.  The row part of the address stays
   // in the vector offset, the only part the hardware range-checks against the descriptor (rows
   // past the edge of the matrix read zeros); the scalar offset carries the k-step and is kept
-  // inside the row by re-reading the last k-step for kt past the end (the slot is never used).
+  // inside the row by re-reading the item's last k-step for kt past its end (the slot is never used).
+  uint32_t step0 = 0;  // first k-step of the current item
   auto copy_a = [&](__amdgpu_buffer_rsrc_t rsrc, int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
-    const uint32_t kk = kt < k_steps ? kt : k_steps - 1;
-    const uint32_t voff = kRaggedK && kk == k_steps - 1 ? tail_a[j & 1] : voff_a[j & 1];
+    const uint32_t kk = step0 + (kt < steps ? kt : steps - 1);
+    const uint32_t voff = kRaggedK && kk == k_steps - 1 ? tail_a[j & 1] : voff_a[j & 1];  // kk is global
     dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff + j * a_step, rsrc, kk * kRowBytes);
   };
   auto copy_b = [&](__amdgpu_buffer_rsrc_t rsrc, int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
-    const uint32_t kk = kt < k_steps ? kt : k_steps - 1;
+    const uint32_t kk = step0 + (kt < steps ? kt : steps - 1);
     const uint32_t voff = kRaggedK && kk == k_steps - 1 ? tail_b[j & 1] : voff_b[j & 1];
     dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff + j * b_step, rsrc, kk * kRowBytes);
   };
   // Opening copies of a tile: A0 B0 A1 B1 A2 into slots 0..4.
   auto open_tile = [&](__amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb) __attribute__((always_inline)) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) copy_a(ra, j, 0, 0);
+    for (int j = 0; j < kCph; ++j) copy_a(ra, j, 0, 0);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) copy_b(rb, j, 1, 0);
+    for (int j = 0; j < kCph; ++j) copy_b(rb, j, 1, 0);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) copy_a(ra, j, 2, 1);
+    for (int j = 0; j < kCph; ++j) copy_a(ra, j, 2, 1);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) copy_b(rb, j, 3, 1);
+    for (int j = 0; j < kCph; ++j) copy_b(rb, j, 3, 1);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) copy_a(ra, j, 4, 2);
+    for (int j = 0; j < kCph; ++j) copy_a(ra, j, 4, 2);
   };
 
   // Fragment geometry: lane l supplies row l%kBlk of a block; group l/kBlk picks the chunks.
   const uint32_t rblk = lane & (kBlk - 1), grp = lane / kBlk;
   const uint32_t swz = swizzle(rblk);  // block bases are multiples of 16 rows
-  const uint32_t a_lane = (wm * 128 + rblk) * kRowBytes;
-  const uint32_t b_lane = (wn * 128 + rblk) * kRowBytes;
+  const uint32_t a_lane = (wm * kWaveTile + rblk) * kRowBytes;
+  const uint32_t b_lane = (wn * kWaveTile + rblk) * kRowBytes;
   // Byte offset inside a row of the e-th chunk this lane reads in slice s.
   auto chunk_off = [&](int s, int e) __attribute__((always_inline)) -> uint32_t {
     return ((uint32_t)(s * kSliceChunks + grp * G::kCpl + e) ^ swz) << 4;
@@ -196,10 +211,28 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
   auto pack_quad = [&](const Acc& a, int q) __attribute__((always_inline)) -> u32x2 {
     return Pack4<OutT>::run(a[4 * q] * scale, a[4 * q + 1] * scale, a[4 * q + 2] * scale, a[4 * q + 3] * scale);
   };
+  // Split-K items store the raw fp32 accumulators instead: 4 consecutive columns per register quad.
+  auto store_partial = [&](int64_t m0, int64_t n0, uint32_t split) __attribute__((always_inline)) {
+    float* base = g.partial + (int64_t)split * g.M * g.N;
+#pragma unroll
+    for (int i = 0; i < kNb; ++i) {
+      const int64_t m = m0 + wm * kWaveTile + i * kBlk + rblk;
+      if (m >= g.M) continue;
+#pragma unroll
+      for (int j = 0; j < kNb; ++j) {
+#pragma unroll
+        for (int q = 0; q < kAccLen / 4; ++q) {
+          const int64_t n = n0 + wn * kWaveTile + j * kBlk + q * 4 * G::kGroups + grp * 4;
+          if (n + 4 <= g.N)
+            *(f32x4*)(base + m * g.N + n) = (f32x4){acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+        }
+      }
+    }
+  };
   auto epilogue = [&](int64_t m0, int64_t n0) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kNb; ++i) {
-      const int64_t m = m0 + wm * 128 + i * kBlk + rblk;
+      const int64_t m = m0 + wm * kWaveTile + i * kBlk + rblk;
       if constexpr (kBlk == 16) {
         // lane group g = l/16 holds columns 4g..4g+3 of every 16-wide block.  After swapping the
         // odd groups of block j with the even groups of block j+1, groups 0,2 hold columns
@@ -209,7 +242,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
           u32x2 x = pack_quad(acc[i][j], 0), y = pack_quad(acc[i][j + 1], 0);
           u32x2 lo = __builtin_amdgcn_permlane16_swap(x[0], y[0], false, false);
           u32x2 hi = __builtin_amdgcn_permlane16_swap(x[1], y[1], false, false);
-          const int64_t n = n0 + wn * 128 + (j + (grp & 1)) * 16 + (grp >> 1) * 8;
+          const int64_t n = n0 + wn * kWaveTile + (j + (grp & 1)) * 16 + (grp >> 1) * 8;
           store8(m, n, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
         }
       } else {
@@ -223,7 +256,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
             u32x2 x = pack_quad(acc[i][j], q), y = pack_quad(acc[i][j], q + 1);
             u32x2 lo = __builtin_amdgcn_permlane32_swap(x[0], y[0], false, false);
             u32x2 hi = __builtin_amdgcn_permlane32_swap(x[1], y[1], false, false);
-            const int64_t n = n0 + wn * 128 + j * 32 + (q >> 1) * 16 + grp * 8;
+            const int64_t n = n0 + wn * kWaveTile + j * 32 + (q >> 1) * 16 + grp * 8;
             store8(m, n, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
           }
         }
@@ -231,9 +264,11 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
     }
   };
 
-  int64_t tile = blockIdx.x;
+  int64_t item = blockIdx.x;
   int64_t tile_m, tile_n;
-  tile_coord(tile, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+  tile_coord(item % total_tiles, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+  uint32_t split = (uint32_t)(item / total_tiles);
+  step0 = __builtin_amdgcn_readfirstlane(split * steps);
   __amdgpu_buffer_rsrc_t rsrc_a = panel_a(tile_m * kTile), rsrc_b = panel_b(tile_n * kTile);
   open_tile(rsrc_a, rsrc_b);
 
@@ -245,14 +280,14 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
 #pragma unroll
         for (int r = 0; r < kAccLen; ++r) acc[i][j][r] = 0.f;
 
-    wait_vmcnt<24>();  // A0 and B0 have landed
+    wait_vmcnt<3 * kCph>();  // A0 and B0 have landed; A1, B1, A2 may be in flight
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int q = 0; q < kReadsPerSlice; ++q)
       read_q(0, q, ring + a_lane, ring + kSlotBytes + b_lane, 0);
 
     uint32_t slot_a = 0;  // slot of A(t); B(t), A(t+1), B(t+1) follow in slot_a+1..+3 (mod 5)
-    for (uint32_t kt = 0; kt < k_steps; ++kt) {
+    for (uint32_t kt = 0; kt < steps; ++kt) {
       const uint32_t slot_b = slot_a + 1 >= kSlots ? slot_a + 1 - kSlots : slot_a + 1;
       const uint32_t slot_a1 = slot_a + 2 >= kSlots ? slot_a + 2 - kSlots : slot_a + 2;
       const uint32_t slot_b1 = slot_a + 3 >= kSlots ? slot_a + 3 - kSlots : slot_a + 3;
@@ -264,14 +299,17 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
       // Event schedule of one k-step, in MFMA positions p = slice * kMfmaPerSlice + u:
       //   reads    one fragment load per MFMA at the start of each slice (for the following slice)
       //   barrier  in slice 0, a few MFMAs after the last read so its data is back
-      //   copies   one every kCopyEvery MFMAs after the barrier, B(t+2) first.  They must not be
+      //   copies   spread evenly over the MFMAs after the barrier, B(t+2) first.  They must not be
       //            issued faster than the texture-address unit retires them (one 1 KiB copy takes
       //            it ~23 cycles and it serves all four waves): a wave whose copy finds the unit's
       //            queue full stalls at issue and its MFMA stream stops with it.
-      constexpr int kBarrierAt = kReadsPerSlice + kMfmaPerSlice / 8;
+      constexpr int kBarrierWant = kReadsPerSlice + kMfmaPerSlice / 8;
+      constexpr int kBarrierAt = kBarrierWant < kMfmaPerSlice ? kBarrierWant : kMfmaPerSlice - 1;
       constexpr int kFirstCopy = kBarrierAt + 1;
-      constexpr int kCopyEvery = (2 * kMfmaPerSlice - kFirstCopy) / 16 > 0 ? (2 * kMfmaPerSlice - kFirstCopy) / 16 : 1;
-      static_assert(kFirstCopy + 15 * kCopyEvery < 2 * kMfmaPerSlice, "copies must fit in the k-step");
+      constexpr int kCopies = 2 * kCph;                                  // B(t+2) then A(t+3)
+      constexpr int kCopySpan = 2 * kMfmaPerSlice - kFirstCopy;          // positions left in the k-step
+      static_assert(kCopySpan > 0, "no room for the copies");
+      // copy c is issued at position kFirstCopy + c * kCopySpan / kCopies (evenly spread)
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
 #pragma unroll
@@ -283,15 +321,19 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
           }
           if (s == 0 && u == kBarrierAt) {
             // My reads of this k-step's slots are back; B(t+1) (and A(t+1) before it) have
-            // landed; only the 8 copies of A(t+2) may still be in flight.
+            // landed; only this wave's copies of A(t+2) may still be in flight.
             wait_lgkmcnt0();
-            wait_vmcnt<8>();
+            wait_vmcnt<kCph>();
             __builtin_amdgcn_s_barrier();
           }
-          if (p >= kFirstCopy && (p - kFirstCopy) % kCopyEvery == 0 && (p - kFirstCopy) / kCopyEvery < 16) {
-            const int c = (p - kFirstCopy) / kCopyEvery;
-            if (c < 8) copy_b(rsrc_b, c, slot_a, kt + 2);
-            else copy_a(rsrc_a, c - 8, slot_b, kt + 3);
+          if (p >= kFirstCopy) {
+#pragma unroll
+            for (int c = 0; c < kCopies; ++c) {
+              if (kFirstCopy + c * kCopySpan / kCopies == p) {
+                if (c < kCph) copy_b(rsrc_b, c, slot_a, kt + 2);
+                else copy_a(rsrc_a, c - kCph, slot_b, kt + 3);
+              }
+            }
           }
           mfma_u(s, u);
           MI355_FENCE();
@@ -306,39 +348,79 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_ring(GemmArgs g) 
     __builtin_amdgcn_s_barrier();
 
     const int64_t done_m0 = tile_m * kTile, done_n0 = tile_n * kTile;
-    tile += gridDim.x;
-    const bool more = tile < total_tiles;
+    const uint32_t done_split = split;
+    item += gridDim.x;
+    const bool more = item < total_items;
     if (more) {
-      tile_coord(tile, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+      tile_coord(item % total_tiles, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
+      split = (uint32_t)(item / total_tiles);
+      step0 = __builtin_amdgcn_readfirstlane(split * steps);
       rsrc_a = panel_a(tile_m * kTile);
       rsrc_b = panel_b(tile_n * kTile);
       open_tile(rsrc_a, rsrc_b);  // in flight while the finished tile is stored
     }
-    epilogue(done_m0, done_n0);
+    if (g.splits > 1) store_partial(done_m0, done_n0, done_split);
+    else epilogue(done_m0, done_n0);
     if (!more) break;
   }
 }
 
-template <class T, class OutT>
-int launch(const GemmArgs& g, hipStream_t stream) {
-  const int64_t tiles = g.tiles_m * g.tiles_n;
-  const int64_t cus = compute_units();
-  const int64_t blocks = tiles < cus ? tiles : cus;  // one resident workgroup per CU (LDS-bound)
+template <class T, class OutT, int kTileT>
+int launch_tile(const GemmArgs& g, hipStream_t stream) {
+  const int64_t items = g.tiles_m * g.tiles_n * g.splits;
+  const int64_t slots = (int64_t)compute_units() * (kTileT == 256 ? 1 : 2);  // resident workgroups (LDS-bound)
+  const int64_t blocks = items < slots ? items : slots;
   if ((g.K * T::kBytes) % kRowBytes == 0)
-    hipLaunchKernelGGL((gemm_tn_tile256_ring<T, OutT, false>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, g);
+    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, false, kTileT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, g);
   else
-    hipLaunchKernelGGL((gemm_tn_tile256_ring<T, OutT, true>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, g);
-  return hipGetLastError() == hipSuccess ? 0 : -1;
+    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, true, kTileT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, g);
+  if (hipGetLastError() != hipSuccess) return -1;
+  if (g.splits > 1)
+    return launch_splitk_reduce(g.partial, g.C, g.M, g.N, g.ldc, g.splits, g.scale, std::is_same<OutT, BF16>::value ? 0 : 1, stream);
+  return 0;
+}
+
+template <class T, class OutT>
+int launch(const GemmArgs& g, int tile, hipStream_t stream) {
+  return tile == 128 ? launch_tile<T, OutT, 128>(g, stream) : launch_tile<T, OutT, 256>(g, stream);
 }
 
 }  // namespace
 
-int launch_tile256_ring(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream) {
+// Tile edge the single-group kernel should use: 256 unless that leaves most CUs idle and the
+// 128x128 variant (about 0.36 of a 256-tile's time per tile, up to two per CU) finishes sooner.
+int ring_tile_edge(int64_t M, int64_t N) {
+  const int64_t cus = 256;  // MI355X; a heuristic only, so no device query here
+  const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
+  const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
+  const double time256 = (double)((t256 + cus - 1) / cus);
+  const double time128 = (double)((t128 + cus - 1) / cus) * 0.36;
+  return time128 < time256 ? 128 : 256;
+}
+
+// K splits for the single-group kernel: only when the tiles alone leave more than half of the CUs
+// idle (the partial tiles cost S*M*N*8 bytes of extra traffic and a second launch), the k-steps
+// divide evenly and every item keeps at least 16 k-steps.
+int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
+  const int tile = ring_tile_edge(M, N);
+  const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile);
+  const int64_t slots = 256;  // one item per CU of an MI355X
+  const int64_t steps = (K * elem_bytes + kRowBytes - 1) / kRowBytes;
+  int best = 1;
+  for (int s = 2; s <= 16; ++s) {
+    if (tiles * s > slots) break;
+    if (steps % s != 0 || steps / s < 16) continue;
+    best = s;
+  }
+  return best;
+}
+
+int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, hipStream_t stream) {
   const bool out_bf16 = out_dtype == 0;
   switch (in_dtype) {
-    case 0: return out_bf16 ? launch<BF16, BF16>(g, stream) : launch<BF16, F16>(g, stream);
-    case 1: return out_bf16 ? launch<F16, BF16>(g, stream) : launch<F16, F16>(g, stream);
-    case 2: return out_bf16 ? launch<E4M3, BF16>(g, stream) : launch<E4M3, F16>(g, stream);
+    case 0: return out_bf16 ? launch<BF16, BF16>(g, tile, stream) : launch<BF16, F16>(g, tile, stream);
+    case 1: return out_bf16 ? launch<F16, BF16>(g, tile, stream) : launch<F16, F16>(g, tile, stream);
+    case 2: return out_bf16 ? launch<E4M3, BF16>(g, tile, stream) : launch<E4M3, F16>(g, tile, stream);
   }
   return -1;
 }

@@ -20,6 +20,8 @@
 #include "gemm_launch.h"
 #include "ring_common.h"
 
+#include <type_traits>
+
 namespace mi355 {
 namespace {
 
@@ -171,12 +173,8 @@ int launch_cfg(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
   hipLaunchKernelGGL((gemm_tn_stream<T, OutT, kMB, kNB, kWM, kWN, kDepth>), dim3((unsigned)tiles, (unsigned)splits),
                      dim3(kThreads), 0, stream, g, partial, splits);
   if (hipGetLastError() != hipSuccess) return -1;
-  if (splits > 1) {
-    const int64_t quads = g.M * (g.N / 4);
-    hipLaunchKernelGGL((splitk_reduce<OutT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, ws,
-                       (uint16_t*)g.C, g.M, g.N, g.ldc, splits, g.scale);
-    if (hipGetLastError() != hipSuccess) return -1;
-  }
+  if (splits > 1)
+    return launch_splitk_reduce(ws, g.C, g.M, g.N, g.ldc, splits, g.scale, std::is_same<OutT, BF16>::value ? 0 : 1, stream);
   return 0;
 }
 
@@ -205,6 +203,17 @@ int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
     if (tiles * s >= want) break;
   }
   return best;
+}
+
+int launch_splitk_reduce(const float* partial, void* C, int64_t M, int64_t N, int64_t ldc, int splits,
+                         float scale, int out_dtype, hipStream_t stream) {
+  const int64_t quads = M * (N / 4);
+  const dim3 grid((unsigned)((quads + 255) / 256));
+  if (out_dtype == 0)
+    hipLaunchKernelGGL((splitk_reduce<BF16>), grid, dim3(256), 0, stream, partial, (uint16_t*)C, M, N, ldc, splits, scale);
+  else
+    hipLaunchKernelGGL((splitk_reduce<F16>), grid, dim3(256), 0, stream, partial, (uint16_t*)C, M, N, ldc, splits, scale);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
 int launch_stream(const GemmArgs& g, int in_dtype, int out_dtype, int splits, void* workspace, hipStream_t stream) {

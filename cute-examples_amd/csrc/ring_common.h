@@ -9,7 +9,6 @@ namespace mi355 {
 
 constexpr int kTile = 256;
 constexpr int kRowBytes = 128;
-constexpr int kSlotBytes = kTile * kRowBytes;  // 32 KiB: one operand, one k-step
 constexpr int kSlots = 5;
 
 __device__ __forceinline__ uint32_t swizzle(uint32_t row) { return (row >> 1) & 7u; }

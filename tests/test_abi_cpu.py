@@ -64,18 +64,21 @@ def test_workspace_bytes(abi):
     f = abi.mi355_gemm_workspace_bytes
     assert f(8192, 8192, 8192, ac.BF16, ac.AUTO) == 0
     assert f(8192, 8192, 8192, ac.BF16, ac.BASIC) == 0
+    assert f(8192, 8192, 8192, ac.BF16, ac.PINGPONG) == 0
+    assert f(256, 4096, 14336, ac.BF16, ac.BASIC) == 4 * 256 * 4096 * 4        # 64 tiles of 128x128 -> 4 K splits
     assert f(16, 512, 128, ac.BF16, ac.SKINNY) == 0              # too few k-steps to split
     need = f(16, 4096, 14336, ac.BF16, ac.AUTO)
     assert need > 0 and need % (16 * 4096 * 4) == 0 and need // (16 * 4096 * 4) <= 16
-    assert f(16, 4096, 14336, ac.BF16, ac.BASIC) == 0
-    assert f(16, 4096, 14336, ac.E4M3, ac.AUTO) == 0             # fp8 has no streaming kernel
+    assert f(16, 4096, 14336, ac.BF16, ac.PINGPONG) == 0
+    assert f(16, 4096, 14336, ac.E4M3, ac.AUTO) == f(16, 4096, 14336, ac.E4M3, ac.BASIC) > 0   # fp8: tiled kernel + K splits
     assert f(-1, 4096, 14336, ac.BF16, ac.AUTO) == 0 and f(16, 4096, 14336, 9, ac.AUTO) == 0
 
 
 def test_select_variant(abi):
     assert abi.mi355_gemm_select_variant(8192, 8192, 8192, ac.BF16) in (ac.BASIC, ac.PINGPONG)
     assert abi.mi355_gemm_select_variant(16, 14336, 4096, ac.BF16) == ac.SKINNY
-    assert abi.mi355_gemm_select_variant(256, 4096, 14336, ac.F16) == ac.SKINNY
+    assert abi.mi355_gemm_select_variant(64, 4096, 14336, ac.F16) == ac.SKINNY
+    assert abi.mi355_gemm_select_variant(256, 4096, 14336, ac.F16) == ac.BASIC   # 128x128 tiles + K splits
     assert abi.mi355_gemm_select_variant(16, 14336, 4096, ac.E4M3) == ac.BASIC
     assert abi.mi355_gemm_select_variant(100, 30, 77, ac.BF16) == ac.SIMPLE
     assert abi.mi355_gemm_select_variant(8192, 8192, 8192, 9) == ac.ERR_DTYPE
