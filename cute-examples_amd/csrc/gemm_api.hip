@@ -11,7 +11,7 @@ namespace {
 
 int elem_bytes(int dtype) { return dtype == MI355_E4M3 ? 1 : 2; }
 
-bool valid_in(int d) { return d == MI355_BF16 || d == MI355_F16 || d == MI355_E4M3; }
+bool valid_in(int d) { return d == MI355_BF16 || d == MI355_F16 || d == MI355_E4M3; }  // MI355_F32: quantiser only
 bool valid_out(int d) { return d == MI355_BF16 || d == MI355_F16; }
 
 // Constraints of the 256x256-tile kernels beyond the generic ones.
@@ -114,9 +114,26 @@ size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int in_dtype,
   return splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 
+int mi355_quantize_e4m3(const void* x, int x_dtype, int64_t n, void* x_q, float* scale_amax, void* stream) {
+  if (x_dtype != MI355_BF16 && x_dtype != MI355_F16 && x_dtype != MI355_F32) return MI355_ERR_DTYPE;
+  if (n < 0) return MI355_ERR_SHAPE;
+  if (!scale_amax || (n > 0 && (!x || !x_q))) return MI355_ERR_NULL;
+  if ((uintptr_t)x % 16 != 0 || (uintptr_t)x_q % 8 != 0 || (uintptr_t)scale_amax % 4 != 0) return MI355_ERR_ALIGN;
+  return mi355::launch_quantize_e4m3(x, x_dtype, n, x_q, scale_amax, (hipStream_t)stream) == 0 ? MI355_OK
+                                                                                              : MI355_ERR_LAUNCH;
+}
+
 int mi355_gemm_tn(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                   int64_t lda, int64_t ldb, int64_t ldc, int in_dtype, int out_dtype, float scale,
                   int variant, void* workspace, size_t workspace_bytes, void* stream) {
+  return mi355_gemm_tn_scaled(A, B, C, M, N, K, lda, ldb, ldc, in_dtype, out_dtype, scale, nullptr, nullptr,
+                              variant, workspace, workspace_bytes, stream);
+}
+
+int mi355_gemm_tn_scaled(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
+                         int64_t lda, int64_t ldb, int64_t ldc, int in_dtype, int out_dtype, float scale,
+                         const float* scale_a, const float* scale_b, int variant, void* workspace,
+                         size_t workspace_bytes, void* stream) {
   int st = check_common(M, N, K, lda, ldb, ldc, in_dtype, out_dtype, variant);
   if (st != MI355_OK) return st;
   if (M == 0 || N == 0) return MI355_OK;  // nothing to write
@@ -131,6 +148,8 @@ int mi355_gemm_tn(const void* A, const void* B, void* C, int64_t M, int64_t N, i
   g.scale = scale;
   g.splits = 1;
   g.partial = nullptr;
+  g.scale_a = scale_a;
+  g.scale_b = scale_b;
   hipStream_t s = (hipStream_t)stream;
 
   if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG || v == MI355_VARIANT_SKINNY) {

@@ -19,7 +19,21 @@ struct GemmArgs {
   // partial[split][M][N]; launch_splitk_reduce then adds the splits in order, scales and rounds.
   int32_t splits;
   float* partial;
+  // Optional device-resident factors (one float each, or null) multiplied into scale by the
+  // kernel that writes C, so that per-tensor fp8 scales never have to visit the host.
+  const float* scale_a;
+  const float* scale_b;
 };
+
+// Effective output scale; wave-uniform, read once per workgroup.
+#if defined(__HIPCC__)
+__device__ __forceinline__ float output_scale(const GemmArgs& g) {
+  float s = g.scale;
+  if (g.scale_a) s *= *g.scale_a;
+  if (g.scale_b) s *= *g.scale_b;
+  return s;
+}
+#endif
 
 // Each returns 0 after a successful enqueue, non-zero if the runtime rejected the launch.
 // in_dtype / out_dtype use the numbering of enum mi355_dtype.
@@ -29,12 +43,13 @@ int launch_tile256_pingpong(const GemmArgs& g, int in_dtype, int out_dtype, hipS
 int ring_tile_edge(int64_t M, int64_t N);
 int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes);
 // C = rne(scale * sum_s partial[s]) for partial laid out [splits][M][N] in fp32.
-int launch_splitk_reduce(const float* partial, void* C, int64_t M, int64_t N, int64_t ldc, int splits,
-                         float scale, int out_dtype, hipStream_t stream);
+int launch_splitk_reduce(const float* partial, const GemmArgs& g, int out_dtype, hipStream_t stream);
 int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, hipStream_t stream);
 // Skinny (small-M) weight-streaming kernel.  stream_splits is a pure host function.
 int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes);
 int launch_stream(const GemmArgs& g, int in_dtype, int out_dtype, int splits, void* workspace, hipStream_t stream);
+// Per-tensor e4m3 quantisation (amax -> scale -> cast); scale_amax points to two floats.
+int launch_quantize_e4m3(const void* x, int in_dtype, int64_t n, void* q, float* scale_amax, hipStream_t stream);
 int launch_simple(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
 
 }  // namespace mi355

@@ -159,7 +159,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_pingpong(GemmArgs
     MI355_FENCE();
   };
 
-  const float scale = g.scale;
+  const float scale = output_scale(g);
   const int64_t ldc = g.ldc;
   uint16_t* const C = (uint16_t*)g.C;
   auto store8 = [&](int64_t m, int64_t n, u32x2 x, u32x2 y) __attribute__((always_inline)) {

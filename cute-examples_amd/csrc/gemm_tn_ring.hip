@@ -191,7 +191,7 @@ __global__ __launch_bounds__(kThreads, kTileT == 256 ? 1 : 2) void gemm_tn_tile_
   //   m = m0 + wm*128 + i*kBlk + l%kBlk,   n = n0 + wn*128 + j*kBlk + q*4*kGroups + 4*(l/kBlk) + e.
   // Two quads that sit 4 columns apart in neighbouring lane groups are swapped so that each lane
   // holds 8 consecutive columns.
-  const float scale = g.scale;
+  const float scale = output_scale(g);
   const int64_t ldc = g.ldc;
   uint16_t* const C = (uint16_t*)g.C;
   auto store8 = [&](int64_t m, int64_t n, u32x2 x, u32x2 y) __attribute__((always_inline)) {
@@ -376,7 +376,7 @@ int launch_tile(const GemmArgs& g, hipStream_t stream) {
     hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, true, kTileT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, g);
   if (hipGetLastError() != hipSuccess) return -1;
   if (g.splits > 1)
-    return launch_splitk_reduce(g.partial, g.C, g.M, g.N, g.ldc, g.splits, g.scale, std::is_same<OutT, BF16>::value ? 0 : 1, stream);
+    return launch_splitk_reduce(g.partial, g, std::is_same<OutT, BF16>::value ? 0 : 1, stream);
   return 0;
 }
 

@@ -18,7 +18,7 @@ __global__ __launch_bounds__(256) void gemm_tn_simple(GemmArgs g) {
   float acc = 0.f;
   for (int64_t k = 0; k < g.K; ++k)
     acc = __builtin_fmaf(Decode<T>::run(g.A, a0 + k), Decode<T>::run(g.B, b0 + k), acc);
-  ((uint16_t*)g.C)[m * g.ldc + n] = Pack4<OutT>::one(acc * g.scale);
+  ((uint16_t*)g.C)[m * g.ldc + n] = Pack4<OutT>::one(acc * output_scale(g));
 }
 
 template <class T, class OutT>

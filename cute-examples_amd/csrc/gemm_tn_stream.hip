@@ -144,7 +144,7 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
       if (partial) {
         *(f32x4*)(partial + ((int64_t)split * g.M + m) * g.N + n) = acc[i][j];
       } else {
-        const float sc = g.scale;
+        const float sc = output_scale(g);
         *(u32x2*)((uint16_t*)g.C + m * g.ldc + n) =
             Pack4<OutT>::run(acc[i][j][0] * sc, acc[i][j][1] * sc, acc[i][j][2] * sc, acc[i][j][3] * sc);
       }
@@ -154,8 +154,11 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
 
 // C[m][n..n+3] = rne(scale * (partial[0] + partial[1] + ... + partial[S-1])), summed in that order.
 template <class OutT>
-__global__ __launch_bounds__(256) void splitk_reduce(const float* partial, uint16_t* C, int64_t M, int64_t N,
-                                                     int64_t ldc, int splits, float scale) {
+__global__ __launch_bounds__(256) void splitk_reduce(const float* partial, GemmArgs g) {
+  uint16_t* C = (uint16_t*)g.C;
+  const int64_t M = g.M, N = g.N, ldc = g.ldc;
+  const int splits = g.splits;
+  const float scale = output_scale(g);
   const int64_t quads_per_row = N / 4;
   const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (q >= M * quads_per_row) return;
@@ -174,45 +177,53 @@ int launch_cfg(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
                      dim3(kThreads), 0, stream, g, partial, splits);
   if (hipGetLastError() != hipSuccess) return -1;
   if (splits > 1)
-    return launch_splitk_reduce(ws, g.C, g.M, g.N, g.ldc, splits, g.scale, std::is_same<OutT, BF16>::value ? 0 : 1, stream);
+  {
+    GemmArgs r = g;
+    r.splits = splits;
+    return launch_splitk_reduce(ws, r, std::is_same<OutT, BF16>::value ? 0 : 1, stream);
+  }
   return 0;
 }
 
+// Ring depth (k-steps) per tile height.  Depths 3..6 measured the same on the LLM projection
+// shapes; the shallow ones leave room for 3-4 workgroups per CU.
+constexpr int kDepth16 = 4, kDepth32 = 4, kDepth64 = 3, kDepth128 = 4, kDepth256 = 3;
+
 template <class T, class OutT>
 int launch_m(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
-  if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, 6>(g, splits, ws, stream);   //  16x64, 10 KiB/step
-  if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, 5>(g, splits, ws, stream);   //  32x64, 12 KiB/step
-  if (g.M <= 64) return launch_cfg<T, OutT, 4, 1, 1, 4, 4>(g, splits, ws, stream);   //  64x64, 16 KiB/step
-  if (g.M <= 128) return launch_cfg<T, OutT, 4, 2, 2, 2, 4>(g, splits, ws, stream);  // 128x64, 24 KiB/step
-  return launch_cfg<T, OutT, 4, 4, 4, 1, 3>(g, splits, ws, stream);                  // 256x64, 40 KiB/step
+  if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, kDepth16>(g, splits, ws, stream);   //  16x64, 10 KiB/step
+  if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, kDepth32>(g, splits, ws, stream);   //  32x64, 12 KiB/step
+  if (g.M <= 64) return launch_cfg<T, OutT, 4, 1, 1, 4, kDepth64>(g, splits, ws, stream);   //  64x64, 16 KiB/step
+  if (g.M <= 128) return launch_cfg<T, OutT, 4, 2, 2, 2, kDepth128>(g, splits, ws, stream);  // 128x64, 24 KiB/step
+  return launch_cfg<T, OutT, 4, 4, 4, 1, kDepth256>(g, splits, ws, stream);                  // 256x64, 40 KiB/step
 }
 
 }  // namespace
 
-// K splits for a skinny problem: enough workgroups to put about two on every CU, each with at
-// least 8 k-steps, and the k-steps must divide evenly.
+// K splits for a skinny problem: as many workgroups as can be resident at once (one wave of
+// workgroups, no tail), each with at least 8 k-steps, and the k-steps must divide evenly.
 int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
   const int64_t tm = M <= 16 ? 16 : M <= 32 ? 32 : M <= 64 ? 64 : M <= 128 ? 128 : 256;
+  const int depth = M <= 16 ? 4 : M <= 32 ? 4 : M <= 64 ? 3 : M <= 128 ? 4 : 3;  // kDepth16 .. kDepth256
+  const int64_t ring_bytes = depth * (tm + kTileN) * kRowBytes;
+  const int64_t per_cu = 163840 / ring_bytes < 8 ? 163840 / ring_bytes : 8;   // LDS-bound residency
+  const int64_t slots = 256 * per_cu;  // MI355X has 256 CUs; a heuristic only, so no device query here
   const int64_t tiles = ((M + tm - 1) / tm) * ((N + kTileN - 1) / kTileN);
   const int64_t steps = (K * elem_bytes + kRowBytes - 1) / kRowBytes;
-  const int64_t want = 2 * 256;  // MI355X has 256 CUs; a heuristic only, so no device query here
   int best = 1;
-  for (int s = 1; s <= 16; ++s) {
+  for (int s = 1; s <= 32; ++s) {
+    if (tiles * s > slots) break;
     if (steps % s != 0 || steps / s < 8) continue;
     best = s;
-    if (tiles * s >= want) break;
   }
   return best;
 }
 
-int launch_splitk_reduce(const float* partial, void* C, int64_t M, int64_t N, int64_t ldc, int splits,
-                         float scale, int out_dtype, hipStream_t stream) {
-  const int64_t quads = M * (N / 4);
+int launch_splitk_reduce(const float* partial, const GemmArgs& g, int out_dtype, hipStream_t stream) {
+  const int64_t quads = g.M * (g.N / 4);
   const dim3 grid((unsigned)((quads + 255) / 256));
-  if (out_dtype == 0)
-    hipLaunchKernelGGL((splitk_reduce<BF16>), grid, dim3(256), 0, stream, partial, (uint16_t*)C, M, N, ldc, splits, scale);
-  else
-    hipLaunchKernelGGL((splitk_reduce<F16>), grid, dim3(256), 0, stream, partial, (uint16_t*)C, M, N, ldc, splits, scale);
+  if (out_dtype == 0) hipLaunchKernelGGL((splitk_reduce<BF16>), grid, dim3(256), 0, stream, partial, g);
+  else hipLaunchKernelGGL((splitk_reduce<F16>), grid, dim3(256), 0, stream, partial, g);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

@@ -1,0 +1,135 @@
+// Per-tensor fp8 quantisation on the device: the step in front of the fp8 GEMM.
+//
+//   amax  = max |x|                       (atomic max over the fp32 bit patterns of |x|)
+//   scale = amax / 448  (1 if amax == 0)  (OCP e4m3 has no infinities; 448 is its largest value)
+//   x_q   = e4m3_rne(clamp(x / scale, -448, 448))
+//
+// so that x ~= scale * x_q.  Three launches on the caller's stream, no host synchronisation: the
+// scale stays in device memory and the GEMM reads it from there.  The reference has no fp8 path;
+// the contract is the benchmark configuration's (operands quantised with per-tensor fp32 scales
+// amax/448) and is checked against torch's float8_e4m3fn cast and the C restatement in the tests.
+#include "cdna4_primitives.h"
+#include "gemm_launch.h"
+
+namespace mi355 {
+namespace {
+
+constexpr float kE4m3Max = 448.0f;
+
+template <class In> struct Load8;  // 8 consecutive elements -> 8 floats
+template <> struct Load8<float> {
+  static __device__ __forceinline__ void run(const void* p, int64_t i, float* v) {
+    const f32x4 a = ((const f32x4*)((const float*)p + i))[0], b = ((const f32x4*)((const float*)p + i))[1];
+    v[0] = a[0]; v[1] = a[1]; v[2] = a[2]; v[3] = a[3]; v[4] = b[0]; v[5] = b[1]; v[6] = b[2]; v[7] = b[3];
+  }
+  static __device__ __forceinline__ float one(const void* p, int64_t i) { return ((const float*)p)[i]; }
+};
+template <> struct Load8<BF16> {
+  static __device__ __forceinline__ void run(const void* p, int64_t i, float* v) {
+    const u32x4 a = *(const u32x4*)((const uint16_t*)p + i);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      v[2 * k] = __builtin_bit_cast(float, a[k] << 16);
+      v[2 * k + 1] = __builtin_bit_cast(float, a[k] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ float one(const void* p, int64_t i) { return Decode<BF16>::run(p, i); }
+};
+template <> struct Load8<F16> {
+  static __device__ __forceinline__ void run(const void* p, int64_t i, float* v) {
+    const f16x8 a = *(const f16x8*)((const _Float16*)p + i);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) v[k] = (float)a[k];
+  }
+  static __device__ __forceinline__ float one(const void* p, int64_t i) { return Decode<F16>::run(p, i); }
+};
+
+__global__ void amax_init(float* out) { out[0] = 1.0f; out[1] = 0.0f; }
+
+// out[1] accumulates amax: for non-negative floats the unsigned order of the bit patterns is the
+// numeric order, so an integer atomic max does it.
+template <class In>
+__global__ __launch_bounds__(256) void amax_kernel(const void* x, int64_t n, float* out) {
+  float m = 0.f;
+  const int64_t stride = (int64_t)gridDim.x * 256 * 8;
+  int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  for (; i + 8 <= n; i += stride) {
+    float v[8];
+    Load8<In>::run(x, i, v);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) m = __builtin_fmaxf(m, __builtin_fabsf(v[k]));
+  }
+  for (; i < n; ++i) m = __builtin_fmaxf(m, __builtin_fabsf(Load8<In>::one(x, i)));  // at most one thread: the tail
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = __builtin_fmaxf(m, __shfl_xor(m, off));
+  __shared__ float wave_max[4];
+  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    m = __builtin_fmaxf(__builtin_fmaxf(wave_max[0], wave_max[1]), __builtin_fmaxf(wave_max[2], wave_max[3]));
+    atomicMax((unsigned*)(out + 1), __builtin_bit_cast(unsigned, m));
+  }
+}
+
+// fp32 -> e4m3 (OCP), round to nearest even, saturating at +-448, NaN -> 0x7f.
+__device__ __forceinline__ uint32_t to_e4m3(float f) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, f);
+  const uint32_t sign = (u >> 24) & 0x80u;
+  const uint32_t a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return 0x7fu;                       // NaN
+  if (a >= 0x43e00000u) return sign | 0x7eu;               // >= 448 (and inf) saturate
+  uint32_t code;
+  if (a < 0x3c800000u) {                                   // < 2^-6: multiples of 2^-9
+    code = (uint32_t)__builtin_rintf(__builtin_bit_cast(float, a) * 512.0f);  // 8 encodes the smallest normal
+  } else {
+    const uint32_t r = a + 0x7ffffu + ((a >> 20) & 1u);    // RNE to 3 mantissa bits, carry into the exponent
+    code = (r >> 20) - (120u << 3);                        // rebias 127 -> 7
+    if (code > 0x7eu) code = 0x7eu;
+  }
+  return sign | code;
+}
+
+template <class In>
+__global__ __launch_bounds__(256) void quantize_kernel(const void* x, int64_t n, uint8_t* q, float* out) {
+  const float amax = out[1];
+  const float scale = amax > 0.f ? amax / kE4m3Max : 1.0f;
+  if (blockIdx.x == 0 && threadIdx.x == 0) out[0] = scale;
+  const int64_t stride = (int64_t)gridDim.x * 256 * 8;
+  int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  for (; i + 8 <= n; i += stride) {
+    float v[8];
+    Load8<In>::run(x, i, v);
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      lo |= to_e4m3(v[k] / scale) << (8 * k);
+      hi |= to_e4m3(v[4 + k] / scale) << (8 * k);
+    }
+    *(u32x2*)(q + i) = (u32x2){lo, hi};
+  }
+  for (; i < n; ++i) q[i] = (uint8_t)to_e4m3(Load8<In>::one(x, i) / scale);
+}
+
+template <class In>
+int run(const void* x, int64_t n, void* q, float* out, hipStream_t stream) {
+  const int64_t want = (n / 8 + 255) / 256;
+  const unsigned blocks = (unsigned)(want < 1 ? 1 : want > 4096 ? 4096 : want);
+  hipLaunchKernelGGL(amax_init, dim3(1), dim3(1), 0, stream, out);
+  hipLaunchKernelGGL((amax_kernel<In>), dim3(blocks), dim3(256), 0, stream, x, n, out);
+  hipLaunchKernelGGL((quantize_kernel<In>), dim3(blocks), dim3(256), 0, stream, x, n, (uint8_t*)q, out);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+}  // namespace
+
+// in_dtype: 0 bf16, 1 fp16, 3 fp32.
+int launch_quantize_e4m3(const void* x, int in_dtype, int64_t n, void* q, float* scale_amax, hipStream_t stream) {
+  switch (in_dtype) {
+    case 0: return run<BF16>(x, n, q, scale_amax, stream);
+    case 1: return run<F16>(x, n, q, scale_amax, stream);
+    case 3: return run<float>(x, n, q, scale_amax, stream);
+  }
+  return -1;
+}
+
+}  // namespace mi355

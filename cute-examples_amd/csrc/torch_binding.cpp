@@ -47,8 +47,16 @@ const char* variant_name(int v) {
   return "?";
 }
 
+// A scale given as a one-element tensor on the GEMM's device is passed by address (no host
+// synchronisation); a Python number or a CPU tensor is folded into the scalar factor.
+struct Scale {
+  float host = 1.0f;
+  const float* device = nullptr;
+  torch::Tensor keep;
+};
+
 torch::Tensor run(const torch::Tensor& A, const torch::Tensor& B, torch::Tensor C, float scale,
-                  int variant, bool fp8) {
+                  int variant, bool fp8, const Scale& sa = Scale(), const Scale& sb = Scale()) {
   // Same order as the reference's checks (gemm_test.cu:15-28), then the ones it lacks.
   TORCH_CHECK(A.device() == B.device(), "All tensors must be on the same device");
   TORCH_CHECK(A.is_contiguous() && B.is_contiguous(), "All tensors must be contiguous");
@@ -90,19 +98,28 @@ torch::Tensor run(const torch::Tensor& A, const torch::Tensor& B, torch::Tensor 
     ws = torch::empty({(int64_t)ws_bytes}, A.options().dtype(torch::kUInt8));
     ws_ptr = ws.data_ptr();
   }
-  st = mi355_gemm_tn(A.const_data_ptr(), B.const_data_ptr(), C.mutable_data_ptr(), M, N, K, K, K,
-                     ldc, in_dt, out_dt, scale, variant, ws_ptr, ws_bytes, (void*)stream);
+  st = mi355_gemm_tn_scaled(A.const_data_ptr(), B.const_data_ptr(), C.mutable_data_ptr(), M, N, K, K, K,
+                            ldc, in_dt, out_dt, scale * sa.host * sb.host, sa.device, sb.device, variant,
+                            ws_ptr, ws_bytes, (void*)stream);
   TORCH_CHECK(st == MI355_OK, "gemm_kernels: ", mi355_gemm_strerror(st));
   return C;
 }
 
-float scalar_of(const pybind11::object& o) {
+Scale scale_of(const pybind11::object& o, const torch::Tensor& like) {
+  Scale s;
   if (THPVariable_Check(o.ptr())) {
     const torch::Tensor& t = THPVariable_Unpack(o.ptr());
     TORCH_CHECK(t.numel() == 1, "a scale tensor must hold exactly one element");
-    return t.item<float>();
+    if (t.is_cuda() && t.device() == like.device() && t.scalar_type() == at::kFloat) {
+      s.keep = t;
+      s.device = t.const_data_ptr<float>();
+    } else {
+      s.host = t.item<float>();
+    }
+  } else {
+    s.host = o.cast<float>();
   }
-  return o.cast<float>();
+  return s;
 }
 
 }  // namespace
@@ -122,7 +139,29 @@ torch::Tensor gemm_tn(const torch::Tensor A, const torch::Tensor B, torch::Tenso
 // C = (scale_a*scale_b) * A_q · B_q^T for per-tensor-scaled float8_e4m3fn operands.
 torch::Tensor gemm_tn_fp8(const torch::Tensor A_q, const torch::Tensor B_q, pybind11::object scale_a,
                           pybind11::object scale_b, torch::Tensor C, const std::string& variant) {
-  return run(A_q, B_q, C, scalar_of(scale_a) * scalar_of(scale_b), variant_code(variant), true);
+  return run(A_q, B_q, C, 1.0f, variant_code(variant), true, scale_of(scale_a, A_q), scale_of(scale_b, A_q));
+}
+
+// (x_q, scale): x_q float8_e4m3fn of x's shape, scale a 0-dim fp32 tensor on x's device, with
+// x ~= scale * x_q, scale = amax|x| / 448.  No host synchronisation.
+std::pair<torch::Tensor, torch::Tensor> quantize_e4m3(const torch::Tensor x) {
+  TORCH_CHECK(x.is_contiguous(), "x must be contiguous");
+  int dt;
+  switch (x.scalar_type()) {
+    case at::kBFloat16: dt = MI355_BF16; break;
+    case at::kHalf: dt = MI355_F16; break;
+    case at::kFloat: dt = MI355_F32; break;
+    default: TORCH_CHECK(false, "x must be bfloat16, float16 or float32");
+  }
+  TORCH_CHECK(x.is_cuda(), "gemm_kernels runs on a HIP device only; got a tensor on ", x.device());
+  c10::DeviceGuard guard(x.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+  torch::Tensor q = torch::empty(x.sizes(), x.options().dtype(at::kFloat8_e4m3fn));
+  torch::Tensor sa = torch::empty({2}, x.options().dtype(at::kFloat));
+  int st = mi355_quantize_e4m3(x.const_data_ptr(), dt, x.numel(), q.mutable_data_ptr(), sa.data_ptr<float>(),
+                               (void*)stream);
+  TORCH_CHECK(st == MI355_OK, "gemm_kernels: ", mi355_gemm_strerror(st));
+  return {q, sa[0]};
 }
 
 std::string select_variant(int64_t M, int64_t N, int64_t K, at::ScalarType dtype) {
@@ -145,6 +184,9 @@ PYBIND11_MODULE(_C, m) {
         "C = scale_a*scale_b * A_q @ B_q.T for float8_e4m3fn operands, bf16/fp16 out",
         py::arg("A_q"), py::arg("B_q"), py::arg("scale_a"), py::arg("scale_b"), py::arg("C"),
         py::arg("variant") = "auto");
+  m.def("quantize_e4m3", &test::quantize_e4m3,
+        "per-tensor fp8 quantisation on the device: returns (x_q float8_e4m3fn, scale 0-dim fp32 tensor)",
+        py::arg("x"));
   m.def("select_variant", &test::select_variant, py::arg("M"), py::arg("N"), py::arg("K"),
         py::arg("dtype"));
   m.def("version", []() { return mi355_gemm_version(); });

@@ -27,7 +27,8 @@ extern "C" {
 enum mi355_dtype {
   MI355_BF16 = 0,
   MI355_F16 = 1,
-  MI355_E4M3 = 2
+  MI355_E4M3 = 2,
+  MI355_F32 = 3   /* accepted by mi355_quantize_e4m3 only */
 };
 
 /* Kernel families.  AUTO picks by shape; the others force one family (and fail with
@@ -78,6 +79,36 @@ int mi355_gemm_tn(const void *A, const void *B, void *C,
                   int64_t lda, int64_t ldb, int64_t ldc,
                   int in_dtype, int out_dtype, float scale, int variant,
                   void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * mi355_gemm_tn with two more factors that live in device memory: C = scale * (*scale_a) *
+ * (*scale_b) * A · B^T.  Either pointer may be NULL (factor 1).  They are read by the kernel that
+ * writes C, so the per-tensor scales produced by mi355_quantize_e4m3 never visit the host.
+ * Counterpart in the reference: none (no fp8 path); same launcher contract as mi355_gemm_tn.
+ */
+int mi355_gemm_tn_scaled(const void *A, const void *B, void *C,
+                         int64_t M, int64_t N, int64_t K,
+                         int64_t lda, int64_t ldb, int64_t ldc,
+                         int in_dtype, int out_dtype, float scale,
+                         const float *scale_a, const float *scale_b, int variant,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Per-tensor fp8 quantisation, the step in front of the fp8 GEMM: amax = max|x|,
+ * scale = amax/448 (1 if amax is 0), x_q[i] = e4m3(x[i]/scale) rounded to nearest even and
+ * saturated at +-448, so that x ~= scale * x_q.
+ *
+ *   x          device pointer, n contiguous elements of x_dtype (MI355_BF16, MI355_F16, MI355_F32),
+ *              16-byte aligned
+ *   x_q        device pointer, n bytes (e4m3), 8-byte aligned
+ *   scale_amax device pointer to two floats: [0] receives scale, [1] is scratch (receives amax)
+ *
+ * Asynchronous on `stream` (three launches, no host synchronisation).  Counterpart in the
+ * reference: none; the contract is the fp8 benchmark configuration's (per-tensor fp32 scales
+ * amax/448).
+ */
+int mi355_quantize_e4m3(const void *x, int x_dtype, int64_t n, void *x_q,
+                        float *scale_amax, void *stream);
 
 /* Scratch bytes mi355_gemm_tn needs for this problem and variant (0 for most shapes).
  * Counterpart: none in the reference (it has no split-K); sizes the split-K partials that

@@ -8,7 +8,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB = os.path.join(ROOT, "cute-examples_amd", "gemm_kernels", "libmi355gemm.so")
 HEADER = os.path.join(ROOT, "include", "mi355_gemm.h")
 
-BF16, F16, E4M3 = 0, 1, 2
+BF16, F16, E4M3, F32 = 0, 1, 2, 3
 AUTO, BASIC, PINGPONG, SKINNY, SIMPLE = 0, 1, 2, 3, 4
 OK, ERR_NULL, ERR_DTYPE, ERR_SHAPE, ERR_VARIANT, ERR_WORKSPACE, ERR_LAUNCH, ERR_ALIGN = 0, -1, -2, -3, -4, -5, -6, -7
 
@@ -17,7 +17,7 @@ def declared_symbols():
     """Function names declared in the public header."""
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(mi355_gemm\w*)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", text)))
 
 
 def load():
@@ -27,6 +27,10 @@ def load():
     i64, vp, ci, f32, sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
     L.mi355_gemm_tn.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, f32, ci, vp, sz, vp]
     L.mi355_gemm_tn.restype = ci
+    L.mi355_gemm_tn_scaled.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, f32, vp, vp, ci, vp, sz, vp]
+    L.mi355_gemm_tn_scaled.restype = ci
+    L.mi355_quantize_e4m3.argtypes = [vp, ci, i64, vp, vp, vp]
+    L.mi355_quantize_e4m3.restype = ci
     L.mi355_gemm_workspace_bytes.argtypes = [i64, i64, i64, ci, ci]
     L.mi355_gemm_workspace_bytes.restype = sz
     L.mi355_gemm_select_variant.argtypes = [i64, i64, i64, ci]

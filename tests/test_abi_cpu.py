@@ -11,7 +11,7 @@ from tests import abi_ctypes as ac
 
 def test_exports_every_declared_symbol(abi):
     names = ac.declared_symbols()
-    assert "mi355_gemm_tn" in names and len(names) >= 7
+    assert {"mi355_gemm_tn", "mi355_gemm_tn_scaled", "mi355_quantize_e4m3"} <= set(names) and len(names) >= 9
     for n in names:
         assert hasattr(abi, n), n
     dyn = subprocess.run(["nm", "-D", "--defined-only", ac.LIB], capture_output=True, text=True).stdout
@@ -58,6 +58,14 @@ def test_gemm_tn_rejects_before_any_device_access(abi):
     assert f(None, None, None, 256, 256, 64, 64, 64, 256, 5, 0, 1.0, 0, None, 0, None) == ac.ERR_DTYPE
     assert f(None, None, None, 256, 256, 64, 8, 64, 256, 0, 0, 1.0, 0, None, 0, None) == ac.ERR_SHAPE
     assert f(None, None, None, 0, 256, 64, 64, 64, 256, 0, 0, 1.0, 0, None, 0, None) == ac.OK  # empty
+
+
+def test_quantize_rejects_before_any_device_access(abi):
+    f = abi.mi355_quantize_e4m3
+    assert f(None, ac.F32, 16, None, None, None) == ac.ERR_NULL
+    assert f(None, ac.E4M3, 16, None, None, None) == ac.ERR_DTYPE
+    assert f(None, ac.F32, -1, None, None, None) == ac.ERR_SHAPE
+    assert f(17, ac.F32, 16, 8, 12, None) == ac.ERR_ALIGN
 
 
 def test_workspace_bytes(abi):

@@ -325,3 +325,63 @@ def test_python_module_variants_streams_and_fp8():
     C = torch.empty(256, 256, dtype=torch.bfloat16, device="cuda")
     gemm_kernels.gemm_tn_fp8(Aq, Bq, sa, sb, C)
     assert oracle.rel_frobenius(C, oracle.gemm_tn_fp32(Aq, Bq, float(sa) * float(sb))) < 3e-2
+
+
+# ---------------------------------------------------------------- device quantiser
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape,std", [((257, 129), 1.0), ((8192, 64), 0.02), ((3, 5), 37.0), ((1, 1), 1.0), ((1000, 1000), 1.0)])
+def test_device_quantiser_matches_oracle_bit_for_bit(dtype, shape, std):
+    import gemm_kernels
+    x = (torch.randn(shape, generator=torch.Generator().manual_seed(shape[0])) * std).to(dtype)
+    q, s = gemm_kernels.quantize_e4m3(x.cuda())
+    q_o, s_o = oracle.quantize_e4m3(x.float())
+    assert q.dtype == torch.float8_e4m3fn and q.shape == x.shape and s.dim() == 0
+    assert float(s) == s_o
+    assert torch.equal(q.cpu().view(torch.uint8), q_o.view(torch.uint8))
+
+
+def test_device_quantiser_every_code_and_every_tie():
+    """amax = 448 makes scale exactly 1, so the kernel's rounding is compared value by value with
+    torch's e4m3fn cast: every representable value, every midpoint between neighbours (ties to
+    even), subnormals and zeros."""
+    import gemm_kernels
+    v = torch.arange(0, 0x7f, dtype=torch.uint8).view(torch.float8_e4m3fn).float().double()
+    mid = (v[:-1] + v[1:]) / 2
+    pts = torch.cat([v, mid, mid * (1 + 2 ** -20), mid * (1 - 2 ** -20), torch.tensor([448.0, 0.0, 2.0 ** -10, 2.0 ** -11])])
+    x = torch.cat([pts, -pts]).float()
+    q, s = gemm_kernels.quantize_e4m3(x.cuda())
+    assert float(s) == 1.0
+    want = x.to(torch.float8_e4m3fn)
+    assert torch.equal(q.cpu().view(torch.uint8) & 0x7f, want.view(torch.uint8) & 0x7f)   # -0 vs +0 sign aside
+    nz = want.float() != 0
+    assert torch.equal(q.cpu().view(torch.uint8)[nz], want.view(torch.uint8)[nz])
+    z, sz = gemm_kernels.quantize_e4m3(torch.zeros(40, device="cuda"))
+    assert float(sz) == 1.0 and not z.float().any()
+
+
+def test_fp8_gemm_with_device_resident_scales(abi):
+    """quantise -> GEMM without a host round trip: the scales stay on the device."""
+    import gemm_kernels
+    a = rand((512, 1024), 80, torch.float32).cuda()
+    b = rand((768, 1024), 81, torch.float32).cuda()
+    (Aq, sa), (Bq, sb) = gemm_kernels.quantize_e4m3(a), gemm_kernels.quantize_e4m3(b)
+    assert sa.is_cuda and sb.is_cuda
+    C = torch.full((512, 768), float("nan"), dtype=torch.bfloat16, device="cuda")
+    gemm_kernels.gemm_tn_fp8(Aq, Bq, sa, sb, C)
+    ref = oracle.gemm_tn_fp32(Aq, Bq, float(sa) * float(sb))
+    assert oracle.no_nan_left(C) and oracle.rel_frobenius(C, ref) < 4e-3
+    C2 = torch.empty_like(C)
+    gemm_kernels.gemm_tn_fp8(Aq, Bq, float(sa), sb.cpu(), C2)      # host-side scales give the same bits
+    assert torch.equal(C, C2)
+    # the same through the C ABI, for every kernel family that takes fp8
+    for variant in (ac.BASIC, ac.PINGPONG, ac.SIMPLE):
+        C3 = torch.empty_like(C)
+        ws_bytes = abi.mi355_gemm_workspace_bytes(512, 768, 1024, ac.E4M3, variant)
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device="cuda")
+        rc = abi.mi355_gemm_tn_scaled(Aq.data_ptr(), Bq.data_ptr(), C3.data_ptr(), 512, 768, 1024, 1024, 1024, 768,
+                                      ac.E4M3, ac.BF16, 1.0, sa.data_ptr(), sb.data_ptr(), variant,
+                                      ws.data_ptr(), ws_bytes, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert oracle.rel_frobenius(C3, ref) < 4e-3, variant
