@@ -43,7 +43,6 @@ __device__ __forceinline__ void dma_16B_to_lds(uint32_t lds_base, uint32_t voffs
                                                __amdgpu_buffer_rsrc_t rsrc, uint32_t soffset) {
   asm volatile(
       "s_mov_b32 m0, %0\n\t"
-      "s_nop 0\n\t"
       "buffer_load_dwordx4 %1, %2, %3 offen lds"
       :
       : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(voffset), "s"(rsrc),

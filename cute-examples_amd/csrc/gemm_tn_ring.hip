@@ -184,7 +184,10 @@ __global__ __launch_bounds__(kThreads, kTileT == 256 ? 1 : 2) void gemm_tn_tile_
   auto mfma_u = [&](int buf, int u) __attribute__((always_inline)) {
     const int i = u / kNb, j = u % kNb;
     // B supplies the MFMA "rows" so each lane ends up with consecutive n of one m.
-    acc[i][j] = G::mfma(fb[buf][j], fa[buf][i], acc[i][j]);
+    // In the 256-wide tile all 256 accumulator registers are live; the in-place form keeps the
+    // compiler from rotating them through copies when it allocates the MFMA's result.
+    if constexpr (kTile == 256) G::mfma_inplace(fb[buf][j], fa[buf][i], acc[i][j]);
+    else acc[i][j] = G::mfma(fb[buf][j], fa[buf][i], acc[i][j]);
   };
 
   // Epilogue of the tile at (m0, n0).  Accumulator register 4q+e of block (i,j) in lane l is C[m][n],

@@ -28,6 +28,14 @@ template <> struct Geo<BF16> {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x),
                                                    __builtin_bit_cast(bf16x8, y), c, 0, 0, 0);
   }
+  // The same instruction with the accumulator tied in place in an accumulation register.  The
+  // single-group 256x256 kernel uses it: with 256 accumulator registers live across a loop
+  // nest the register allocator otherwise rotates a few accumulator tiles through VGPR copies
+  // every k-step.  The callers keep dependent uses of c far apart (64 MFMAs, or a barrier and
+  // the whole tile set-up before the epilogue), beyond any MFMA result hazard.
+  static __device__ __forceinline__ void mfma_inplace(Frag x, Frag y, Acc& c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));
+  }
 };
 template <> struct Geo<F16> {
   static constexpr int kBlk = 16, kGroups = 4, kCpl = 1;
@@ -37,6 +45,9 @@ template <> struct Geo<F16> {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, x),
                                                   __builtin_bit_cast(f16x8, y), c, 0, 0, 0);
   }
+  static __device__ __forceinline__ void mfma_inplace(Frag x, Frag y, Acc& c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));
+  }
 };
 template <> struct Geo<E4M3> {
   static constexpr int kBlk = 32, kGroups = 2, kCpl = 2;
@@ -45,6 +56,7 @@ template <> struct Geo<E4M3> {
   static __device__ __forceinline__ Acc mfma(Frag x, Frag y, Acc c) {
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, c, 0, 0, 0, 0, 0, 0);
   }
+  static __device__ __forceinline__ void mfma_inplace(Frag x, Frag y, Acc& c) { c = mfma(x, y, c); }
 };
 
 
