@@ -23,6 +23,8 @@ bool tile256_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64
   if (N % 4 != 0 || ldc % 4 != 0) return false;             // 8-byte output stores
   // A 256-row panel must stay below 2 GiB: offsets from 2^31 up mark chunks to be dropped.
   if (256 * lda * es >= (int64_t)1 << 31 || 256 * ldb * es >= (int64_t)1 << 31) return false;
+  // 32-bit offsets inside a 256-row tile of C and of an fp32 split-K plane (row stride N <= ldc)
+  if (256 * ldc * 4 >= (int64_t)1 << 31) return false;
   return true;
 }
 

@@ -27,6 +27,7 @@
 #include "gemm_launch.h"
 #include "ring_common.h"
 #include "tile_map.h"
+#include "tile_store.h"
 
 namespace mi355 {
 namespace {
@@ -64,7 +65,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_pingpong(GemmArgs
   // fetched from an out-of-range offset (the hardware returns zeros), see tail_or_oob below.
   const uint32_t k_steps = __builtin_amdgcn_readfirstlane((k_bytes + kRowBytes - 1) / kRowBytes);
   const uint32_t tail_bytes = __builtin_amdgcn_readfirstlane(k_bytes % kRowBytes);
-  const int64_t total_tiles = g.tiles_m * g.tiles_n;
+  const uint32_t total_tiles = (uint32_t)(g.tiles_m * g.tiles_n);
 
   auto panel_a = [&](int64_t m0) __attribute__((always_inline)) {
     const int64_t rows = g.M - m0 < kTile ? g.M - m0 : kTile;
@@ -160,56 +161,15 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_pingpong(GemmArgs
   };
 
   const float scale = output_scale(g);
-  const int64_t ldc = g.ldc;
-  uint16_t* const C = (uint16_t*)g.C;
-  auto store8 = [&](int64_t m, int64_t n, u32x2 x, u32x2 y) __attribute__((always_inline)) {
-    if (m >= g.M) return;
-    uint16_t* p = C + m * ldc + n;
-    if constexpr (kBlk == 16) {
-      if (n + 8 <= g.N) __builtin_nontemporal_store((u32x4){x[0], x[1], y[0], y[1]}, (u32x4*)p);
-      else if (n + 4 <= g.N) __builtin_nontemporal_store(x, (u32x2*)p);
-    } else {
-      if (n + 8 <= g.N) *(u32x4*)p = (u32x4){x[0], x[1], y[0], y[1]};
-      else if (n + 4 <= g.N) *(u32x2*)p = x;
-    }
-  };
-  auto pack_quad = [&](const Acc& a, int q) __attribute__((always_inline)) -> u32x2 {
-    return Pack4<OutT>::run(a[4 * q] * scale, a[4 * q + 1] * scale, a[4 * q + 2] * scale, a[4 * q + 3] * scale);
-  };
-  // Same register-to-element map and lane-group swaps as the single-group kernel's epilogue.
   auto epilogue = [&](int64_t m0, int64_t n0) __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = 0; i < kNbA; ++i) {
-      const int64_t m = m0 + wm * 128 + i * kBlk + rblk;
-      if constexpr (kBlk == 16) {
-#pragma unroll
-        for (int j = 0; j < kNbB; j += 2) {
-          u32x2 x = pack_quad(acc[i][j], 0), y = pack_quad(acc[i][j + 1], 0);
-          u32x2 lo = __builtin_amdgcn_permlane16_swap(x[0], y[0], false, false);
-          u32x2 hi = __builtin_amdgcn_permlane16_swap(x[1], y[1], false, false);
-          const int64_t n = n0 + wn * 64 + (j + (grp & 1)) * 16 + (grp >> 1) * 8;
-          store8(m, n, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < kNbB; ++j) {
-#pragma unroll
-          for (int q = 0; q < 4; q += 2) {
-            u32x2 x = pack_quad(acc[i][j], q), y = pack_quad(acc[i][j], q + 1);
-            u32x2 lo = __builtin_amdgcn_permlane32_swap(x[0], y[0], false, false);
-            u32x2 hi = __builtin_amdgcn_permlane32_swap(x[1], y[1], false, false);
-            const int64_t n = n0 + wn * 64 + j * 32 + (q >> 1) * 16 + grp * 8;
-            store8(m, n, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
-          }
-        }
-      }
-    }
+    store_output_tile<T, OutT, kNbA, kNbB, false>(acc, g, m0, n0, kTile, wm * 128, wn * 64, lane, scale);
   };
 
-  int64_t tile = blockIdx.x;
-  int64_t tile_m, tile_n;
-  tile_coord(tile, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-  __amdgpu_buffer_rsrc_t rsrc_a = panel_a(tile_m * kTile), rsrc_b = panel_b(tile_n * kTile);
+  const uint32_t tiles_m = (uint32_t)g.tiles_m, tiles_n = (uint32_t)g.tiles_n;  // below 2^31 tiles (launcher)
+  uint32_t tile = blockIdx.x;
+  uint32_t tile_m, tile_n;
+  tile_coord_t<uint32_t>(tile, tiles_m, tiles_n, &tile_m, &tile_n);
+  __amdgpu_buffer_rsrc_t rsrc_a = panel_a((int64_t)tile_m * kTile), rsrc_b = panel_b((int64_t)tile_n * kTile);
   open_tile(rsrc_a, rsrc_b);
 
   for (;;) {
@@ -261,13 +221,13 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_pingpong(GemmArgs
     wait_vmcnt<0>();
     phase_barrier();
 
-    const int64_t done_m0 = tile_m * kTile, done_n0 = tile_n * kTile;
+    const int64_t done_m0 = (int64_t)tile_m * kTile, done_n0 = (int64_t)tile_n * kTile;
     tile += gridDim.x;
     const bool more = tile < total_tiles;
     if (more) {
-      tile_coord(tile, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-      rsrc_a = panel_a(tile_m * kTile);
-      rsrc_b = panel_b(tile_n * kTile);
+      tile_coord_t<uint32_t>(tile, tiles_m, tiles_n, &tile_m, &tile_n);
+      rsrc_a = panel_a((int64_t)tile_m * kTile);
+      rsrc_b = panel_b((int64_t)tile_n * kTile);
       open_tile(rsrc_a, rsrc_b);
     }
     epilogue(done_m0, done_n0);
@@ -278,6 +238,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_pingpong(GemmArgs
 template <class T, class OutT>
 int launch(const GemmArgs& g, hipStream_t stream) {
   const int64_t tiles = g.tiles_m * g.tiles_n;
+  if (tiles >= ((int64_t)1 << 31)) return -1;  // the kernel counts tiles in 32 bits
   const int64_t cus = compute_units();
   const int64_t blocks = tiles < cus ? tiles : cus;
   if ((g.K * T::kBytes) % kRowBytes == 0)

@@ -42,13 +42,25 @@
 #include "gemm_launch.h"
 #include "ring_common.h"
 #include "tile_map.h"
+#include "tile_store.h"
 
 #include <type_traits>
+#include <utility>
 
 namespace mi355 {
 namespace {
 
-constexpr int kThreads = 256;
+// Waves of a workgroup form a 2 x kWavesN grid over the tile.
+constexpr int threads_of(int waves_n) { return 128 * waves_n; }
+
+// MFMA position of copy c when n copies are spread evenly over `span` positions from `first`,
+// and the first copy whose position is not before p.
+constexpr int copy_position(int c, int first, int span, int n) { return first + c * span / n; }
+constexpr int first_copy_at(int p, int first, int span, int n) {
+  int c = 0;
+  while (c < n && copy_position(c, first, span, n) < p) ++c;
+  return c;
+}
 
 // kRaggedK: K*elem_bytes is not a multiple of the 128-byte k-step.  Kept out of the common
 // instantiation because selecting the per-lane offset inside the loop puts a dependent VALU
@@ -56,29 +68,37 @@ constexpr int kThreads = 256;
 // kTileT: rows of A and of B per workgroup, 256 or 128.  The 128 variant (64x64 per wave, 80 KiB
 // ring, two workgroups per CU) is for problems with too few 256x256 tiles to occupy the CUs; it
 // moves twice the bytes per flop, so it is copy-bound at about two thirds of the MFMA rate.
-template <class T, class OutT, bool kRaggedK, int kTileT>
-__global__ __launch_bounds__(kThreads, kTileT == 256 ? 1 : 2) void gemm_tn_tile_ring(GemmArgs g) {
+template <class T, class OutT, bool kRaggedK, int kTileT, int kWavesN = 2>
+__global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void gemm_tn_tile_ring(GemmArgs g) {
   constexpr int kTile = kTileT;
   constexpr int kSlotBytes = kTile * kRowBytes;   // one operand, one k-step
-  constexpr int kWaveTile = kTile / 2;            // rows and columns per wave
-  constexpr int kCph = kTile / 32;                // copies (8 rows each) per operand per k-step per wave
+  constexpr int kWaveTileM = kTile / 2;           // rows (of A) per wave
+  constexpr int kWaveTileN = kTile / kWavesN;     // columns (rows of B) per wave
+  constexpr int kWaves = 2 * kWavesN;
+  // One direct-to-LDS instruction moves 16 B per lane: 8 rows of 128 B.  (4 B per lane, 2 rows,
+  // costs an MFMA stream nothing per instruction in isolation, but four times as many copies
+  // through the texture-address unit made the kernel 11 % slower.)
+  constexpr int kCopyRows = 8;
+  constexpr int kCopyBytes = kCopyRows * kRowBytes;
+  constexpr int kCph = kTile / kWaves / kCopyRows;  // copies per operand per k-step per wave
+  constexpr int kPar = 2;                           // copies j and j+kPar share their per-lane swizzle
   __shared__ __attribute__((aligned(1024))) uint8_t ring[kSlots * kSlotBytes];
   typedef Geo<T> G;
   typedef typename G::Frag Frag;
   typedef typename G::Acc Acc;
   constexpr int kBlk = G::kBlk;
-  constexpr int kNb = kWaveTile / kBlk;                 // blocks per wave per dimension
+  constexpr int kNbM = kWaveTileM / kBlk, kNbN = kWaveTileN / kBlk;  // blocks per wave
   constexpr int kSliceChunks = G::kGroups * G::kCpl;    // chunks of a row consumed per slice
   constexpr int kSlices = 8 / kSliceChunks;
   constexpr int kAccLen = kBlk * kBlk / 64;
-  constexpr int kMfmaPerSlice = kNb * kNb;
-  constexpr int kReadsPerSlice = 2 * kNb;               // fragment loads (each kCpl ds_read_b128)
+  constexpr int kMfmaPerSlice = kNbM * kNbN;
+  constexpr int kReadsPerSlice = kNbM + kNbN;               // fragment loads (each kCpl ds_read_b128)
   static_assert(kSlices == 2, "the schedule below assumes two slices per k-step");
 
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & 63u;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const uint32_t wm = wave >> 1, wn = wave & 1u;
+  const uint32_t wm = wave / kWavesN, wn = wave % kWavesN;
 
   const uint32_t lda_b = (uint32_t)(g.lda * T::kBytes), ldb_b = (uint32_t)(g.ldb * T::kBytes);
   const uint32_t k_bytes = (uint32_t)(g.K * T::kBytes);
@@ -86,10 +106,11 @@ __global__ __launch_bounds__(kThreads, kTileT == 256 ? 1 : 2) void gemm_tn_tile_
   // fetched from an out-of-range offset (the hardware returns zeros), see tail_or_oob below.
   const uint32_t k_steps = __builtin_amdgcn_readfirstlane((k_bytes + kRowBytes - 1) / kRowBytes);
   const uint32_t tail_bytes = __builtin_amdgcn_readfirstlane(k_bytes % kRowBytes);
-  const int64_t total_tiles = g.tiles_m * g.tiles_n;
+  const uint32_t tiles_m = (uint32_t)g.tiles_m, tiles_n = (uint32_t)g.tiles_n;
+  const uint32_t total_tiles = tiles_m * tiles_n;  // the launcher keeps items below 2^31
   // Work items are (tile, split) pairs, split-major, so that workgroups running together read the
   // same range of K.  steps is the number of k-steps of one item.
-  const int64_t total_items = total_tiles * g.splits;
+  const uint32_t total_items = total_tiles * (uint32_t)g.splits;
   const uint32_t steps = __builtin_amdgcn_readfirstlane(k_steps / (uint32_t)g.splits);
 
   // Descriptors of the A and B row panels of a tile; rows past the matrix edge are out of range.
@@ -102,61 +123,63 @@ __global__ __launch_bounds__(kThreads, kTileT == 256 ? 1 : 2) void gemm_tn_tile_
     return make_raw_buffer((const uint8_t*)g.B + n0 * (int64_t)ldb_b, (uint32_t)((rows - 1) * ldb_b + k_bytes));
   };
 
-  // Copy geometry: one wave instruction moves 8 rows x 128 B.  Wave w issues copies 8w..8w+7 of
-  // an operand (rows 64w .. 64w+63).  Lane l fills LDS chunk l%8 of row l/8 with the global
-  // chunk (l%8) ^ swizzle(row); swizzle(row) depends only on the copy's parity and l/16, so two
-  // per-lane offsets per operand suffice; copy j adds j*8 rows to them.
-  const uint32_t r8 = lane >> 3, c8 = lane & 7u;
+  // Copy geometry.  Wave w fills rows [w*kTile/4, (w+1)*kTile/4) of a slot, kCopyRows rows per
+  // instruction, the LDS side linear in the lane number.  Lane l therefore fills bytes
+  // sub..sub+n of LDS chunk lchunk of row lrow of the copy's rows, and fetches them from global
+  // chunk lchunk ^ swizzle(row).  swizzle(row) repeats every kPar copies, so kPar per-lane
+  // offsets per operand suffice; copy j adds j*kCopyRows rows to them.
+  const uint32_t lrow = lane >> 3, lchunk = lane & 7u;
   constexpr uint32_t kOutOfRange = 0x80000000u;  // row panels are smaller than 2 GiB (host check)
-  uint32_t voff_a[2], voff_b[2], tail_a[2], tail_b[2];
+  uint32_t voff_a[kPar], voff_b[kPar], tail_a[kRaggedK ? kPar : 1], tail_b[kRaggedK ? kPar : 1];
 #pragma unroll
-  for (int par = 0; par < 2; ++par) {
-    const uint32_t chunk = c8 ^ swizzle(par * 8 + r8);
-    voff_a[par] = (wave * (kCph * 8) + r8) * lda_b + chunk * 16;
-    voff_b[par] = (wave * (kCph * 8) + r8) * ldb_b + chunk * 16;
-    const bool tail_or_oob = tail_bytes != 0 && chunk * 16 >= tail_bytes;
-    tail_a[par] = tail_or_oob ? kOutOfRange : voff_a[par];
-    tail_b[par] = tail_or_oob ? kOutOfRange : voff_b[par];
+  for (int par = 0; par < kPar; ++par) {
+    const uint32_t chunk = lchunk ^ swizzle(par * kCopyRows + lrow);
+    voff_a[par] = (wave * (kCph * kCopyRows) + lrow) * lda_b + chunk * 16;
+    voff_b[par] = (wave * (kCph * kCopyRows) + lrow) * ldb_b + chunk * 16;
+    if constexpr (kRaggedK) {
+      const bool tail_or_oob = tail_bytes != 0 && chunk * 16 >= tail_bytes;
+      tail_a[par] = tail_or_oob ? kOutOfRange : voff_a[par];
+      tail_b[par] = tail_or_oob ? kOutOfRange : voff_b[par];
+    }
   }
-  const uint32_t a_step = __builtin_amdgcn_readfirstlane(8 * lda_b);
-  const uint32_t b_step = __builtin_amdgcn_readfirstlane(8 * ldb_b);
+  const uint32_t a_step = __builtin_amdgcn_readfirstlane(kCopyRows * lda_b);
+  const uint32_t b_step = __builtin_amdgcn_readfirstlane(kCopyRows * ldb_b);
   const uint32_t ring0 = __builtin_amdgcn_readfirstlane(lds_address(ring));
-  const uint32_t dma_wave = ring0 + wave * (kCph * 1024);  // this wave's share of a slot
+  const uint32_t dma_wave = ring0 + wave * (kCph * kCopyBytes);  // this wave's share of a slot
 
-  // Copy j (0..7) of an operand's k-step kt into slot `slot`.  The row part of the address stays
+  // Copy j of an operand's k-step kt into slot `slot`.  The row part of the address stays
   // in the vector offset, the only part the hardware range-checks against the descriptor (rows
   // past the edge of the matrix read zeros); the scalar offset carries the k-step and is kept
   // inside the row by re-reading the item's last k-step for kt past its end (the slot is never used).
   uint32_t step0 = 0;  // first k-step of the current item
-  auto copy_a = [&](__amdgpu_buffer_rsrc_t rsrc, int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
-    const uint32_t kk = step0 + (kt < steps ? kt : steps - 1);
-    const uint32_t voff = kRaggedK && kk == k_steps - 1 ? tail_a[j & 1] : voff_a[j & 1];  // kk is global
-    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff + j * a_step, rsrc, kk * kRowBytes);
+  auto copy_rows = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, uint32_t slot, uint32_t kt, const uint32_t* voff,
+                       const uint32_t* tail, uint32_t step) __attribute__((always_inline)) {
+    constexpr int j = decltype(jc)::value;
+    const uint32_t kk = step0 + (kt < steps ? kt : steps - 1);  // global k-step
+    uint32_t v = voff[j % kPar];
+    if constexpr (kRaggedK) v = kk == k_steps - 1 ? tail[j % kPar] : v;
+    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * kCopyBytes, v + j * step, rsrc, kk * kRowBytes);
   };
-  auto copy_b = [&](__amdgpu_buffer_rsrc_t rsrc, int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
-    const uint32_t kk = step0 + (kt < steps ? kt : steps - 1);
-    const uint32_t voff = kRaggedK && kk == k_steps - 1 ? tail_b[j & 1] : voff_b[j & 1];
-    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff + j * b_step, rsrc, kk * kRowBytes);
+  auto copy_a = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
+    copy_rows(rsrc, jc, slot, kt, voff_a, tail_a, a_step);
+  };
+  auto copy_b = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
+    copy_rows(rsrc, jc, slot, kt, voff_b, tail_b, b_step);
   };
   // Opening copies of a tile: A0 B0 A1 B1 A2 into slots 0..4.
   auto open_tile = [&](__amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb) __attribute__((always_inline)) {
-#pragma unroll
-    for (int j = 0; j < kCph; ++j) copy_a(ra, j, 0, 0);
-#pragma unroll
-    for (int j = 0; j < kCph; ++j) copy_b(rb, j, 1, 0);
-#pragma unroll
-    for (int j = 0; j < kCph; ++j) copy_a(ra, j, 2, 1);
-#pragma unroll
-    for (int j = 0; j < kCph; ++j) copy_b(rb, j, 3, 1);
-#pragma unroll
-    for (int j = 0; j < kCph; ++j) copy_a(ra, j, 4, 2);
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, 0, 0); });
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, 1, 0); });
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, 2, 1); });
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, 3, 1); });
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, 4, 2); });
   };
 
   // Fragment geometry: lane l supplies row l%kBlk of a block; group l/kBlk picks the chunks.
   const uint32_t rblk = lane & (kBlk - 1), grp = lane / kBlk;
   const uint32_t swz = swizzle(rblk);  // block bases are multiples of 16 rows
-  const uint32_t a_lane = (wm * kWaveTile + rblk) * kRowBytes;
-  const uint32_t b_lane = (wn * kWaveTile + rblk) * kRowBytes;
+  const uint32_t a_lane = (wm * kWaveTileM + rblk) * kRowBytes;
+  const uint32_t b_lane = (wn * kWaveTileN + rblk) * kRowBytes;
   // Byte offset inside a row of the e-th chunk this lane reads in slice s.
   auto chunk_off = [&](int s, int e) __attribute__((always_inline)) -> uint32_t {
     return ((uint32_t)(s * kSliceChunks + grp * G::kCpl + e) ^ swz) << 4;
@@ -172,17 +195,17 @@ __global__ __launch_bounds__(kThreads, kTileT == 256 ? 1 : 2) void gemm_tn_tile_
     }
   };
 
-  Acc acc[kNb][kNb];
-  Frag fa[2][kNb], fb[2][kNb];  // [fragment buffer][block]
+  Acc acc[kNbM][kNbN];
+  Frag fa[2][kNbM], fb[2][kNbN];  // [fragment buffer][block]
 
   // Load number q (0..kReadsPerSlice-1) of a slice: B blocks first (every MFMA row needs them all).
   auto read_q = [&](int buf, int q, const uint8_t* a_rows, const uint8_t* b_rows, int s)
       __attribute__((always_inline)) {
-    if (q < kNb) fb[buf][q] = load_frag(b_rows, q, s);
-    else fa[buf][q - kNb] = load_frag(a_rows, q - kNb, s);
+    if (q < kNbN) fb[buf][q] = load_frag(b_rows, q, s);
+    else fa[buf][q - kNbN] = load_frag(a_rows, q - kNbN, s);
   };
   auto mfma_u = [&](int buf, int u) __attribute__((always_inline)) {
-    const int i = u / kNb, j = u % kNb;
+    const int i = u / kNbN, j = u % kNbN;
     // B supplies the MFMA "rows" so each lane ends up with consecutive n of one m.
     // In the 256-wide tile all 256 accumulator registers are live; the in-place form keeps the
     // compiler from rotating them through copies when it allocates the MFMA's result.
@@ -190,100 +213,34 @@ __global__ __launch_bounds__(kThreads, kTileT == 256 ? 1 : 2) void gemm_tn_tile_
     else acc[i][j] = G::mfma(fb[buf][j], fa[buf][i], acc[i][j]);
   };
 
-  // Epilogue of the tile at (m0, n0).  Accumulator register 4q+e of block (i,j) in lane l is C[m][n],
-  //   m = m0 + wm*128 + i*kBlk + l%kBlk,   n = n0 + wn*128 + j*kBlk + q*4*kGroups + 4*(l/kBlk) + e.
-  // Two quads that sit 4 columns apart in neighbouring lane groups are swapped so that each lane
-  // holds 8 consecutive columns.
+  // Stores of the tile at (m0, n0): converted output, or fp32 partials for a split-K item.
   const float scale = output_scale(g);
-  const int64_t ldc = g.ldc;
-  uint16_t* const C = (uint16_t*)g.C;
-  auto store8 = [&](int64_t m, int64_t n, u32x2 x, u32x2 y) __attribute__((always_inline)) {
-    if (m >= g.M) return;
-    uint16_t* p = C + m * ldc + n;
-    // Non-temporal stores keep C out of L2 (it is written once and would evict operand panels).
-    // They only pay when a store instruction covers at least 64 contiguous bytes per row, which
-    // the 16-wide blocks do (two blocks side by side) and the 32-wide blocks do not (32 bytes).
-    if constexpr (kBlk == 16) {
-      if (n + 8 <= g.N) __builtin_nontemporal_store((u32x4){x[0], x[1], y[0], y[1]}, (u32x4*)p);
-      else if (n + 4 <= g.N) __builtin_nontemporal_store(x, (u32x2*)p);
-    } else {
-      if (n + 8 <= g.N) *(u32x4*)p = (u32x4){x[0], x[1], y[0], y[1]};
-      else if (n + 4 <= g.N) *(u32x2*)p = x;
-    }
-  };
-  auto pack_quad = [&](const Acc& a, int q) __attribute__((always_inline)) -> u32x2 {
-    return Pack4<OutT>::run(a[4 * q] * scale, a[4 * q + 1] * scale, a[4 * q + 2] * scale, a[4 * q + 3] * scale);
-  };
-  // Split-K items store the raw fp32 accumulators instead: 4 consecutive columns per register quad.
-  auto store_partial = [&](int64_t m0, int64_t n0, uint32_t split) __attribute__((always_inline)) {
-    float* base = g.partial + (int64_t)split * g.M * g.N;
-#pragma unroll
-    for (int i = 0; i < kNb; ++i) {
-      const int64_t m = m0 + wm * kWaveTile + i * kBlk + rblk;
-      if (m >= g.M) continue;
-#pragma unroll
-      for (int j = 0; j < kNb; ++j) {
-#pragma unroll
-        for (int q = 0; q < kAccLen / 4; ++q) {
-          const int64_t n = n0 + wn * kWaveTile + j * kBlk + q * 4 * G::kGroups + grp * 4;
-          if (n + 4 <= g.N)
-            *(f32x4*)(base + m * g.N + n) = (f32x4){acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-        }
-      }
-    }
-  };
+  constexpr bool kAsmMfma = kTile == 256;  // see mfma_u
   auto epilogue = [&](int64_t m0, int64_t n0) __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = 0; i < kNb; ++i) {
-      const int64_t m = m0 + wm * kWaveTile + i * kBlk + rblk;
-      if constexpr (kBlk == 16) {
-        // lane group g = l/16 holds columns 4g..4g+3 of every 16-wide block.  After swapping the
-        // odd groups of block j with the even groups of block j+1, groups 0,2 hold columns
-        // 0..7 / 8..15 of block j and groups 1,3 the same of block j+1.
-#pragma unroll
-        for (int j = 0; j < kNb; j += 2) {
-          u32x2 x = pack_quad(acc[i][j], 0), y = pack_quad(acc[i][j + 1], 0);
-          u32x2 lo = __builtin_amdgcn_permlane16_swap(x[0], y[0], false, false);
-          u32x2 hi = __builtin_amdgcn_permlane16_swap(x[1], y[1], false, false);
-          const int64_t n = n0 + wn * kWaveTile + (j + (grp & 1)) * 16 + (grp >> 1) * 8;
-          store8(m, n, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
-        }
-      } else {
-        // lane group g = l/32 holds columns 8q+4g..8q+4g+3 (q = 0..3) of every 32-wide block.
-        // After swapping the upper half of quad q with the lower half of quad q+1, group 0 holds
-        // columns 16(q/2)..+7 and group 1 columns 16(q/2)+8..+15.
-#pragma unroll
-        for (int j = 0; j < kNb; ++j) {
-#pragma unroll
-          for (int q = 0; q < 4; q += 2) {
-            u32x2 x = pack_quad(acc[i][j], q), y = pack_quad(acc[i][j], q + 1);
-            u32x2 lo = __builtin_amdgcn_permlane32_swap(x[0], y[0], false, false);
-            u32x2 hi = __builtin_amdgcn_permlane32_swap(x[1], y[1], false, false);
-            const int64_t n = n0 + wn * kWaveTile + j * 32 + (q >> 1) * 16 + grp * 8;
-            store8(m, n, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
-          }
-        }
-      }
-    }
+    store_output_tile<T, OutT, kNbM, kNbN, kAsmMfma>(acc, g, m0, n0, kTile, wm * kWaveTileM, wn * kWaveTileN, lane, scale);
+  };
+  auto store_partial = [&](int64_t m0, int64_t n0, uint32_t split) __attribute__((always_inline)) {
+    store_partial_tile<T, kNbM, kNbN, kAsmMfma>(acc, g, m0, n0, kTile, split, wm * kWaveTileM, wn * kWaveTileN, lane);
   };
 
-  int64_t item = blockIdx.x;
-  int64_t tile_m, tile_n;
-  tile_coord(item % total_tiles, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-  uint32_t split = (uint32_t)(item / total_tiles);
+  uint32_t item = blockIdx.x;
+  uint32_t tile_m, tile_n;
+  tile_coord_t<uint32_t>(item % total_tiles, tiles_m, tiles_n, &tile_m, &tile_n);
+  uint32_t split = item / total_tiles;
   step0 = __builtin_amdgcn_readfirstlane(split * steps);
-  __amdgpu_buffer_rsrc_t rsrc_a = panel_a(tile_m * kTile), rsrc_b = panel_b(tile_n * kTile);
+  __amdgpu_buffer_rsrc_t rsrc_a = panel_a((int64_t)tile_m * kTile), rsrc_b = panel_b((int64_t)tile_n * kTile);
   open_tile(rsrc_a, rsrc_b);
 
   for (;;) {
 #pragma unroll
-    for (int i = 0; i < kNb; ++i)
+    for (int i = 0; i < kNbM; ++i)
 #pragma unroll
-      for (int j = 0; j < kNb; ++j)
+      for (int j = 0; j < kNbN; ++j)
 #pragma unroll
         for (int r = 0; r < kAccLen; ++r) acc[i][j][r] = 0.f;
 
-    wait_vmcnt<3 * kCph>();  // A0 and B0 have landed; A1, B1, A2 may be in flight
+    // A0 and B0 have landed; A1, B1, A2 may be in flight (the counter saturates at 63).
+    wait_vmcnt<(3 * kCph < 63 ? 3 * kCph : 63)>();
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int q = 0; q < kReadsPerSlice; ++q)
@@ -313,35 +270,34 @@ __global__ __launch_bounds__(kThreads, kTileT == 256 ? 1 : 2) void gemm_tn_tile_
       constexpr int kCopySpan = 2 * kMfmaPerSlice - kFirstCopy;          // positions left in the k-step
       static_assert(kCopySpan > 0, "no room for the copies");
       // copy c is issued at position kFirstCopy + c * kCopySpan / kCopies (evenly spread)
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-#pragma unroll
-        for (int u = 0; u < kMfmaPerSlice; ++u) {
-          const int p = s * kMfmaPerSlice + u;
-          if (u < kReadsPerSlice) {
-            if (s == 0) read_q(1, u, a_rows, b_rows, 1);       // slice 1 of this k-step
-            else read_q(0, u, a1_rows, b1_rows, 0);           // slice 0 of the next k-step
-          }
-          if (s == 0 && u == kBarrierAt) {
-            // My reads of this k-step's slots are back; B(t+1) (and A(t+1) before it) have
-            // landed; only this wave's copies of A(t+2) may still be in flight.
-            wait_lgkmcnt0();
-            wait_vmcnt<kCph>();
-            __builtin_amdgcn_s_barrier();
-          }
-          if (p >= kFirstCopy) {
-#pragma unroll
-            for (int c = 0; c < kCopies; ++c) {
-              if (kFirstCopy + c * kCopySpan / kCopies == p) {
-                if (c < kCph) copy_b(rsrc_b, c, slot_a, kt + 2);
-                else copy_a(rsrc_a, c - kCph, slot_b, kt + 3);
-              }
-            }
-          }
-          mfma_u(s, u);
-          MI355_FENCE();
+      constexpr int kMaxCopiesPerGap = (kCopies + kCopySpan - 1) / kCopySpan + 1;
+      static_for<2 * kMfmaPerSlice>([&](auto pc) __attribute__((always_inline)) {
+        constexpr int p = decltype(pc)::value;
+        constexpr int s = p / kMfmaPerSlice, u = p % kMfmaPerSlice;
+        if constexpr (u < kReadsPerSlice) {
+          if constexpr (s == 0) read_q(1, u, a_rows, b_rows, 1);       // slice 1 of this k-step
+          else read_q(0, u, a1_rows, b1_rows, 0);                      // slice 0 of the next k-step
         }
-      }
+        if constexpr (s == 0 && u == kBarrierAt) {
+          // My reads of this k-step's slots are back; B(t+1) (and A(t+1) before it) have
+          // landed; only this wave's copies of A(t+2) may still be in flight.
+          wait_lgkmcnt0();
+          wait_vmcnt<kCph>();
+          __builtin_amdgcn_s_barrier();
+        }
+        if constexpr (p >= kFirstCopy) {
+          constexpr int c0 = first_copy_at(p, kFirstCopy, kCopySpan, kCopies);
+          static_for<kMaxCopiesPerGap>([&](auto ic) __attribute__((always_inline)) {
+            constexpr int c = c0 + decltype(ic)::value;
+            if constexpr (c < kCopies && copy_position(c, kFirstCopy, kCopySpan, kCopies) == p) {
+              if constexpr (c < kCph) copy_b(rsrc_b, std::integral_constant<int, c>{}, slot_a, kt + 2);
+              else copy_a(rsrc_a, std::integral_constant<int, c - kCph>{}, slot_b, kt + 3);
+            }
+          });
+        }
+        mfma_u(s, u);
+        MI355_FENCE();
+      });
       slot_a = slot_a1;
     }
     // The tail copies (past the end of K) must have landed, and every wave must be past its last
@@ -350,16 +306,16 @@ __global__ __launch_bounds__(kThreads, kTileT == 256 ? 1 : 2) void gemm_tn_tile_
     wait_lgkmcnt0();
     __builtin_amdgcn_s_barrier();
 
-    const int64_t done_m0 = tile_m * kTile, done_n0 = tile_n * kTile;
+    const int64_t done_m0 = (int64_t)tile_m * kTile, done_n0 = (int64_t)tile_n * kTile;
     const uint32_t done_split = split;
     item += gridDim.x;
     const bool more = item < total_items;
     if (more) {
-      tile_coord(item % total_tiles, g.tiles_m, g.tiles_n, &tile_m, &tile_n);
-      split = (uint32_t)(item / total_tiles);
+      tile_coord_t<uint32_t>(item % total_tiles, tiles_m, tiles_n, &tile_m, &tile_n);
+      split = item / total_tiles;
       step0 = __builtin_amdgcn_readfirstlane(split * steps);
-      rsrc_a = panel_a(tile_m * kTile);
-      rsrc_b = panel_b(tile_n * kTile);
+      rsrc_a = panel_a((int64_t)tile_m * kTile);
+      rsrc_b = panel_b((int64_t)tile_n * kTile);
       open_tile(rsrc_a, rsrc_b);  // in flight while the finished tile is stored
     }
     if (g.splits > 1) store_partial(done_m0, done_n0, done_split);
@@ -371,12 +327,14 @@ __global__ __launch_bounds__(kThreads, kTileT == 256 ? 1 : 2) void gemm_tn_tile_
 template <class T, class OutT, int kTileT>
 int launch_tile(const GemmArgs& g, hipStream_t stream) {
   const int64_t items = g.tiles_m * g.tiles_n * g.splits;
+  if (items >= ((int64_t)1 << 31)) return -1;  // the kernel counts items in 32 bits
   const int64_t slots = (int64_t)compute_units() * (kTileT == 256 ? 1 : 2);  // resident workgroups (LDS-bound)
   const int64_t blocks = items < slots ? items : slots;
+  constexpr int kWavesN = 2;
   if ((g.K * T::kBytes) % kRowBytes == 0)
-    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, false, kTileT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, g);
+    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, false, kTileT, kWavesN>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
   else
-    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, true, kTileT>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, g);
+    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, true, kTileT, kWavesN>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
   if (hipGetLastError() != hipSuccess) return -1;
   if (g.splits > 1)
     return launch_splitk_reduce(g.partial, g, std::is_same<OutT, BF16>::value ? 0 : 1, stream);

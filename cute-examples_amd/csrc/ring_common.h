@@ -4,6 +4,8 @@
 #include "cdna4_primitives.h"
 
 #include <atomic>
+#include <type_traits>
+#include <utility>
 
 namespace mi355 {
 
@@ -14,6 +16,17 @@ constexpr int kSlots = 5;
 __device__ __forceinline__ uint32_t swizzle(uint32_t row) { return (row >> 1) & 7u; }
 
 #define MI355_FENCE() __builtin_amdgcn_sched_barrier(0)
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, kN - 1>), unrolled at compile time.
+template <int kN, class F, int... kI>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, kI...>) {
+  (f(std::integral_constant<int, kI>{}), ...);
+}
+template <int kN, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl<kN>(f, std::make_integer_sequence<int, kN>{});
+}
+
 
 // Per-dtype MFMA geometry.
 //   kBlk      rows (and columns) of one MFMA block
@@ -56,7 +69,10 @@ template <> struct Geo<E4M3> {
   static __device__ __forceinline__ Acc mfma(Frag x, Frag y, Acc c) {
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, c, 0, 0, 0, 0, 0, 0);
   }
-  static __device__ __forceinline__ void mfma_inplace(Frag x, Frag y, Acc& c) { c = mfma(x, y, c); }
+  // Both operand formats default to e4m3 (cbsz = blgp = 0), as the builtin call above passes.
+  static __device__ __forceinline__ void mfma_inplace(Frag x, Frag y, Acc& c) {
+    asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));
+  }
 };
 
 

@@ -21,26 +21,38 @@ namespace mi355 {
 constexpr int kNumXcd = 8;
 constexpr int kGroupM = 8;
 
-MI355_HD int64_t xcd_contiguous_id(int64_t block, int64_t total) {
+// I is int64_t on the host and uint32_t in kernels (the launchers refuse grids of 2^31 tiles or
+// more), where 64-bit division would cost thousands of cycles per tile.
+template <class I>
+MI355_HD I xcd_contiguous_id_t(I block, I total) {
   // XCD x receives blocks x, x+8, x+16, ...: the first (total % 8) XCDs get one more block.
-  const int64_t per = (total + kNumXcd - 1) / kNumXcd;
-  const int64_t tall = total % kNumXcd == 0 ? kNumXcd : total % kNumXcd;
-  const int64_t xcd = block % kNumXcd;
-  const int64_t local = block / kNumXcd;
+  const I per = (total + kNumXcd - 1) / kNumXcd;
+  const I tall = total % kNumXcd == 0 ? (I)kNumXcd : total % kNumXcd;
+  const I xcd = block % kNumXcd;
+  const I local = block / kNumXcd;
   if (xcd < tall) return xcd * per + local;
   return tall * per + (xcd - tall) * (per - 1) + local;
 }
 
-MI355_HD void tile_coord(int64_t block, int64_t tiles_m, int64_t tiles_n,
-                         int64_t* tile_m, int64_t* tile_n) {
-  const int64_t p = xcd_contiguous_id(block, tiles_m * tiles_n);
-  const int64_t band_size = (int64_t)kGroupM * tiles_n;
-  const int64_t band = p / band_size;
-  const int64_t in_band = p % band_size;
-  const int64_t first_m = band * kGroupM;
-  const int64_t rows = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
+template <class I>
+MI355_HD void tile_coord_t(I block, I tiles_m, I tiles_n, I* tile_m, I* tile_n) {
+  const I p = xcd_contiguous_id_t<I>(block, tiles_m * tiles_n);
+  const I band_size = (I)kGroupM * tiles_n;
+  const I band = p / band_size;
+  const I in_band = p % band_size;
+  const I first_m = band * kGroupM;
+  const I rows = tiles_m - first_m < (I)kGroupM ? tiles_m - first_m : (I)kGroupM;
   *tile_m = first_m + in_band % rows;
   *tile_n = in_band / rows;
+}
+
+MI355_HD int64_t xcd_contiguous_id(int64_t block, int64_t total) {
+  return xcd_contiguous_id_t<int64_t>(block, total);
+}
+
+MI355_HD void tile_coord(int64_t block, int64_t tiles_m, int64_t tiles_n,
+                         int64_t* tile_m, int64_t* tile_n) {
+  tile_coord_t<int64_t>(block, tiles_m, tiles_n, tile_m, tile_n);
 }
 
 }  // namespace mi355

@@ -1,0 +1,141 @@
+// Writing a finished tile: accumulators -> bf16/fp16 rows of C, or -> fp32 rows of a split-K plane.
+// Shared by the ring-buffered tile kernels; each wave stores the kNbM x kNbN MFMA blocks it owns.
+//
+// Register-to-element map (MFMA with B as the "row" operand): accumulator register 4q+e of block
+// (i, j) in lane l is the output element
+//   m = wave_row + i*kBlk + l%kBlk,   n = wave_col + j*kBlk + q*4*kGroups + 4*(l/kBlk) + e.
+//
+// All stores go through a buffer descriptor of the tile itself: offsets are 32 bits, the
+// descriptor's size cuts off rows past M, and a lane whose columns lie past N gets an
+// out-of-range offset, so the hardware drops what must not be written and the code has no
+// per-store branch or 64-bit address arithmetic.  Row block i goes into the scalar offset, the
+// column into the instruction's immediate.  Few live registers matter here as much as few
+// instructions: a spill reload between two stores waits on the memory counter, i.e. for every
+// store issued before it, and that serialisation once made this phase four times longer.
+#pragma once
+#include "gemm_launch.h"
+#include "ring_common.h"
+
+namespace mi355 {
+
+constexpr uint32_t kStoreOutOfRange = 0x80000000u;  // tiles of C span less than 2 GiB (host check)
+
+// One accumulator value.  kAsmRead: the kernel's MFMAs are inline assembly on accumulation
+// registers, and so is the read; it then stays at this point of the program, and the register
+// allocator does not move whole accumulator tiles into VGPRs (and from there into scratch) when
+// the k loop ends.
+template <bool kAsmRead, class Acc>
+__device__ __forceinline__ float acc_value(const Acc& a, int e) {
+  if constexpr (kAsmRead) {
+    float r;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(r) : "a"(a[e]));
+    return r;
+  } else {
+    return a[e];
+  }
+}
+
+// The wave's part of the output tile at (m0, n0), tile_edge rows and columns at most.
+// wave_row / wave_col: first row / column of the wave inside the tile.
+template <class T, class OutT, int kNbM, int kNbN, bool kAsmRead>
+__device__ __forceinline__ void store_output_tile(const typename Geo<T>::Acc (&acc)[kNbM][kNbN], const GemmArgs& g,
+                                                  int64_t m0, int64_t n0, int tile_edge, uint32_t wave_row,
+                                                  uint32_t wave_col, uint32_t lane, float scale) {
+  typedef Geo<T> G;
+  typedef typename G::Acc Acc;
+  constexpr int kBlk = G::kBlk;
+  // Non-temporal stores (aux bit 1) keep C out of L2: it is written once and would evict operand
+  // panels.  They only pay when a store instruction covers at least 64 contiguous bytes per row,
+  // which the 16-wide blocks do (two blocks side by side) and the 32-wide blocks do not (32 bytes).
+  constexpr int kAux = kBlk == 16 ? 2 : 0;
+  const uint32_t rblk = lane & (kBlk - 1), grp = lane / kBlk;
+  const int64_t rows = g.M - m0 < tile_edge ? g.M - m0 : tile_edge;
+  const uint32_t cols = (uint32_t)(g.N - n0 < tile_edge ? g.N - n0 : tile_edge);
+  const uint32_t ldc_b = (uint32_t)g.ldc * 2;
+  const __amdgpu_buffer_rsrc_t rc =
+      make_raw_buffer((const uint16_t*)g.C + m0 * g.ldc + n0, (uint32_t)(((rows - 1) * g.ldc + cols) * 2));
+  // After the lane-group swaps below every lane holds 8 consecutive columns, starting here.
+  const uint32_t lane_col = kBlk == 16 ? (grp & 1) * 16 + (grp >> 1) * 8 : grp * 8;
+  const uint32_t col0 = wave_col + lane_col;
+  const uint32_t v0 = (wave_row + rblk) * ldc_b + col0 * 2;
+  const uint32_t block_step = __builtin_amdgcn_readfirstlane(kBlk * ldc_b);
+  const bool whole = cols == (uint32_t)tile_edge;
+
+  auto pack_quad = [&](const Acc& a, int q) __attribute__((always_inline)) -> u32x2 {
+    return Pack4<OutT>::run(acc_value<kAsmRead>(a, 4 * q) * scale, acc_value<kAsmRead>(a, 4 * q + 1) * scale,
+                            acc_value<kAsmRead>(a, 4 * q + 2) * scale, acc_value<kAsmRead>(a, 4 * q + 3) * scale);
+  };
+  // x = the lane's first four outputs, y = the last four, `col` columns right of col0 in row block i.
+  auto emit = [&](auto ic, auto colc, u32x2 x, u32x2 y) __attribute__((always_inline)) {
+    constexpr int i = decltype(ic)::value, col = decltype(colc)::value;
+    if (whole) {
+      __builtin_amdgcn_raw_buffer_store_b128((u32x4){x[0], x[1], y[0], y[1]}, rc, v0 + col * 2, i * block_step, kAux);
+    } else {
+      // N is a multiple of 4 (host check), so each half of the 8 columns is in or out as a whole.
+      const uint32_t vx = col0 + col + 4 <= cols ? v0 + col * 2 : kStoreOutOfRange;
+      const uint32_t vy = col0 + col + 8 <= cols ? v0 + col * 2 + 8 : kStoreOutOfRange;
+      __builtin_amdgcn_raw_buffer_store_b64(x, rc, vx, i * block_step, 0);
+      __builtin_amdgcn_raw_buffer_store_b64(y, rc, vy, i * block_step, 0);
+    }
+  };
+  static_for<kNbM>([&](auto ic) __attribute__((always_inline)) {
+    constexpr int i = decltype(ic)::value;
+    if constexpr (kBlk == 16) {
+      // Lane group g = l/16 holds columns 4g..4g+3 of every 16-wide block.  After swapping the
+      // odd groups of block j with the even groups of block j+1, groups 0,2 hold columns
+      // 0..7 / 8..15 of block j and groups 1,3 the same of block j+1.
+      static_for<kNbN / 2>([&](auto jc) __attribute__((always_inline)) {
+        constexpr int j = 2 * decltype(jc)::value;
+        u32x2 x = pack_quad(acc[i][j], 0), y = pack_quad(acc[i][j + 1], 0);
+        u32x2 lo = __builtin_amdgcn_permlane16_swap(x[0], y[0], false, false);
+        u32x2 hi = __builtin_amdgcn_permlane16_swap(x[1], y[1], false, false);
+        emit(ic, std::integral_constant<int, j * 16>{}, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
+      });
+    } else {
+      // Lane group g = l/32 holds columns 8q+4g..8q+4g+3 (q = 0..3) of every 32-wide block.
+      // After swapping the upper half of quad q with the lower half of quad q+1, group 0 holds
+      // columns 16(q/2)..+7 and group 1 columns 16(q/2)+8..+15.
+      static_for<kNbN * 2>([&](auto jq) __attribute__((always_inline)) {
+        constexpr int j = decltype(jq)::value / 2, q = 2 * (decltype(jq)::value % 2);
+        u32x2 x = pack_quad(acc[i][j], q), y = pack_quad(acc[i][j], q + 1);
+        u32x2 lo = __builtin_amdgcn_permlane32_swap(x[0], y[0], false, false);
+        u32x2 hi = __builtin_amdgcn_permlane32_swap(x[1], y[1], false, false);
+        emit(ic, std::integral_constant<int, j * 32 + (q >> 1) * 16>{}, (u32x2){lo[0], hi[0]},
+             (u32x2){lo[1], hi[1]});
+      });
+    }
+  });
+}
+
+// The same part of the tile as raw fp32 accumulators into plane `split` (M x N floats, row stride
+// N) of the split-K workspace: 4 consecutive columns per register quad, no lane exchange.
+template <class T, int kNbM, int kNbN, bool kAsmRead>
+__device__ __forceinline__ void store_partial_tile(const typename Geo<T>::Acc (&acc)[kNbM][kNbN], const GemmArgs& g,
+                                                   int64_t m0, int64_t n0, int tile_edge, uint32_t split,
+                                                   uint32_t wave_row, uint32_t wave_col, uint32_t lane) {
+  typedef Geo<T> G;
+  constexpr int kBlk = G::kBlk;
+  constexpr int kQuads = kBlk * kBlk / 64 / 4;
+  const uint32_t rblk = lane & (kBlk - 1), grp = lane / kBlk;
+  const int64_t rows = g.M - m0 < tile_edge ? g.M - m0 : tile_edge;
+  const uint32_t cols = (uint32_t)(g.N - n0 < tile_edge ? g.N - n0 : tile_edge);
+  const uint32_t ldp_b = (uint32_t)g.N * 4;
+  const __amdgpu_buffer_rsrc_t rp = make_raw_buffer(g.partial + ((int64_t)split * g.M + m0) * g.N + n0,
+                                                    (uint32_t)(((rows - 1) * g.N + cols) * 4));
+  const uint32_t col0 = wave_col + grp * 4;
+  const uint32_t v0 = (wave_row + rblk) * ldp_b + col0 * 4;
+  const uint32_t block_step = __builtin_amdgcn_readfirstlane(kBlk * ldp_b);
+  static_for<kNbM>([&](auto ic) __attribute__((always_inline)) {
+    constexpr int i = decltype(ic)::value;
+    static_for<kNbN * kQuads>([&](auto jq) __attribute__((always_inline)) {
+      constexpr int j = decltype(jq)::value / kQuads, q = decltype(jq)::value % kQuads;
+      constexpr int col = j * kBlk + q * 4 * G::kGroups;
+      const uint32_t v = col0 + col + 4 <= cols ? v0 + col * 4 : kStoreOutOfRange;
+      const f32x4 quad = {acc_value<kAsmRead>(acc[i][j], 4 * q), acc_value<kAsmRead>(acc[i][j], 4 * q + 1),
+                          acc_value<kAsmRead>(acc[i][j], 4 * q + 2), acc_value<kAsmRead>(acc[i][j], 4 * q + 3)};
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, quad), rp, v, i * block_step, 0);
+    });
+  });
+}
+
+}  // namespace mi355
