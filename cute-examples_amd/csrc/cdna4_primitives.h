@@ -50,6 +50,20 @@ __device__ __forceinline__ void dma_16B_to_lds(uint32_t lds_base, uint32_t voffs
       : "memory");
 }
 
+// The same copy with the LDS base given as a scalar register plus a compile-time constant, folded
+// into the one instruction that writes M0 (it also writes SCC).
+template <uint32_t kLdsAdd>
+__device__ __forceinline__ void dma_16B_to_lds_at(uint32_t lds_base, uint32_t voffset,
+                                                  __amdgpu_buffer_rsrc_t rsrc, uint32_t soffset) {
+  asm volatile(
+      "s_add_u32 m0, %0, %4\n\t"
+      "buffer_load_dwordx4 %1, %2, %3 offen lds"
+      :
+      : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(voffset), "s"(rsrc),
+        "s"(__builtin_amdgcn_readfirstlane(soffset)), "n"(kLdsAdd)
+      : "memory", "scc");
+}
+
 // Same copy through the compiler's own intrinsic: the compiler then sets M0, tracks the copy in
 // vmcnt against reads of the destination LDS object, and can schedule it like any VMEM load.
 // imm is added to both the buffer offset and the LDS address.

@@ -147,32 +147,38 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   const uint32_t ring0 = __builtin_amdgcn_readfirstlane(lds_address(ring));
   const uint32_t dma_wave = ring0 + wave * (kCph * kCopyBytes);  // this wave's share of a slot
 
-  // Copy j of an operand's k-step kt into slot `slot`.  The row part of the address stays
-  // in the vector offset, the only part the hardware range-checks against the descriptor (rows
-  // past the edge of the matrix read zeros); the scalar offset carries the k-step and is kept
-  // inside the row by re-reading the item's last k-step for kt past its end (the slot is never used).
-  uint32_t step0 = 0;  // first k-step of the current item
-  auto copy_rows = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, uint32_t slot, uint32_t kt, const uint32_t* voff,
+  // Copy j of an operand's k-step into slot `slot`; soff is the k-step's byte offset inside a row.
+  // The row part of the address stays in the vector offset, the only part the hardware
+  // range-checks against the descriptor (rows past the edge of the matrix read zeros); the scalar
+  // offset carries the k-step.  Past the end of an item's K range the copies re-read its last
+  // k-step, into a slot nobody reads, so the loop body stays branch-free.
+  const uint32_t soff_tail = (k_steps - 1) * kRowBytes;  // the k-step that may be ragged
+  auto copy_rows = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, auto slotc, uint32_t soff, const uint32_t* voff,
                        const uint32_t* tail, uint32_t step) __attribute__((always_inline)) {
     constexpr int j = decltype(jc)::value;
-    const uint32_t kk = step0 + (kt < steps ? kt : steps - 1);  // global k-step
+    constexpr uint32_t slot = decltype(slotc)::value;
     uint32_t v = voff[j % kPar];
-    if constexpr (kRaggedK) v = kk == k_steps - 1 ? tail[j % kPar] : v;
-    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * kCopyBytes, v + j * step, rsrc, kk * kRowBytes);
+    if constexpr (kRaggedK) v = soff == soff_tail ? tail[j % kPar] : v;
+    dma_16B_to_lds_at<slot * kSlotBytes + j * kCopyBytes>(dma_wave, v + j * step, rsrc, soff);
   };
-  auto copy_a = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
-    copy_rows(rsrc, jc, slot, kt, voff_a, tail_a, a_step);
+  auto copy_a = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, auto slotc, uint32_t soff) __attribute__((always_inline)) {
+    copy_rows(rsrc, jc, slotc, soff, voff_a, tail_a, a_step);
   };
-  auto copy_b = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
-    copy_rows(rsrc, jc, slot, kt, voff_b, tail_b, b_step);
+  auto copy_b = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, auto slotc, uint32_t soff) __attribute__((always_inline)) {
+    copy_rows(rsrc, jc, slotc, soff, voff_b, tail_b, b_step);
+  };
+  // Byte offset of k-step kt of the item that starts at global k-step step0, clamped to its last.
+  auto soff_of = [&](uint32_t step0, uint32_t kt) __attribute__((always_inline)) -> uint32_t {
+    return __builtin_amdgcn_readfirstlane((step0 + (kt < steps ? kt : steps - 1)) * kRowBytes);
   };
   // Opening copies of a tile: A0 B0 A1 B1 A2 into slots 0..4.
-  auto open_tile = [&](__amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb) __attribute__((always_inline)) {
-    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, 0, 0); });
-    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, 1, 0); });
-    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, 2, 1); });
-    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, 3, 1); });
-    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, 4, 2); });
+  auto open_tile = [&](__amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb, uint32_t step0) __attribute__((always_inline)) {
+    const uint32_t s0 = soff_of(step0, 0), s1 = soff_of(step0, 1), s2 = soff_of(step0, 2);
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, std::integral_constant<uint32_t, 0>{}, s0); });
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, std::integral_constant<uint32_t, 1>{}, s0); });
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, std::integral_constant<uint32_t, 2>{}, s1); });
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, std::integral_constant<uint32_t, 3>{}, s1); });
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, std::integral_constant<uint32_t, 4>{}, s2); });
   };
 
   // Fragment geometry: lane l supplies row l%kBlk of a block; group l/kBlk picks the chunks.
@@ -227,9 +233,9 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   uint32_t tile_m, tile_n;
   tile_coord_t<uint32_t>(item % total_tiles, tiles_m, tiles_n, &tile_m, &tile_n);
   uint32_t split = item / total_tiles;
-  step0 = __builtin_amdgcn_readfirstlane(split * steps);
+  uint32_t step0 = __builtin_amdgcn_readfirstlane(split * steps);  // first k-step of the current item
   __amdgpu_buffer_rsrc_t rsrc_a = panel_a((int64_t)tile_m * kTile), rsrc_b = panel_b((int64_t)tile_n * kTile);
-  open_tile(rsrc_a, rsrc_b);
+  open_tile(rsrc_a, rsrc_b, step0);
 
   for (;;) {
 #pragma unroll
@@ -246,11 +252,18 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     for (int q = 0; q < kReadsPerSlice; ++q)
       read_q(0, q, ring + a_lane, ring + kSlotBytes + b_lane, 0);
 
-    uint32_t slot_a = 0;  // slot of A(t); B(t), A(t+1), B(t+1) follow in slot_a+1..+3 (mod 5)
-    for (uint32_t kt = 0; kt < steps; ++kt) {
-      const uint32_t slot_b = slot_a + 1 >= kSlots ? slot_a + 1 - kSlots : slot_a + 1;
-      const uint32_t slot_a1 = slot_a + 2 >= kSlots ? slot_a + 2 - kSlots : slot_a + 2;
-      const uint32_t slot_b1 = slot_a + 3 >= kSlots ? slot_a + 3 - kSlots : slot_a + 3;
+    // The slot of A(t) walks 0, 2, 4, 1, 3 and repeats, so the loop is unrolled over five phases in
+    // which every slot number, and with it every LDS offset, is a compile-time constant.
+    // Row offsets of the operand k-steps the loop copies next, B(t+2) and A(t+3).
+    const uint32_t soff_last = soff_of(step0, steps - 1);
+    uint32_t soff_b = soff_of(step0, 2), soff_a = soff_of(step0, 3);
+    uint32_t kt = 0;
+    bool last = false;
+    for (;;) {
+    static_for<kSlots>([&](auto phase) __attribute__((always_inline)) {
+      if (last) return;
+      constexpr uint32_t slot_a = (2 * decltype(phase)::value) % kSlots;
+      constexpr uint32_t slot_b = (slot_a + 1) % kSlots, slot_a1 = (slot_a + 2) % kSlots, slot_b1 = (slot_a + 3) % kSlots;
       const uint8_t* a_rows = ring + slot_a * kSlotBytes + a_lane;
       const uint8_t* b_rows = ring + slot_b * kSlotBytes + b_lane;
       const uint8_t* a1_rows = ring + slot_a1 * kSlotBytes + a_lane;
@@ -290,15 +303,22 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
           static_for<kMaxCopiesPerGap>([&](auto ic) __attribute__((always_inline)) {
             constexpr int c = c0 + decltype(ic)::value;
             if constexpr (c < kCopies && copy_position(c, kFirstCopy, kCopySpan, kCopies) == p) {
-              if constexpr (c < kCph) copy_b(rsrc_b, std::integral_constant<int, c>{}, slot_a, kt + 2);
-              else copy_a(rsrc_a, std::integral_constant<int, c - kCph>{}, slot_b, kt + 3);
+              if constexpr (c < kCph)
+                copy_b(rsrc_b, std::integral_constant<int, c>{}, std::integral_constant<uint32_t, slot_a>{}, soff_b);
+              else
+                copy_a(rsrc_a, std::integral_constant<int, c - kCph>{}, std::integral_constant<uint32_t, slot_b>{}, soff_a);
             }
           });
         }
         mfma_u(s, u);
         MI355_FENCE();
       });
-      slot_a = slot_a1;
+      soff_b = soff_b + kRowBytes < soff_last ? soff_b + kRowBytes : soff_last;
+      soff_a = soff_a + kRowBytes < soff_last ? soff_a + kRowBytes : soff_last;
+      ++kt;
+      last = kt == steps;
+    });
+    if (last) break;
     }
     // The tail copies (past the end of K) must have landed, and every wave must be past its last
     // LDS read, before the ring is refilled for the next tile.
@@ -316,7 +336,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
       step0 = __builtin_amdgcn_readfirstlane(split * steps);
       rsrc_a = panel_a((int64_t)tile_m * kTile);
       rsrc_b = panel_b((int64_t)tile_n * kTile);
-      open_tile(rsrc_a, rsrc_b);  // in flight while the finished tile is stored
+      open_tile(rsrc_a, rsrc_b, step0);  // in flight while the finished tile is stored
     }
     if (g.splits > 1) store_partial(done_m0, done_n0, done_split);
     else epilogue(done_m0, done_n0);

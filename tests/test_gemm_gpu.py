@@ -26,13 +26,15 @@ def run_abi(abi, A, B, variant=ac.AUTO, scale=1.0, out_dtype=None, ldc=None):
     """NaN-prefilled C (gemm_test.py:28), one call through the C ABI, result on the CPU."""
     M, N = A.shape[0], B.shape[0]
     out_dtype = out_dtype or out_dtype_of(A.dtype)
-    Cfull = torch.full((M, ldc or N), float("nan"), dtype=out_dtype, device="cuda")
-    C = Cfull[:, :N]
+    guard = 8  # rows after the last one: the kernels clip rows in hardware, so watch what lies behind them
+    Cfull = torch.full((M + guard, ldc or N), float("nan"), dtype=out_dtype, device="cuda")
+    C = Cfull[:M, :N]
     rc = ac.gemm_tn(abi, A.cuda(), B.cuda(), C, scale, variant)
     assert rc == 0, abi.mi355_gemm_strerror(rc)
     torch.cuda.synchronize()
+    assert torch.isnan(Cfull[M:].float()).all(), "wrote behind the M rows of C"
     if ldc:
-        assert torch.isnan(Cfull[:, N:].float()).all(), "wrote outside the N columns of C"
+        assert torch.isnan(Cfull[:M, N:].float()).all(), "wrote outside the N columns of C"
     return C.cpu()
 
 
