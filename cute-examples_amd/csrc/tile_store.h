@@ -20,19 +20,28 @@ namespace mi355 {
 
 constexpr uint32_t kStoreOutOfRange = 0x80000000u;  // tiles of C span less than 2 GiB (host check)
 
-// One accumulator value.  kAsmRead: the kernel's MFMAs are inline assembly on accumulation
-// registers, and so is the read; it then stays at this point of the program, and the register
-// allocator does not move whole accumulator tiles into VGPRs (and from there into scratch) when
-// the k loop ends.
-template <bool kAsmRead, class Acc>
-__device__ __forceinline__ float acc_value(const Acc& a, int e) {
-  if constexpr (kAsmRead) {
-    float r;
-    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(r) : "a"(a[e]));
-    return r;
-  } else {
-    return a[e];
-  }
+// A copy of one accumulator block to read element by element.  kPinned: the kernel's MFMAs are inline
+// assembly on accumulation registers; the empty statement here keeps the block in those registers up
+// to this point of the program, so the register allocator moves it to VGPRs here, block by block,
+// and not all 256 registers at once when the k loop ends (which would spill).  The reads
+// themselves stay ordinary compiler-generated moves: the compiler then also keeps them clear of the
+// data registers of stores still being issued, which hand-placed reads once overwrote.
+// A 16-byte buffer store followed by idle cycles.  The store reads its four data registers a few
+// cycles after it issues; the instructions that refill them for the next store come right behind
+// it, and with only the compiler's two wait states in between (as s_nop) a few lanes of the first
+// register were seen to pick up the new value.  Eight idle cycles per store are below measurement.
+__device__ __forceinline__ void store_16B_guarded(u32x4 data, __amdgpu_buffer_rsrc_t rsrc, uint32_t voffset,
+                                                  uint32_t soffset, int aux_nt) {
+  if (aux_nt) __builtin_amdgcn_raw_buffer_store_b128(data, rsrc, voffset, soffset, 2);
+  else __builtin_amdgcn_raw_buffer_store_b128(data, rsrc, voffset, soffset, 0);
+  asm volatile("s_nop 7");
+}
+
+template <bool kPinned, class Acc>
+__device__ __forceinline__ Acc acc_block(const Acc& a) {
+  Acc t = a;
+  if constexpr (kPinned) asm volatile("" : "+a"(t));
+  return t;
 }
 
 // The wave's part of the output tile at (m0, n0), tile_edge rows and columns at most.
@@ -59,52 +68,58 @@ __device__ __forceinline__ void store_output_tile(const typename Geo<T>::Acc (&a
   const uint32_t col0 = wave_col + lane_col;
   const uint32_t v0 = (wave_row + rblk) * ldc_b + col0 * 2;
   const uint32_t block_step = __builtin_amdgcn_readfirstlane(kBlk * ldc_b);
-  const bool whole = cols == (uint32_t)tile_edge;
 
   auto pack_quad = [&](const Acc& a, int q) __attribute__((always_inline)) -> u32x2 {
-    return Pack4<OutT>::run(acc_value<kAsmRead>(a, 4 * q) * scale, acc_value<kAsmRead>(a, 4 * q + 1) * scale,
-                            acc_value<kAsmRead>(a, 4 * q + 2) * scale, acc_value<kAsmRead>(a, 4 * q + 3) * scale);
+    return Pack4<OutT>::run(a[4 * q] * scale, a[4 * q + 1] * scale, a[4 * q + 2] * scale, a[4 * q + 3] * scale);
   };
-  // x = the lane's first four outputs, y = the last four, `col` columns right of col0 in row block i.
-  auto emit = [&](auto ic, auto colc, u32x2 x, u32x2 y) __attribute__((always_inline)) {
-    constexpr int i = decltype(ic)::value, col = decltype(colc)::value;
-    if (whole) {
-      __builtin_amdgcn_raw_buffer_store_b128((u32x4){x[0], x[1], y[0], y[1]}, rc, v0 + col * 2, i * block_step, kAux);
-    } else {
-      // N is a multiple of 4 (host check), so each half of the 8 columns is in or out as a whole.
+  // emit(i, col, x, y): x = the lane's first four outputs, y = the last four, `col` columns right of
+  // col0 in row block i (both compile-time values).
+  auto convert = [&](auto&& emit) __attribute__((always_inline)) {
+    static_for<kNbM>([&](auto ic) __attribute__((always_inline)) {
+      constexpr int i = decltype(ic)::value;
+      if constexpr (kBlk == 16) {
+        // Lane group g = l/16 holds columns 4g..4g+3 of every 16-wide block.  After swapping the
+        // odd groups of block j with the even groups of block j+1, groups 0,2 hold columns
+        // 0..7 / 8..15 of block j and groups 1,3 the same of block j+1.
+        static_for<kNbN / 2>([&](auto jc) __attribute__((always_inline)) {
+          constexpr int j = 2 * decltype(jc)::value;
+          const Acc c0 = acc_block<kAsmRead>(acc[i][j]), c1 = acc_block<kAsmRead>(acc[i][j + 1]);
+          u32x2 x = pack_quad(c0, 0), y = pack_quad(c1, 0);
+          u32x2 lo = __builtin_amdgcn_permlane16_swap(x[0], y[0], false, false);
+          u32x2 hi = __builtin_amdgcn_permlane16_swap(x[1], y[1], false, false);
+          emit(ic, std::integral_constant<int, j * 16>{}, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
+        });
+      } else {
+        // Lane group g = l/32 holds columns 8q+4g..8q+4g+3 (q = 0..3) of every 32-wide block.
+        // After swapping the upper half of quad q with the lower half of quad q+1, group 0 holds
+        // columns 16(q/2)..+7 and group 1 columns 16(q/2)+8..+15.
+        static_for<kNbN * 2>([&](auto jq) __attribute__((always_inline)) {
+          constexpr int j = decltype(jq)::value / 2, q = 2 * (decltype(jq)::value % 2);
+          const Acc c = acc_block<kAsmRead>(acc[i][j]);
+          u32x2 x = pack_quad(c, q), y = pack_quad(c, q + 1);
+          u32x2 lo = __builtin_amdgcn_permlane32_swap(x[0], y[0], false, false);
+          u32x2 hi = __builtin_amdgcn_permlane32_swap(x[1], y[1], false, false);
+          emit(ic, std::integral_constant<int, j * 32 + (q >> 1) * 16>{}, (u32x2){lo[0], hi[0]},
+               (u32x2){lo[1], hi[1]});
+        });
+      }
+    });
+  };
+  if (cols == (uint32_t)tile_edge) {
+    convert([&](auto ic, auto colc, u32x2 x, u32x2 y) __attribute__((always_inline)) {
+      constexpr int i = decltype(ic)::value, col = decltype(colc)::value;
+      store_16B_guarded((u32x4){x[0], x[1], y[0], y[1]}, rc, v0 + col * 2, i * block_step, kAux);
+    });
+  } else {
+    // N is a multiple of 4 (host check), so each half of the 8 columns is in or out as a whole.
+    convert([&](auto ic, auto colc, u32x2 x, u32x2 y) __attribute__((always_inline)) {
+      constexpr int i = decltype(ic)::value, col = decltype(colc)::value;
       const uint32_t vx = col0 + col + 4 <= cols ? v0 + col * 2 : kStoreOutOfRange;
       const uint32_t vy = col0 + col + 8 <= cols ? v0 + col * 2 + 8 : kStoreOutOfRange;
       __builtin_amdgcn_raw_buffer_store_b64(x, rc, vx, i * block_step, 0);
       __builtin_amdgcn_raw_buffer_store_b64(y, rc, vy, i * block_step, 0);
-    }
-  };
-  static_for<kNbM>([&](auto ic) __attribute__((always_inline)) {
-    constexpr int i = decltype(ic)::value;
-    if constexpr (kBlk == 16) {
-      // Lane group g = l/16 holds columns 4g..4g+3 of every 16-wide block.  After swapping the
-      // odd groups of block j with the even groups of block j+1, groups 0,2 hold columns
-      // 0..7 / 8..15 of block j and groups 1,3 the same of block j+1.
-      static_for<kNbN / 2>([&](auto jc) __attribute__((always_inline)) {
-        constexpr int j = 2 * decltype(jc)::value;
-        u32x2 x = pack_quad(acc[i][j], 0), y = pack_quad(acc[i][j + 1], 0);
-        u32x2 lo = __builtin_amdgcn_permlane16_swap(x[0], y[0], false, false);
-        u32x2 hi = __builtin_amdgcn_permlane16_swap(x[1], y[1], false, false);
-        emit(ic, std::integral_constant<int, j * 16>{}, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
-      });
-    } else {
-      // Lane group g = l/32 holds columns 8q+4g..8q+4g+3 (q = 0..3) of every 32-wide block.
-      // After swapping the upper half of quad q with the lower half of quad q+1, group 0 holds
-      // columns 16(q/2)..+7 and group 1 columns 16(q/2)+8..+15.
-      static_for<kNbN * 2>([&](auto jq) __attribute__((always_inline)) {
-        constexpr int j = decltype(jq)::value / 2, q = 2 * (decltype(jq)::value % 2);
-        u32x2 x = pack_quad(acc[i][j], q), y = pack_quad(acc[i][j], q + 1);
-        u32x2 lo = __builtin_amdgcn_permlane32_swap(x[0], y[0], false, false);
-        u32x2 hi = __builtin_amdgcn_permlane32_swap(x[1], y[1], false, false);
-        emit(ic, std::integral_constant<int, j * 32 + (q >> 1) * 16>{}, (u32x2){lo[0], hi[0]},
-             (u32x2){lo[1], hi[1]});
-      });
-    }
-  });
+    });
+  }
 }
 
 // The same part of the tile as raw fp32 accumulators into plane `split` (M x N floats, row stride
@@ -131,9 +146,9 @@ __device__ __forceinline__ void store_partial_tile(const typename Geo<T>::Acc (&
       constexpr int j = decltype(jq)::value / kQuads, q = decltype(jq)::value % kQuads;
       constexpr int col = j * kBlk + q * 4 * G::kGroups;
       const uint32_t v = col0 + col + 4 <= cols ? v0 + col * 4 : kStoreOutOfRange;
-      const f32x4 quad = {acc_value<kAsmRead>(acc[i][j], 4 * q), acc_value<kAsmRead>(acc[i][j], 4 * q + 1),
-                          acc_value<kAsmRead>(acc[i][j], 4 * q + 2), acc_value<kAsmRead>(acc[i][j], 4 * q + 3)};
-      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, quad), rp, v, i * block_step, 0);
+      const typename G::Acc c = acc_block<kAsmRead>(acc[i][j]);
+      const f32x4 quad = {c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
+      store_16B_guarded(__builtin_bit_cast(u32x4, quad), rp, v, i * block_step, 0);
     });
   });
 }

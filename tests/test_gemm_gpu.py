@@ -245,6 +245,31 @@ def test_config5_fp8_8192_full_size(abi, variant):
     _sampled_rows_check(C.cpu(), A.cpu(), B.cpu(), scale, 3e-2)
 
 
+@pytest.mark.parametrize("variant", TILED)
+@pytest.mark.parametrize("dt,M,N,K", [(torch.bfloat16, 4352, 4352, 1024), (torch.float16, 4352, 4096, 1032),
+                                      (torch.float8_e4m3fn, 4352, 4352, 1024), (torch.bfloat16, 4352, 4100, 520)])
+def test_uneven_work_per_workgroup_every_element(abi, variant, dt, M, N, K):
+    """17 tile rows over 256 workgroups: some store a tile while others are still in their main loop,
+    the load pattern under which a store once picked up the registers of the one after it.  Every
+    element is compared with the one-thread-per-output kernel, three launches in a row."""
+    if dt == torch.float8_e4m3fn:
+        A = torch.randint(0, 120, (M, K), dtype=torch.uint8, generator=torch.Generator().manual_seed(70)).view(dt)
+        B = torch.randint(0, 120, (N, K), dtype=torch.uint8, generator=torch.Generator().manual_seed(71)).view(dt)
+        scale = 2.0 ** -6
+    else:
+        A, B, scale = rand((M, K), 70, dt), rand((N, K), 71, dt), 1.0
+    Ad, Bd = A.cuda(), B.cuda()
+    S = torch.empty((M, N), dtype=out_dtype_of(dt), device="cuda")
+    assert ac.gemm_tn(abi, Ad, Bd, S, scale, ac.SIMPLE) == 0
+    for _ in range(3):
+        C = torch.full((M, N), float("nan"), dtype=out_dtype_of(dt), device="cuda")
+        assert ac.gemm_tn(abi, Ad, Bd, C, scale, variant) == 0
+        torch.cuda.synchronize()
+        d = (C.float() - S.float()).abs()
+        bad = d > 2e-2 * S.float().abs() + 2e-2 * (K ** 0.5) * scale
+        assert not torch.isnan(C).any() and int(bad.sum()) == 0, (int(bad.sum()), float(d.max()))
+
+
 @pytest.mark.parametrize("N,K", [(14336, 4096), (4096, 14336), (6144, 4096)])
 @pytest.mark.parametrize("M", [16, 64, 256])
 def test_config4_skinny_projections(abi, M, N, K):
