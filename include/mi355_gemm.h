@@ -35,7 +35,7 @@ enum mi355_dtype {
  * MI355_ERR_SHAPE when the shape does not meet that family's constraints). */
 enum mi355_variant {
   MI355_VARIANT_AUTO = 0,
-  MI355_VARIANT_BASIC = 1,    /* 256x256 tile, one wave group in lock step, LDS double buffer */
+  MI355_VARIANT_BASIC = 1,    /* 256x256 or 128x128 tile, one wave group, 5-slot LDS ring     */
   MI355_VARIANT_PINGPONG = 2, /* same tile, two wave groups alternating MFMA and load phases   */
   MI355_VARIANT_SKINNY = 3,   /* small-M weight-streaming kernel with split-K                  */
   MI355_VARIANT_SIMPLE = 4    /* one thread per output element; any shape; slow; self-check    */
@@ -71,8 +71,9 @@ enum mi355_status {
  * Replaces test::gemm_tn_test (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92): same operand
  * layout and the argument checks of :15-41, plus checks of C the reference omits; divisibility
  * by the tile is not required (the tiled variants need K*elem_bytes % 16 == 0, row strides that
- * are multiples of 16 bytes, N % 4 == 0 and ldc % 4 == 0; MI355_VARIANT_AUTO routes anything else
- * to the generic kernel).  Asynchronous: returns after enqueueing.
+ * are multiples of 16 bytes, N % 4 == 0, ldc % 4 == 0, 256 rows of A and of B below 2 GiB and
+ * 256*ldc below 2^29 elements; MI355_VARIANT_AUTO routes anything else to the generic kernel).
+ * Asynchronous: returns after enqueueing.
  */
 int mi355_gemm_tn(const void *A, const void *B, void *C,
                   int64_t M, int64_t N, int64_t K,
