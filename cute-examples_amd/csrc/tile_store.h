@@ -20,12 +20,6 @@ namespace mi355 {
 
 constexpr uint32_t kStoreOutOfRange = 0x80000000u;  // tiles of C span less than 2 GiB (host check)
 
-// A copy of one accumulator block to read element by element.  kPinned: the kernel's MFMAs are inline
-// assembly on accumulation registers; the empty statement here keeps the block in those registers up
-// to this point of the program, so the register allocator moves it to VGPRs here, block by block,
-// and not all 256 registers at once when the k loop ends (which would spill).  The reads
-// themselves stay ordinary compiler-generated moves: the compiler then also keeps them clear of the
-// data registers of stores still being issued, which hand-placed reads once overwrote.
 // A 16-byte buffer store followed by idle cycles.  The store reads its four data registers a few
 // cycles after it issues; the instructions that refill them for the next store come right behind
 // it, and with only the compiler's two wait states in between (as s_nop) a few lanes of the first
@@ -37,17 +31,22 @@ __device__ __forceinline__ void store_16B_guarded(u32x4 data, __amdgpu_buffer_rs
   asm volatile("s_nop 7");
 }
 
+// Called on an accumulator block right before it is read element by element.  kPinned: the kernel's
+// MFMAs are inline assembly on accumulation registers; the empty statement here keeps the block in
+// those registers up to this point of the program, so the register allocator moves it to VGPRs
+// here, block by block, and not all 256 registers at once when the k loop ends (which would
+// spill).  The reads themselves stay ordinary compiler-generated moves: the compiler then also keeps
+// them clear of the data registers of stores still being issued, which hand-placed reads once
+// overwrote.
 template <bool kPinned, class Acc>
-__device__ __forceinline__ Acc acc_block(const Acc& a) {
-  Acc t = a;
-  if constexpr (kPinned) asm volatile("" : "+a"(t));
-  return t;
+__device__ __forceinline__ void pin_acc_block(Acc& a) {
+  if constexpr (kPinned) asm volatile("" : "+a"(a));
 }
 
 // The wave's part of the output tile at (m0, n0), tile_edge rows and columns at most.
 // wave_row / wave_col: first row / column of the wave inside the tile.
 template <class T, class OutT, int kNbM, int kNbN, bool kAsmRead>
-__device__ __forceinline__ void store_output_tile(const typename Geo<T>::Acc (&acc)[kNbM][kNbN], const GemmArgs& g,
+__device__ __forceinline__ void store_output_tile(typename Geo<T>::Acc (&acc)[kNbM][kNbN], const GemmArgs& g,
                                                   int64_t m0, int64_t n0, int tile_edge, uint32_t wave_row,
                                                   uint32_t wave_col, uint32_t lane, float scale) {
   typedef Geo<T> G;
@@ -83,8 +82,9 @@ __device__ __forceinline__ void store_output_tile(const typename Geo<T>::Acc (&a
         // 0..7 / 8..15 of block j and groups 1,3 the same of block j+1.
         static_for<kNbN / 2>([&](auto jc) __attribute__((always_inline)) {
           constexpr int j = 2 * decltype(jc)::value;
-          const Acc c0 = acc_block<kAsmRead>(acc[i][j]), c1 = acc_block<kAsmRead>(acc[i][j + 1]);
-          u32x2 x = pack_quad(c0, 0), y = pack_quad(c1, 0);
+          pin_acc_block<kAsmRead>(acc[i][j]);
+          pin_acc_block<kAsmRead>(acc[i][j + 1]);
+          u32x2 x = pack_quad(acc[i][j], 0), y = pack_quad(acc[i][j + 1], 0);
           u32x2 lo = __builtin_amdgcn_permlane16_swap(x[0], y[0], false, false);
           u32x2 hi = __builtin_amdgcn_permlane16_swap(x[1], y[1], false, false);
           emit(ic, std::integral_constant<int, j * 16>{}, (u32x2){lo[0], hi[0]}, (u32x2){lo[1], hi[1]});
@@ -95,8 +95,8 @@ __device__ __forceinline__ void store_output_tile(const typename Geo<T>::Acc (&a
         // columns 16(q/2)..+7 and group 1 columns 16(q/2)+8..+15.
         static_for<kNbN * 2>([&](auto jq) __attribute__((always_inline)) {
           constexpr int j = decltype(jq)::value / 2, q = 2 * (decltype(jq)::value % 2);
-          const Acc c = acc_block<kAsmRead>(acc[i][j]);
-          u32x2 x = pack_quad(c, q), y = pack_quad(c, q + 1);
+          if constexpr (q == 0) pin_acc_block<kAsmRead>(acc[i][j]);
+          u32x2 x = pack_quad(acc[i][j], q), y = pack_quad(acc[i][j], q + 1);
           u32x2 lo = __builtin_amdgcn_permlane32_swap(x[0], y[0], false, false);
           u32x2 hi = __builtin_amdgcn_permlane32_swap(x[1], y[1], false, false);
           emit(ic, std::integral_constant<int, j * 32 + (q >> 1) * 16>{}, (u32x2){lo[0], hi[0]},
@@ -125,7 +125,7 @@ __device__ __forceinline__ void store_output_tile(const typename Geo<T>::Acc (&a
 // The same part of the tile as raw fp32 accumulators into plane `split` (M x N floats, row stride
 // N) of the split-K workspace: 4 consecutive columns per register quad, no lane exchange.
 template <class T, int kNbM, int kNbN, bool kAsmRead>
-__device__ __forceinline__ void store_partial_tile(const typename Geo<T>::Acc (&acc)[kNbM][kNbN], const GemmArgs& g,
+__device__ __forceinline__ void store_partial_tile(typename Geo<T>::Acc (&acc)[kNbM][kNbN], const GemmArgs& g,
                                                    int64_t m0, int64_t n0, int tile_edge, uint32_t split,
                                                    uint32_t wave_row, uint32_t wave_col, uint32_t lane) {
   typedef Geo<T> G;
@@ -146,7 +146,8 @@ __device__ __forceinline__ void store_partial_tile(const typename Geo<T>::Acc (&
       constexpr int j = decltype(jq)::value / kQuads, q = decltype(jq)::value % kQuads;
       constexpr int col = j * kBlk + q * 4 * G::kGroups;
       const uint32_t v = col0 + col + 4 <= cols ? v0 + col * 4 : kStoreOutOfRange;
-      const typename G::Acc c = acc_block<kAsmRead>(acc[i][j]);
+      if constexpr (q == 0) pin_acc_block<kAsmRead>(acc[i][j]);
+      const typename G::Acc& c = acc[i][j];
       const f32x4 quad = {c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
       store_16B_guarded(__builtin_bit_cast(u32x4, quad), rp, v, i * block_step, 0);
     });
