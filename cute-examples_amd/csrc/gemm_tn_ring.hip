@@ -21,16 +21,17 @@
 //   slice 1: MFMAs on buffer 1 | ds_reads of slice 0 of k-step t+1 -> buffer 0
 //   from the barrier to the end of the k-step: the 16 direct-to-LDS loads of B(t+2), A(t+3),
 //            spread evenly between the MFMAs
-// One workgroup barrier per k-step; the loop body is branch-free (loads past the end of K re-read the
-// last k-step into a slot nobody reads).
+// One workgroup barrier and one scalar branch per k-step: a workgroup has one wave per SIMD, so
+// every branch is a bubble in its MFMA stream.  The k loop is unrolled over the five positions of
+// the ring, which makes every LDS offset an immediate; copies past the end of K re-read the last
+// k-step into a slot nobody reads instead of being branched around.  The MFMAs are inline
+// assembly with the accumulator tied in place; fragment loads and everything else are compiled
+// code pinned between them with scheduling barriers.
 //
-// Tiles.  The grid is persistent: one workgroup per CU walks tiles blockIdx.x, +gridDim.x, ...
-// After the last k-step of a tile the workgroup first queues the five opening copies of its next
-// tile and only then converts and stores the finished accumulators, so the store phase of one
-// tile hides the load latency of the next.  Stores: two lanes' 4-element quads are exchanged with
-// v_permlane16_swap / v_permlane32_swap so that every lane writes 8 consecutive outputs (16 B),
-// with the non-temporal hint where a store covers whole 64-byte runs (C is written once and
-// should not evict operand panels from L2).
+// Tiles.  The grid is persistent: one workgroup per CU walks (tile, K-split) items blockIdx.x,
+// +gridDim.x, ...  After the last k-step of a tile the workgroup first queues the five opening
+// copies of its next tile and only then converts and stores the finished accumulators
+// (tile_store.h), so the store phase of one tile hides the load latency of the next.
 //
 // MFMA shape: bf16/fp16 use v_mfma_f32_16x16x32 (8x8 blocks per wave); on random data it sustains
 // a higher clock under the board power limit than 32x32x16.  fp8 uses v_mfma_f32_32x32x64_f8f6f4
