@@ -24,10 +24,11 @@ constexpr uint32_t kStoreOutOfRange = 0x80000000u;  // tiles of C span less than
 // cycles after it issues; the instructions that refill them for the next store come right behind
 // it, and with only the compiler's two wait states in between (as s_nop) a few lanes of the first
 // register were seen to pick up the new value.  Eight idle cycles per store are below measurement.
+// kAux: cache-policy bits of the store (1 = sc0, 2 = nt, 16 = sc1).
+template <int kAux>
 __device__ __forceinline__ void store_16B_guarded(u32x4 data, __amdgpu_buffer_rsrc_t rsrc, uint32_t voffset,
-                                                  uint32_t soffset, int aux_nt) {
-  if (aux_nt) __builtin_amdgcn_raw_buffer_store_b128(data, rsrc, voffset, soffset, 2);
-  else __builtin_amdgcn_raw_buffer_store_b128(data, rsrc, voffset, soffset, 0);
+                                                  uint32_t soffset) {
+  __builtin_amdgcn_raw_buffer_store_b128(data, rsrc, voffset, soffset, kAux);
   asm volatile("s_nop 7");
 }
 
@@ -52,10 +53,11 @@ __device__ __forceinline__ void store_output_tile(typename Geo<T>::Acc (&acc)[kN
   typedef Geo<T> G;
   typedef typename G::Acc Acc;
   constexpr int kBlk = G::kBlk;
-  // Non-temporal stores (aux bit 1) keep C out of L2: it is written once and would evict operand
-  // panels.  They only pay when a store instruction covers at least 64 contiguous bytes per row,
-  // which the 16-wide blocks do (two blocks side by side) and the 32-wide blocks do not (32 bytes).
-  constexpr int kAux = kBlk == 16 ? 2 : 0;
+  // Non-temporal, write-through stores (nt + sc1) keep C out of L2: it is written once and would
+  // evict operand panels.  They only pay when a store instruction covers at least 64 contiguous
+  // bytes per row, which the 16-wide blocks do (two blocks side by side) and the 32-wide blocks do
+  // not (32 bytes: measured 3 % slower with sc1, 25 % with nt + sc1).
+  constexpr int kAux = kBlk == 16 ? 18 : 0;
   const uint32_t rblk = lane & (kBlk - 1), grp = lane / kBlk;
   const int64_t rows = g.M - m0 < tile_edge ? g.M - m0 : tile_edge;
   const uint32_t cols = (uint32_t)(g.N - n0 < tile_edge ? g.N - n0 : tile_edge);
@@ -108,7 +110,7 @@ __device__ __forceinline__ void store_output_tile(typename Geo<T>::Acc (&acc)[kN
   if (cols == (uint32_t)tile_edge) {
     convert([&](auto ic, auto colc, u32x2 x, u32x2 y) __attribute__((always_inline)) {
       constexpr int i = decltype(ic)::value, col = decltype(colc)::value;
-      store_16B_guarded((u32x4){x[0], x[1], y[0], y[1]}, rc, v0 + col * 2, i * block_step, kAux);
+      store_16B_guarded<kAux>((u32x4){x[0], x[1], y[0], y[1]}, rc, v0 + col * 2, i * block_step);
     });
   } else {
     // N is a multiple of 4 (host check), so each half of the 8 columns is in or out as a whole.
@@ -149,7 +151,8 @@ __device__ __forceinline__ void store_partial_tile(typename Geo<T>::Acc (&acc)[k
       if constexpr (q == 0) pin_acc_block<kAsmRead>(acc[i][j]);
       const typename G::Acc& c = acc[i][j];
       const f32x4 quad = {c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
-      store_16B_guarded(__builtin_bit_cast(u32x4, quad), rp, v, i * block_step, 0);
+      // write-through: the partials are read back by another kernel, not by this one (+8 % measured)
+      store_16B_guarded<16>(__builtin_bit_cast(u32x4, quad), rp, v, i * block_step);
     });
   });
 }
