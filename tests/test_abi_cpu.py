@@ -46,6 +46,12 @@ def test_version_and_strerror(abi):
     ((257, 256, 128, 128, 128, 256, ac.BF16, ac.BF16, ac.SKINNY), ac.ERR_SHAPE),     # M > 256
     ((64, 256, 128, 128, 128, 256, ac.E4M3, ac.BF16, ac.SKINNY), ac.ERR_SHAPE),      # fp8
     ((0, 0, 0, 0, 0, 0, ac.BF16, ac.BF16, ac.AUTO), ac.OK),
+    # 32-bit offsets inside a tile: 256 rows of A or B below 2 GiB, 256 rows of fp32 partials too
+    ((256, 256, 64, 1 << 22, 64, 256, ac.BF16, ac.BF16, ac.BASIC), ac.ERR_SHAPE),
+    ((256, 256, 64, 1 << 22, 64, 256, ac.BF16, ac.BF16, ac.AUTO), ac.OK),
+    ((256, 256, 64, 64, 64, 1 << 21, ac.BF16, ac.BF16, ac.BASIC), ac.ERR_SHAPE),
+    ((256, 256, 64, 64, 64, (1 << 21) - 4, ac.BF16, ac.BF16, ac.BASIC), ac.OK),
+    ((256, 256, 64, 64, 64, 1 << 21, ac.BF16, ac.BF16, ac.AUTO), ac.OK),
 ])
 def test_check(abi, args, want):
     assert abi.mi355_gemm_check(*args) == want
@@ -92,7 +98,8 @@ def test_select_variant(abi):
     assert abi.mi355_gemm_select_variant(8192, 8192, 8192, 9) == ac.ERR_DTYPE
 
 
-@pytest.mark.parametrize("tm,tn", [(32, 32), (16, 16), (1, 1), (1, 56), (3, 5), (7, 9), (33, 31), (2, 24), (17, 1)])
+@pytest.mark.parametrize("tm,tn", [(32, 32), (16, 16), (1, 1), (1, 56), (3, 5), (7, 9), (33, 31), (2, 24), (17, 1),
+                                   (17, 17), (17, 16), (64, 64)])
 def test_tile_map_is_a_bijection(abi, tm, tn):
     seen = set()
     a, b = ctypes.c_int64(), ctypes.c_int64()
