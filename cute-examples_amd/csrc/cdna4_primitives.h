@@ -64,16 +64,6 @@ __device__ __forceinline__ void dma_16B_to_lds_at(uint32_t lds_base, uint32_t vo
       : "memory", "scc");
 }
 
-// Same copy through the compiler's own intrinsic: the compiler then sets M0, tracks the copy in
-// vmcnt against reads of the destination LDS object, and can schedule it like any VMEM load.
-// imm is added to both the buffer offset and the LDS address.
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-template <int kImm = 0>
-__device__ __forceinline__ void dma_16B_to_lds_tracked(void* lds_dst, uint32_t voffset,
-                                                       __amdgpu_buffer_rsrc_t rsrc, uint32_t soffset) {
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)lds_dst, 16, voffset, soffset, kImm, 0);
-}
-
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -83,34 +73,6 @@ __device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcn
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(uintptr_t)p;
 }
-
-// acc += X · Y^T for one 32x32 block.  x holds the block's "row" operand (lane%32 = row index,
-// lane/32 selects which k-chunks), y the "column" operand; result register r of lane l is
-// D[8*(r/4) + 4*(l/32) + r%4][l%32].
-template <class T> struct Mfma32;
-
-template <> struct Mfma32<BF16> {
-  typedef i32x4 Frag;
-  static __device__ __forceinline__ f32x16 run(Frag x, Frag y, f32x16 acc) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, x),
-                                                   __builtin_bit_cast(bf16x8, y), acc, 0, 0, 0);
-  }
-};
-template <> struct Mfma32<F16> {
-  typedef i32x4 Frag;
-  static __device__ __forceinline__ f32x16 run(Frag x, Frag y, f32x16 acc) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, x),
-                                                  __builtin_bit_cast(f16x8, y), acc, 0, 0, 0);
-  }
-};
-template <> struct Mfma32<E4M3> {
-  typedef i32x8 Frag;
-  static __device__ __forceinline__ f32x16 run(Frag x, Frag y, f32x16 acc) {
-    // cbsz = blgp = 0 selects e4m3 for both operands; zero scale operands select the unscaled
-    // form of the instruction.
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(x, y, acc, 0, 0, 0, 0, 0, 0);
-  }
-};
 
 // Four fp32 -> four 16-bit values (round to nearest even), packed into 8 bytes.
 template <class OutT> struct Pack4;
