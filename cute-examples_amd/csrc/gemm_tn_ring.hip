@@ -63,6 +63,10 @@ constexpr int first_copy_at(int p, int first, int span, int n) {
   return c;
 }
 
+// Geometry the kernel uses for an input type: fp8 runs on the 16x16x128 shape here.
+template <class T> struct RingGeo { typedef Geo<T> type; };
+template <> struct RingGeo<E4M3> { typedef GeoE4M3Rows type; };
+
 // kRaggedK: K*elem_bytes is not a multiple of the 128-byte k-step.  Kept out of the common
 // instantiation because selecting the per-lane offset inside the loop puts a dependent VALU
 // chain in front of every copy and costs ~8 % at 8192^3.
@@ -84,17 +88,20 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   constexpr int kCph = kTile / kWaves / kCopyRows;  // copies per operand per k-step per wave
   constexpr int kPar = 2;                           // copies j and j+kPar share their per-lane swizzle
   __shared__ __attribute__((aligned(1024))) uint8_t ring[kSlots * kSlotBytes];
-  typedef Geo<T> G;
+  typedef typename RingGeo<T>::type G;
   typedef typename G::Frag Frag;
   typedef typename G::Acc Acc;
   constexpr int kBlk = G::kBlk;
   constexpr int kNbM = kWaveTileM / kBlk, kNbN = kWaveTileN / kBlk;  // blocks per wave
-  constexpr int kSliceChunks = G::kGroups * G::kCpl;    // chunks of a row consumed per slice
-  constexpr int kSlices = 8 / kSliceChunks;
+  constexpr int kSliceChunks = G::kGroups * G::kCpl;    // chunks of a row consumed by one MFMA
   constexpr int kAccLen = kBlk * kBlk / 64;
-  constexpr int kMfmaPerSlice = kNbM * kNbN;
-  constexpr int kReadsPerSlice = kNbM + kNbN;               // fragment loads (each kCpl ds_read_b128)
-  static_assert(kSlices == 2, "the schedule below assumes two slices per k-step");
+  // A k-step is worked off in two slices: two halves of its 128 bytes of K, or, when one MFMA
+  // spans all of them, the two halves of the wave's rows of A.
+  constexpr bool kRowSliced = G::kRowSliced;
+  constexpr int kHalfM = kNbM / 2;                       // row blocks of A per slice when kRowSliced
+  constexpr int kMfmaPerSlice = kRowSliced ? kHalfM * kNbN : kNbM * kNbN;
+  constexpr int kReadsPerSlice = kNbM + kNbN;            // fragment loads per slice (K-sliced case)
+  static_assert(8 / kSliceChunks == (kRowSliced ? 1 : 2), "two slices per k-step");
 
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & 63u;
@@ -203,7 +210,11 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   };
 
   Acc acc[kNbM][kNbN];
-  Frag fa[2][kNbM], fb[2][kNbN];  // [fragment buffer][block]
+  // Fragments, [buffer][block].  K-sliced: slice s computes from buffer s while the other buffer is
+  // loaded for the next slice.  Row-sliced: slice s uses rows fa[s][0..kHalfM) of A and all of
+  // fb[0]; fa[s^1] is loaded meanwhile, and in slice 1 each block of B is reloaded for the next
+  // k-step as soon as its last MFMA has been issued (the MFMAs run B-block by B-block there).
+  Frag fa[2][kRowSliced ? kHalfM : kNbM], fb[kRowSliced ? 1 : 2][kNbN];
 
   // Load number q (0..kReadsPerSlice-1) of a slice: B blocks first (every MFMA row needs them all).
   auto read_q = [&](int buf, int q, const uint8_t* a_rows, const uint8_t* b_rows, int s)
@@ -219,15 +230,21 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     if constexpr (kTile == 256) G::mfma_inplace(fb[buf][j], fa[buf][i], acc[i][j]);
     else acc[i][j] = G::mfma(fb[buf][j], fa[buf][i], acc[i][j]);
   };
+  // Row-sliced order: B-block j outermost, the slice's kHalfM row blocks of A inside.
+  auto mfma_rows = [&](int s, int u) __attribute__((always_inline)) {
+    const int j = u / kHalfM, r = u % kHalfM;
+    if constexpr (kTile == 256) G::mfma_inplace(fb[0][j], fa[s][r], acc[s * kHalfM + r][j]);
+    else acc[s * kHalfM + r][j] = G::mfma(fb[0][j], fa[s][r], acc[s * kHalfM + r][j]);
+  };
 
   // Stores of the tile at (m0, n0): converted output, or fp32 partials for a split-K item.
   const float scale = output_scale(g);
   constexpr bool kAsmMfma = kTile == 256;  // see mfma_u
   auto epilogue = [&](int64_t m0, int64_t n0) __attribute__((always_inline)) {
-    store_output_tile<T, OutT, kNbM, kNbN, kAsmMfma>(acc, g, m0, n0, kTile, wm * kWaveTileM, wn * kWaveTileN, lane, scale);
+    store_output_tile<G, OutT, kNbM, kNbN, kAsmMfma>(acc, g, m0, n0, kTile, wm * kWaveTileM, wn * kWaveTileN, lane, scale);
   };
   auto store_partial = [&](int64_t m0, int64_t n0, uint32_t split) __attribute__((always_inline)) {
-    store_partial_tile<T, kNbM, kNbN, kAsmMfma>(acc, g, m0, n0, kTile, split, wm * kWaveTileM, wn * kWaveTileN, lane);
+    store_partial_tile<G, kNbM, kNbN, kAsmMfma>(acc, g, m0, n0, kTile, split, wm * kWaveTileM, wn * kWaveTileN, lane);
   };
 
   uint32_t item = blockIdx.x;
@@ -249,9 +266,15 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     // A0 and B0 have landed; A1, B1, A2 may be in flight (the counter saturates at 63).
     wait_vmcnt<(3 * kCph < 63 ? 3 * kCph : 63)>();
     __builtin_amdgcn_s_barrier();
+    if constexpr (kRowSliced) {
 #pragma unroll
-    for (int q = 0; q < kReadsPerSlice; ++q)
-      read_q(0, q, ring + a_lane, ring + kSlotBytes + b_lane, 0);
+      for (int j = 0; j < kNbN; ++j) fb[0][j] = load_frag(ring + kSlotBytes + b_lane, j, 0);
+#pragma unroll
+      for (int r = 0; r < kHalfM; ++r) fa[0][r] = load_frag(ring + a_lane, r, 0);
+    } else {
+#pragma unroll
+      for (int q = 0; q < kReadsPerSlice; ++q) read_q(0, q, ring + a_lane, ring + kSlotBytes + b_lane, 0);
+    }
 
     // The slot of A(t) walks 0, 2, 4, 1, 3 and repeats, so the loop is unrolled over five phases in
     // which every slot number, and with it every LDS offset, is a compile-time constant.
@@ -277,7 +300,13 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
       //            issued faster than the texture-address unit retires them (one 1 KiB copy takes
       //            it ~23 cycles and it serves all four waves): a wave whose copy finds the unit's
       //            queue full stalls at issue and its MFMA stream stops with it.
-      constexpr int kBarrierWant = kReadsPerSlice + kMfmaPerSlice / 8;
+      // Row-sliced read schedule (position u of a slice, before MFMA u is issued):
+      //   slice 0  u = 1: B block kNbN-1 of THIS k-step (its last MFMA of the previous k-step was the
+      //            last one of that k-step); u = 2 .. kHalfM+1: the second half of A's rows
+      //   slice 1  u = 0 .. kHalfM-1: the first half of A's rows of the next k-step;
+      //            u = kHalfM*(j+1)+1: B block j of the next k-step, one MFMA after its last use
+      constexpr int kLastOwnRead = kRowSliced ? kHalfM + 1 : kReadsPerSlice - 1;
+      constexpr int kBarrierWant = kLastOwnRead + 1 + kMfmaPerSlice / 8;
       constexpr int kBarrierAt = kBarrierWant < kMfmaPerSlice ? kBarrierWant : kMfmaPerSlice - 1;
       constexpr int kFirstCopy = kBarrierAt + 1;
       constexpr int kCopies = 2 * kCph;                                  // B(t+2) then A(t+3)
@@ -288,7 +317,16 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
       static_for<2 * kMfmaPerSlice>([&](auto pc) __attribute__((always_inline)) {
         constexpr int p = decltype(pc)::value;
         constexpr int s = p / kMfmaPerSlice, u = p % kMfmaPerSlice;
-        if constexpr (u < kReadsPerSlice) {
+        if constexpr (kRowSliced) {
+          if constexpr (s == 0) {
+            if constexpr (u == 1) fb[0][kNbN - 1] = load_frag(b_rows, kNbN - 1, 0);
+            if constexpr (u >= 2 && u < 2 + kHalfM) fa[1][u - 2] = load_frag(a_rows, kHalfM + u - 2, 0);
+          } else {
+            if constexpr (u < kHalfM) fa[0][u] = load_frag(a1_rows, u, 0);
+            if constexpr (u > kHalfM && (u - 1) % kHalfM == 0 && (u - 1) / kHalfM - 1 < kNbN - 1)
+              fb[0][(u - 1) / kHalfM - 1] = load_frag(b1_rows, (u - 1) / kHalfM - 1, 0);
+          }
+        } else if constexpr (u < kReadsPerSlice) {
           if constexpr (s == 0) read_q(1, u, a_rows, b_rows, 1);       // slice 1 of this k-step
           else read_q(0, u, a1_rows, b1_rows, 0);                      // slice 0 of the next k-step
         }
@@ -311,7 +349,8 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
             }
           });
         }
-        mfma_u(s, u);
+        if constexpr (kRowSliced) mfma_rows(s, u);
+        else mfma_u(s, u);
         MI355_FENCE();
       });
       soff_b = soff_b + kRowBytes < soff_last ? soff_b + kRowBytes : soff_last;

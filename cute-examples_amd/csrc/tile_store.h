@@ -46,11 +46,10 @@ __device__ __forceinline__ void pin_acc_block(Acc& a) {
 
 // The wave's part of the output tile at (m0, n0), tile_edge rows and columns at most.
 // wave_row / wave_col: first row / column of the wave inside the tile.
-template <class T, class OutT, int kNbM, int kNbN, bool kAsmRead>
-__device__ __forceinline__ void store_output_tile(typename Geo<T>::Acc (&acc)[kNbM][kNbN], const GemmArgs& g,
+template <class G, class OutT, int kNbM, int kNbN, bool kAsmRead>
+__device__ __forceinline__ void store_output_tile(typename G::Acc (&acc)[kNbM][kNbN], const GemmArgs& g,
                                                   int64_t m0, int64_t n0, int tile_edge, uint32_t wave_row,
                                                   uint32_t wave_col, uint32_t lane, float scale) {
-  typedef Geo<T> G;
   typedef typename G::Acc Acc;
   constexpr int kBlk = G::kBlk;
   // Non-temporal, write-through stores (nt + sc1) keep C out of L2: it is written once and would
@@ -126,11 +125,10 @@ __device__ __forceinline__ void store_output_tile(typename Geo<T>::Acc (&acc)[kN
 
 // The same part of the tile as raw fp32 accumulators into plane `split` (M x N floats, row stride
 // N) of the split-K workspace: 4 consecutive columns per register quad, no lane exchange.
-template <class T, int kNbM, int kNbN, bool kAsmRead>
-__device__ __forceinline__ void store_partial_tile(typename Geo<T>::Acc (&acc)[kNbM][kNbN], const GemmArgs& g,
+template <class G, int kNbM, int kNbN, bool kAsmRead>
+__device__ __forceinline__ void store_partial_tile(typename G::Acc (&acc)[kNbM][kNbN], const GemmArgs& g,
                                                    int64_t m0, int64_t n0, int tile_edge, uint32_t split,
                                                    uint32_t wave_row, uint32_t wave_col, uint32_t lane) {
-  typedef Geo<T> G;
   constexpr int kBlk = G::kBlk;
   constexpr int kQuads = kBlk * kBlk / 64 / 4;
   const uint32_t rblk = lane & (kBlk - 1), grp = lane / kBlk;
