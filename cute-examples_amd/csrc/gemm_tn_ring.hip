@@ -34,8 +34,10 @@
 // (tile_store.h), so the store phase of one tile hides the load latency of the next.
 //
 // MFMA shape: bf16/fp16 use v_mfma_f32_16x16x32 (8x8 blocks per wave); on random data it sustains
-// a higher clock under the board power limit than 32x32x16.  fp8 uses v_mfma_f32_32x32x64_f8f6f4
-// (4x4 blocks), which keeps the fragment registers within budget.
+// a higher clock under the board power limit than 32x32x16.  fp8 uses v_mfma_f32_16x16x128_f8f6f4
+// (8x8 blocks) for the same reason; one such MFMA spans the whole k-step, so the two slices of a
+// k-step are the two halves of the wave's rows of A instead of two halves of K, and the blocks of
+// B are reloaded in place, each right after its last use (see the fragment arrays below).
 //
 // Counterpart in the reference: the cooperative kernel, kernels/gemm_kernels/sm90a/gemm.cuh:246-418
 // (TMA producer warpgroup, mbarrier full/empty ring of 3 stages, two consumer warpgroups); here
