@@ -147,6 +147,39 @@ def test_ragged_shapes(abi, dt, M, N, K, variant):
     assert oracle.rel_frobenius(C, oracle.c_gemm_tn_f32(A, B)) <= TOL[dt]
 
 
+def _random_shapes(count, seed):
+    """Seeded shapes that the tiled kernels accept: any M, N a multiple of 4, K*elem_bytes a multiple of 16."""
+    import random
+    rng = random.Random(seed)
+    shapes = []
+    for _ in range(count):
+        M = rng.choice([rng.randint(1, 64), rng.randint(65, 700), rng.randint(701, 2200)])
+        N = 4 * rng.choice([rng.randint(1, 16), rng.randint(17, 200), rng.randint(201, 600)])
+        K = 16 * rng.choice([rng.randint(1, 8), rng.randint(9, 64), rng.randint(65, 300)])
+        shapes.append((M, N, K))
+    return shapes
+
+
+@pytest.mark.parametrize("dt", list(DTYPES.values()))
+def test_random_shape_sweep(abi, dt):
+    """40 seeded random shapes per input type through AUTO and both tiled variants, each against
+    the oracle's fp32 product and with NaN guards around C (edge tiles in M and N, ragged and tiny K,
+    128- and 256-wide tiles, K splits, the streaming kernel)."""
+    for (M, N, K) in _random_shapes(40, 2024):
+        if dt == torch.float8_e4m3fn:
+            a, b = rand((M, K), M + K, torch.float32), rand((N, K), N + K, torch.float32)
+            (A, sa), (B, sb) = oracle.quantize_e4m3(a), oracle.quantize_e4m3(b)
+            scale = float(sa) * float(sb)
+        else:
+            A, B, scale = rand((M, K), M + K, dt), rand((N, K), N + K, dt), 1.0
+        ref = oracle.gemm_tn_fp32(A, B, scale)
+        for variant in [ac.AUTO] + TILED:
+            C = run_abi(abi, A, B, variant, scale=scale, ldc=N + 8 if (M + N) % 3 == 0 else None)
+            assert oracle.no_nan_left(C), (M, N, K, variant)
+            err = oracle.rel_frobenius(C, ref)
+            assert err <= TOL[dt], (M, N, K, variant, err)
+
+
 @pytest.mark.parametrize("M,N,K", [(5, 7, 3), (33, 17, 50), (100, 30, 77), (64, 64, 4)])
 @pytest.mark.parametrize("dt", list(DTYPES.values()))
 def test_shapes_only_the_simple_kernel_takes(abi, dt, M, N, K):
