@@ -21,6 +21,8 @@ typedef __attribute__((ext_vector_type(4))) unsigned u32x4;
 struct BF16 { static constexpr int kBytes = 2; static constexpr int kSliceChunks = 1; };
 struct F16  { static constexpr int kBytes = 2; static constexpr int kSliceChunks = 1; };
 struct E4M3 { static constexpr int kBytes = 1; static constexpr int kSliceChunks = 2; };
+// e4m3 elements that carry one E8M0 scale per 32 consecutive elements of K (OCP MX block scaling).
+struct MxE4M3 : E4M3 {};
 
 // Raw (unstructured) buffer descriptor over [base, base+bytes): loads beyond `bytes` return 0,
 // which is how ragged tile edges are handled.
@@ -64,9 +66,26 @@ __device__ __forceinline__ void dma_16B_to_lds_at(uint32_t lds_base, uint32_t vo
       : "memory", "scc");
 }
 
+// 8 bytes per lane from buffer offset voffset(l) + soffset into a register pair, WITHOUT the
+// compiler knowing that the result arrives later: the caller must pass the pair through
+// wait_vmcnt_for<N>() (N = vector-memory instructions issued after this one) before its first use,
+// and must check in the generated code that the pair is not copied in between.
+__device__ __forceinline__ void load_8B_async(u32x2& dst, __amdgpu_buffer_rsrc_t rsrc, uint32_t voffset,
+                                              uint32_t soffset) {
+  asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen"
+               : "=v"(dst)
+               : "v"(voffset), "s"(rsrc), "s"(__builtin_amdgcn_readfirstlane(soffset))
+               : "memory");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// The same wait, naming the registers whose asynchronous loads it completes.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_for(u32x2& a, u32x2& b) {
+  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
 }
 __device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 

@@ -125,6 +125,93 @@ int mi355_quantize_e4m3(const void* x, int x_dtype, int64_t n, void* x_q, float*
                                                                                               : MI355_ERR_LAUNCH;
 }
 
+size_t mi355_mx_shuffled_bytes(int64_t rows, int64_t K) {
+  if (rows <= 0 || K <= 0 || K % 128 != 0) return 0;
+  return mi355::mx_shuffled_bytes(rows, K);
+}
+
+int mi355_mx_shuffle_scales(const uint8_t* scales, int64_t rows, int64_t K, int64_t ld, uint8_t* out, void* stream) {
+  if (rows < 0 || K < 0 || K % 128 != 0 || ld < K / 32) return MI355_ERR_SHAPE;
+  if (rows == 0 || K == 0) return MI355_OK;
+  if (!scales || !out) return MI355_ERR_NULL;
+  if ((uintptr_t)out % 8 != 0) return MI355_ERR_ALIGN;
+  return mi355::launch_mx_shuffle(scales, rows, K, ld, out, (hipStream_t)stream) == 0 ? MI355_OK : MI355_ERR_LAUNCH;
+}
+
+int mi355_quantize_mxfp8(const void* x, int x_dtype, int64_t rows, int64_t K, int64_t ldx, void* x_q,
+                         uint8_t* scales, void* stream) {
+  if (x_dtype != MI355_BF16 && x_dtype != MI355_F16 && x_dtype != MI355_F32) return MI355_ERR_DTYPE;
+  if (rows < 0 || K < 0 || K % 32 != 0 || ldx < K) return MI355_ERR_SHAPE;
+  if (rows == 0 || K == 0) return MI355_OK;
+  if (!x || !x_q || !scales) return MI355_ERR_NULL;
+  const int64_t es = x_dtype == MI355_F32 ? 4 : 2;
+  if ((uintptr_t)x % 16 != 0 || (ldx * es) % 16 != 0 || (uintptr_t)x_q % 16 != 0) return MI355_ERR_ALIGN;
+  return mi355::launch_quantize_mxfp8(x, x_dtype, rows, K, ldx, x_q, scales, (hipStream_t)stream) == 0
+             ? MI355_OK : MI355_ERR_LAUNCH;
+}
+
+int mi355_gemm_mx_check(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int out_dtype) {
+  if (!valid_out(out_dtype)) return MI355_ERR_DTYPE;
+  if (M < 0 || N < 0 || K < 0) return MI355_ERR_SHAPE;
+  if (lda < K || ldb < K || ldc < N) return MI355_ERR_SHAPE;
+  if (K % 128 != 0) return MI355_ERR_SHAPE;
+  if (M == 0 || N == 0) return MI355_OK;
+  if (K > 0 && !tile256_ok(M, N, K, lda, ldb, ldc, MI355_E4M3)) return MI355_ERR_SHAPE;
+  // 32-bit offsets into the shuffled scale arrays
+  if (mi355::mx_shuffled_bytes(M, K) >= ((size_t)1 << 31) || mi355::mx_shuffled_bytes(N, K) >= ((size_t)1 << 31))
+    return MI355_ERR_SHAPE;
+  return MI355_OK;
+}
+
+size_t mi355_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int scales_shuffled) {
+  if (scales_shuffled || M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
+  return mi355::mx_shuffled_bytes(M, K) + mi355::mx_shuffled_bytes(N, K);
+}
+
+int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                        int64_t ldb, int64_t ldc, const uint8_t* scale_a, int64_t ld_scale_a,
+                        const uint8_t* scale_b, int64_t ld_scale_b, int scales_shuffled, int out_dtype,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+  int st = mi355_gemm_mx_check(M, N, K, lda, ldb, ldc, out_dtype);
+  if (st != MI355_OK) return st;
+  if (M == 0 || N == 0) return MI355_OK;
+  if (!C) return MI355_ERR_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  mi355::GemmArgs g;
+  g.A = A_q; g.B = B_q; g.C = C;
+  g.M = M; g.N = N; g.K = K;
+  g.lda = lda; g.ldb = ldb; g.ldc = ldc;
+  g.scale = 1.0f;
+  g.splits = 1;
+  g.partial = nullptr;
+  g.scale_a = g.scale_b = nullptr;
+  g.mx_a = g.mx_b = nullptr;
+  if (K == 0) {  // an empty sum: zeros, written by the generic kernel
+    g.tiles_m = g.tiles_n = 0;
+    return mi355::launch_simple(g, MI355_E4M3, out_dtype, s) == 0 ? MI355_OK : MI355_ERR_LAUNCH;
+  }
+  if (!A_q || !B_q || !scale_a || !scale_b) return MI355_ERR_NULL;
+  if ((uintptr_t)A_q % 16 != 0 || (uintptr_t)B_q % 16 != 0 || (uintptr_t)C % 8 != 0) return MI355_ERR_ALIGN;
+  if (scales_shuffled) {
+    if ((uintptr_t)scale_a % 8 != 0 || (uintptr_t)scale_b % 8 != 0) return MI355_ERR_ALIGN;
+    g.mx_a = scale_a;
+    g.mx_b = scale_b;
+  } else {
+    if (ld_scale_a < K / 32 || ld_scale_b < K / 32) return MI355_ERR_SHAPE;
+    const size_t bytes_a = mi355::mx_shuffled_bytes(M, K), bytes_b = mi355::mx_shuffled_bytes(N, K);
+    if (!workspace || workspace_bytes < bytes_a + bytes_b || (uintptr_t)workspace % 16 != 0) return MI355_ERR_WORKSPACE;
+    uint8_t* wa = (uint8_t*)workspace;
+    uint8_t* wb = wa + bytes_a;  // bytes_a is a multiple of 1024
+    if (mi355::launch_mx_shuffle(scale_a, M, K, ld_scale_a, wa, s) != 0) return MI355_ERR_LAUNCH;
+    if (mi355::launch_mx_shuffle(scale_b, N, K, ld_scale_b, wb, s) != 0) return MI355_ERR_LAUNCH;
+    g.mx_a = wa;
+    g.mx_b = wb;
+  }
+  g.tiles_m = (M + 255) / 256;
+  g.tiles_n = (N + 255) / 256;
+  return mi355::launch_tile_ring_mx(g, out_dtype, s) == 0 ? MI355_OK : MI355_ERR_LAUNCH;
+}
+
 int mi355_gemm_tn(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
                   int64_t lda, int64_t ldb, int64_t ldc, int in_dtype, int out_dtype, float scale,
                   int variant, void* workspace, size_t workspace_bytes, void* stream) {
@@ -152,6 +239,7 @@ int mi355_gemm_tn_scaled(const void* A, const void* B, void* C, int64_t M, int64
   g.partial = nullptr;
   g.scale_a = scale_a;
   g.scale_b = scale_b;
+  g.mx_a = g.mx_b = nullptr;
   hipStream_t s = (hipStream_t)stream;
 
   if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG || v == MI355_VARIANT_SKINNY) {

@@ -23,6 +23,9 @@ struct GemmArgs {
   // kernel that writes C, so that per-tensor fp8 scales never have to visit the host.
   const float* scale_a;
   const float* scale_b;
+  // Block scales (MX) of A and of B in the shuffled layout, or null.
+  const uint8_t* mx_a;
+  const uint8_t* mx_b;
 };
 
 // Effective output scale; wave-uniform, read once per workgroup.
@@ -45,6 +48,14 @@ int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes);
 // C = rne(scale * sum_s partial[s]) for partial laid out [splits][M][N] in fp32.
 int launch_splitk_reduce(const float* partial, const GemmArgs& g, int out_dtype, hipStream_t stream);
 int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, hipStream_t stream);
+int launch_tile_ring_mx(const GemmArgs& g, int out_dtype, hipStream_t stream);
+// Block scales: bytes of the shuffled layout for `rows` rows and K elements per row; the shuffle
+// itself (natural (rows, K/32) row-major bytes -> shuffled); and the MX quantiser
+// (x (rows, K) -> e4m3 elements + natural-layout E8M0 scales).
+size_t mx_shuffled_bytes(int64_t rows, int64_t K);
+int launch_mx_shuffle(const uint8_t* scales, int64_t rows, int64_t K, int64_t ld, uint8_t* out, hipStream_t stream);
+int launch_quantize_mxfp8(const void* x, int in_dtype, int64_t rows, int64_t K, int64_t ldx, void* q,
+                          uint8_t* scales, hipStream_t stream);
 // Skinny (small-M) weight-streaming kernel.  stream_splits is a pure host function.
 int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes);
 int launch_stream(const GemmArgs& g, int in_dtype, int out_dtype, int splits, void* workspace, hipStream_t stream);

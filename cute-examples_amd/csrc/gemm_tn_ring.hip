@@ -68,6 +68,13 @@ constexpr int first_copy_at(int p, int first, int span, int n) {
 // Geometry the kernel uses for an input type: fp8 runs on the 16x16x128 shape here.
 template <class T> struct RingGeo { typedef Geo<T> type; };
 template <> struct RingGeo<E4M3> { typedef GeoE4M3Rows type; };
+template <> struct RingGeo<MxE4M3> { typedef GeoMxE4M3Rows type; };
+
+// Layout of block scales as the kernel reads them ("shuffled", written by mx_scales.hip): one
+// 512-byte unit per (group of 128 rows, k-step); lane l of the wave that owns those rows reads the
+// 8 bytes at 8*l: byte i is the scale of row 16*i + l%16 of the group for K block 4*kstep + l/16.
+// Units are ordered [row group][k-step], and the arrays are padded to whole 256-row tiles.
+constexpr uint32_t kMxUnitBytes = 512;
 
 // kRaggedK: K*elem_bytes is not a multiple of the 128-byte k-step.  Kept out of the common
 // instantiation because selecting the per-lane offset inside the loop puts a dependent VALU
@@ -100,6 +107,9 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   // A k-step is worked off in two slices: two halves of its 128 bytes of K, or, when one MFMA
   // spans all of them, the two halves of the wave's rows of A.
   constexpr bool kRowSliced = G::kRowSliced;
+  constexpr bool kMx = G::kMx;
+  static_assert(!kMx || (kRowSliced && !kRaggedK && kWaveTileM == 128 && kWaveTileN == 128),
+                "block scales: whole k-steps, one 128-row scale group per wave and operand");
   constexpr int kHalfM = kNbM / 2;                       // row blocks of A per slice when kRowSliced
   constexpr int kMfmaPerSlice = kRowSliced ? kHalfM * kNbN : kNbM * kNbN;
   constexpr int kReadsPerSlice = kNbM + kNbN;            // fragment loads per slice (K-sliced case)
@@ -182,6 +192,25 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     return __builtin_amdgcn_readfirstlane((step0 + (kt < steps ? kt : steps - 1)) * kRowBytes);
   };
   // Opening copies of a tile: A0 B0 A1 B1 A2 into slots 0..4.
+  // Block scales (kMx only).  Set ph holds the scales of the k-step worked off in ring phase ph:
+  // [0] rows 0..63 and [1] rows 64..127 of the wave's rows of A (sca) and of B (scb), one byte per
+  // 16-row block.  A set is loaded two k-steps ahead by load_8B_async; see the waits at its users.
+  u32x2 sca[kSlots], scb[kSlots];
+  const __amdgpu_buffer_rsrc_t rsrc_sa = make_raw_buffer(g.mx_a, kMx ? tiles_m * 2u * k_steps * kMxUnitBytes : 0u);
+  const __amdgpu_buffer_rsrc_t rsrc_sb = make_raw_buffer(g.mx_b, kMx ? tiles_n * 2u * k_steps * kMxUnitBytes : 0u);
+  uint32_t voff_sa = 0, voff_sb = 0;  // lane's bytes of the current item's first unit
+  // Scale offset of k-step kt of the current item, clamped to its last like soff_of.
+  auto mx_soff_of = [&](uint32_t kt) __attribute__((always_inline)) -> uint32_t {
+    return __builtin_amdgcn_readfirstlane((kt < steps ? kt : steps - 1) * kMxUnitBytes);
+  };
+  auto mx_open_tile = [&](uint32_t tm, uint32_t tn, uint32_t step0) __attribute__((always_inline)) {
+    voff_sa = ((tm * 2 + wm) * k_steps + step0) * kMxUnitBytes + lane * 8;
+    voff_sb = ((tn * 2 + wn) * k_steps + step0) * kMxUnitBytes + lane * 8;
+    load_8B_async(sca[0], rsrc_sa, voff_sa, mx_soff_of(0));
+    load_8B_async(scb[0], rsrc_sb, voff_sb, mx_soff_of(0));
+    load_8B_async(sca[1], rsrc_sa, voff_sa, mx_soff_of(1));
+    load_8B_async(scb[1], rsrc_sb, voff_sb, mx_soff_of(1));
+  };
   auto open_tile = [&](__amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb, uint32_t step0) __attribute__((always_inline)) {
     const uint32_t s0 = soff_of(step0, 0), s1 = soff_of(step0, 1), s2 = soff_of(step0, 2);
     static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, std::integral_constant<uint32_t, 0>{}, s0); });
@@ -197,8 +226,10 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   const uint32_t a_lane = (wm * kWaveTileM + rblk) * kRowBytes;
   const uint32_t b_lane = (wn * kWaveTileN + rblk) * kRowBytes;
   // Byte offset inside a row of the e-th chunk this lane reads in slice s.
+  // With block scales the order of K inside the MFMA matters: group g supplies chunks g and 4+g.
   auto chunk_off = [&](int s, int e) __attribute__((always_inline)) -> uint32_t {
-    return ((uint32_t)(s * kSliceChunks + grp * G::kCpl + e) ^ swz) << 4;
+    if constexpr (kMx) return ((uint32_t)(grp + 4 * e) ^ swz) << 4;
+    else return ((uint32_t)(s * kSliceChunks + grp * G::kCpl + e) ^ swz) << 4;
   };
   auto load_frag = [&](const uint8_t* slot_rows, int blk, int s) __attribute__((always_inline)) -> Frag {
     const uint8_t* p = slot_rows + blk * kBlk * kRowBytes;
@@ -233,10 +264,17 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     else acc[i][j] = G::mfma(fb[buf][j], fa[buf][i], acc[i][j]);
   };
   // Row-sliced order: B-block j outermost, the slice's kHalfM row blocks of A inside.
-  auto mfma_rows = [&](int s, int u) __attribute__((always_inline)) {
-    const int j = u / kHalfM, r = u % kHalfM;
-    if constexpr (kTile == 256) G::mfma_inplace(fb[0][j], fa[s][r], acc[s * kHalfM + r][j]);
-    else acc[s * kHalfM + r][j] = G::mfma(fb[0][j], fa[s][r], acc[s * kHalfM + r][j]);
+  auto mfma_rows = [&](auto phc, auto sc, auto uc) __attribute__((always_inline)) {
+    constexpr int ph = decltype(phc)::value, s = decltype(sc)::value, u = decltype(uc)::value;
+    constexpr int j = u / kHalfM, r = u % kHalfM, i = s * kHalfM + r;
+    if constexpr (kMx) {
+      static_assert(kTile == 256, "block scales run on the 256-wide tile only");
+      G::template mfma_scaled_inplace<j % 4, i % 4>(fb[0][j], fa[s][r], acc[i][j], scb[ph][j / 4], sca[ph][i / 4]);
+    } else {
+      (void)ph;
+      if constexpr (kTile == 256) G::mfma_inplace(fb[0][j], fa[s][r], acc[i][j]);
+      else acc[i][j] = G::mfma(fb[0][j], fa[s][r], acc[i][j]);
+    }
   };
 
   // Stores of the tile at (m0, n0): converted output, or fp32 partials for a split-K item.
@@ -255,6 +293,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   uint32_t split = item / total_tiles;
   uint32_t step0 = __builtin_amdgcn_readfirstlane(split * steps);  // first k-step of the current item
   __amdgpu_buffer_rsrc_t rsrc_a = panel_a((int64_t)tile_m * kTile), rsrc_b = panel_b((int64_t)tile_n * kTile);
+  if constexpr (kMx) mx_open_tile(tile_m, tile_n, step0);  // before the copies: see the waits
   open_tile(rsrc_a, rsrc_b, step0);
 
   for (;;) {
@@ -283,6 +322,9 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     // Row offsets of the operand k-steps the loop copies next, B(t+2) and A(t+3).
     const uint32_t soff_last = soff_of(step0, steps - 1);
     uint32_t soff_b = soff_of(step0, 2), soff_a = soff_of(step0, 3);
+    // Offset of the scales the loop loads next (those of k-step t+2).
+    const uint32_t mx_soff_last = mx_soff_of(steps - 1);
+    uint32_t mx_soff = mx_soff_of(2);
     uint32_t kt = 0;
     bool last = false;
     for (;;) {
@@ -316,6 +358,15 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
       static_assert(kCopySpan > 0, "no room for the copies");
       // copy c is issued at position kFirstCopy + c * kCopySpan / kCopies (evenly spread)
       constexpr int kMaxCopiesPerGap = (kCopies + kCopySpan - 1) / kCopySpan + 1;
+      constexpr int ph = decltype(phase)::value;
+      if constexpr (kMx) {
+        // The scales of this k-step were requested two k-steps ago (or with the opening copies of
+        // the tile, ahead of them).  Vector-memory instructions issued since: that k-step's copies,
+        // the next request, the copies of the k-step after it.  Loads return in order.
+        wait_vmcnt_for<2 * kCopies + 2>(sca[ph], scb[ph]);
+        load_8B_async(sca[(ph + 2) % kSlots], rsrc_sa, voff_sa, mx_soff);
+        load_8B_async(scb[(ph + 2) % kSlots], rsrc_sb, voff_sb, mx_soff);
+      }
       static_for<2 * kMfmaPerSlice>([&](auto pc) __attribute__((always_inline)) {
         constexpr int p = decltype(pc)::value;
         constexpr int s = p / kMfmaPerSlice, u = p % kMfmaPerSlice;
@@ -336,7 +387,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
           // My reads of this k-step's slots are back; B(t+1) (and A(t+1) before it) have
           // landed; only this wave's copies of A(t+2) may still be in flight.
           wait_lgkmcnt0();
-          wait_vmcnt<kCph>();
+          wait_vmcnt<kCph + (kMx ? 2 : 0)>();  // the two scale requests of this k-step are younger still
           __builtin_amdgcn_s_barrier();
         }
         if constexpr (p >= kFirstCopy) {
@@ -351,12 +402,14 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
             }
           });
         }
-        if constexpr (kRowSliced) mfma_rows(s, u);
+        if constexpr (kRowSliced)
+          mfma_rows(phase, std::integral_constant<int, s>{}, std::integral_constant<int, u>{});
         else mfma_u(s, u);
         MI355_FENCE();
       });
       soff_b = soff_b + kRowBytes < soff_last ? soff_b + kRowBytes : soff_last;
       soff_a = soff_a + kRowBytes < soff_last ? soff_a + kRowBytes : soff_last;
+      if constexpr (kMx) mx_soff = mx_soff + kMxUnitBytes < mx_soff_last ? mx_soff + kMxUnitBytes : mx_soff_last;
       ++kt;
       last = kt == steps;
     });
@@ -378,6 +431,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
       step0 = __builtin_amdgcn_readfirstlane(split * steps);
       rsrc_a = panel_a((int64_t)tile_m * kTile);
       rsrc_b = panel_b((int64_t)tile_n * kTile);
+      if constexpr (kMx) mx_open_tile(tile_m, tile_n, step0);
       open_tile(rsrc_a, rsrc_b, step0);  // in flight while the finished tile is stored
     }
     if (g.splits > 1) store_partial(done_m0, done_n0, done_split);
@@ -393,10 +447,12 @@ int launch_tile(const GemmArgs& g, hipStream_t stream) {
   const int64_t slots = (int64_t)compute_units() * (kTileT == 256 ? 1 : 2);  // resident workgroups (LDS-bound)
   const int64_t blocks = items < slots ? items : slots;
   constexpr int kWavesN = 2;
-  if ((g.K * T::kBytes) % kRowBytes == 0)
+  if ((g.K * T::kBytes) % kRowBytes == 0) {
     hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, false, kTileT, kWavesN>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
-  else
-    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, true, kTileT, kWavesN>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
+  } else {
+    if constexpr (std::is_same<T, MxE4M3>::value) return -1;  // block scales need whole k-steps (host check)
+    else hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, true, kTileT, kWavesN>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
+  }
   if (hipGetLastError() != hipSuccess) return -1;
   if (g.splits > 1)
     return launch_splitk_reduce(g.partial, g, std::is_same<OutT, BF16>::value ? 0 : 1, stream);
@@ -446,6 +502,12 @@ int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, h
     case 2: return out_bf16 ? launch<E4M3, BF16>(g, tile, stream) : launch<E4M3, F16>(g, tile, stream);
   }
   return -1;
+}
+
+// e4m3 operands with block scales in the shuffled layout (g.mx_a, g.mx_b); 256x256 tiles, no K split.
+int launch_tile_ring_mx(const GemmArgs& g, int out_dtype, hipStream_t stream) {
+  if (g.splits != 1 || !g.mx_a || !g.mx_b) return -1;
+  return out_dtype == 0 ? launch_tile<MxE4M3, BF16, 256>(g, stream) : launch_tile<MxE4M3, F16, 256>(g, stream);
 }
 
 }  // namespace mi355

@@ -1,0 +1,120 @@
+// OCP MX block scaling for the fp8 GEMM: the quantiser and the scale shuffle.
+//
+// An MX-quantised matrix X (rows, K), K % 32 == 0, is a pair
+//   x_q     (rows, K)      e4m3 elements
+//   scales  (rows, K/32)   one E8M0 byte per block of 32 consecutive elements of a row,
+//                          value 2^(byte - 127)
+// with X ~= x_q * scale of its block.  The quantiser follows the OCP Microscaling Formats (MX)
+// specification v1.0, section 6.3: the shared exponent of a block is floor(log2(amax)) - 8 (8 is
+// the exponent of the largest e4m3 binade), elements are x / 2^shared rounded to nearest even and
+// saturated at +-448.  A block of zeros gets the scale 1.  NaN and infinity are not supported.
+// The reference has no fp8 path; this is the block-scaled variant of the quantiser in
+// quantize_e4m3.hip, and the format the scaled MFMA of gfx950 consumes.
+//
+// The GEMM kernel reads scales in a "shuffled" layout (gemm_tn_ring.hip: kMxUnitBytes), produced
+// here from the natural row-major one: one 512-byte unit per (group of 128 rows, k-step of 128
+// elements), units ordered [row group][k-step], 8 bytes per lane: byte i of lane l is the scale of
+// row 16*i + l%16 of the group for block 4*kstep + l/16.  Rows are padded to whole 256-row tiles
+// with the scale 1 (their elements read as zeros).
+#include "cdna4_primitives.h"
+#include "gemm_launch.h"
+#include "quantize_convert.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int kMxBlock = 32;
+
+__global__ __launch_bounds__(256) void mx_shuffle_kernel(const uint8_t* __restrict__ scales, int64_t rows,
+                                                         int64_t ld, uint32_t k_steps, uint64_t slots,
+                                                         uint8_t* __restrict__ out) {
+  const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;  // one lane slot of 8 bytes
+  if (id >= slots) return;
+  const uint32_t lane = (uint32_t)(id & 63u);
+  const uint64_t unit = id >> 6;
+  const uint64_t group = unit / k_steps;
+  const uint32_t kstep = (uint32_t)(unit % k_steps);
+  const int64_t block = 4 * (int64_t)kstep + lane / 16;
+  uint32_t w[2] = {0, 0};
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int64_t row = (int64_t)group * 128 + 16 * i + lane % 16;
+    const uint32_t b = row < rows ? scales[row * ld + block] : 127u;
+    w[i / 4] |= b << (8 * (i % 4));
+  }
+  *(u32x2*)(out + id * 8) = (u32x2){w[0], w[1]};
+}
+
+// One thread per block of 32 elements.
+template <class In>
+__global__ __launch_bounds__(256) void mx_quantize_kernel(const void* __restrict__ x, int64_t rows, int64_t blocks_per_row,
+                                                          int64_t ldx, uint8_t* __restrict__ q,
+                                                          uint8_t* __restrict__ scales) {
+  const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (id >= rows * blocks_per_row) return;
+  const int64_t row = id / blocks_per_row, blk = id % blocks_per_row;
+  const int64_t at = row * ldx + blk * kMxBlock;
+  float v[kMxBlock];
+#pragma unroll
+  for (int i = 0; i < kMxBlock; i += 8) Load8<In>::run(x, at + i, v + i);
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < kMxBlock; ++i) amax = __builtin_fmaxf(amax, __builtin_fabsf(v[i]));
+  // floor(log2(amax)) is the exponent field of amax minus 127 (fields below 8, including the
+  // fp32 subnormals, clamp to the smallest scale).
+  const uint32_t field = __builtin_bit_cast(uint32_t, amax) >> 23;
+  const uint32_t byte = amax == 0.f ? 127u : (field > 8u ? field - 8u : 0u);
+  const float inv = __builtin_bit_cast(float, (254u - byte) << 23);  // 2^(127 - byte), exact
+  uint32_t w[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    w[i] = 0;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) w[i] |= to_e4m3(v[4 * i + k] * inv) << (8 * k);
+  }
+  u32x4* dst = (u32x4*)(q + row * blocks_per_row * kMxBlock + blk * kMxBlock);
+  dst[0] = (u32x4){w[0], w[1], w[2], w[3]};
+  dst[1] = (u32x4){w[4], w[5], w[6], w[7]};
+  scales[id] = (uint8_t)byte;
+}
+
+template <class In>
+int run_quantize(const void* x, int64_t rows, int64_t K, int64_t ldx, void* q, uint8_t* scales, hipStream_t stream) {
+  const int64_t n = rows * (K / kMxBlock);
+  if (n == 0) return 0;
+  const int64_t blocks = (n + 255) / 256;
+  if (blocks >= ((int64_t)1 << 31)) return -1;
+  hipLaunchKernelGGL((mx_quantize_kernel<In>), dim3((unsigned)blocks), dim3(256), 0, stream, x, rows, K / kMxBlock, ldx,
+                     (uint8_t*)q, scales);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+}  // namespace
+
+size_t mx_shuffled_bytes(int64_t rows, int64_t K) {
+  if (rows <= 0 || K <= 0) return 0;
+  return (size_t)((rows + 255) / 256 * 256) * (size_t)(K / kMxBlock);
+}
+
+int launch_mx_shuffle(const uint8_t* scales, int64_t rows, int64_t K, int64_t ld, uint8_t* out, hipStream_t stream) {
+  const uint64_t slots = mx_shuffled_bytes(rows, K) / 8;
+  if (slots == 0) return 0;
+  const uint64_t blocks = (slots + 255) / 256;
+  if (blocks >= ((uint64_t)1 << 31)) return -1;
+  hipLaunchKernelGGL(mx_shuffle_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, scales, rows, ld,
+                     (uint32_t)(K / 128), slots, out);
+  return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// in_dtype: 0 bf16, 1 fp16, 3 fp32.
+int launch_quantize_mxfp8(const void* x, int in_dtype, int64_t rows, int64_t K, int64_t ldx, void* q,
+                          uint8_t* scales, hipStream_t stream) {
+  switch (in_dtype) {
+    case 0: return run_quantize<BF16>(x, rows, K, ldx, q, scales, stream);
+    case 1: return run_quantize<F16>(x, rows, K, ldx, q, scales, stream);
+    case 3: return run_quantize<float>(x, rows, K, ldx, q, scales, stream);
+  }
+  return -1;
+}
+
+}  // namespace mi355

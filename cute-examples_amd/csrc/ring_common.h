@@ -35,7 +35,7 @@ __device__ __forceinline__ void static_for(F&& f) {
 template <class T> struct Geo;
 template <> struct Geo<BF16> {
   static constexpr int kBlk = 16, kGroups = 4, kCpl = 1;
-  static constexpr bool kRowSliced = false;
+  static constexpr bool kRowSliced = false, kMx = false;
   typedef i32x4 Frag;
   typedef f32x4 Acc;
   static __device__ __forceinline__ Acc mfma(Frag x, Frag y, Acc c) {
@@ -53,7 +53,7 @@ template <> struct Geo<BF16> {
 };
 template <> struct Geo<F16> {
   static constexpr int kBlk = 16, kGroups = 4, kCpl = 1;
-  static constexpr bool kRowSliced = false;
+  static constexpr bool kRowSliced = false, kMx = false;
   typedef i32x4 Frag;
   typedef f32x4 Acc;
   static __device__ __forceinline__ Acc mfma(Frag x, Frag y, Acc c) {
@@ -66,7 +66,7 @@ template <> struct Geo<F16> {
 };
 template <> struct Geo<E4M3> {
   static constexpr int kBlk = 32, kGroups = 2, kCpl = 2;
-  static constexpr bool kRowSliced = false;
+  static constexpr bool kRowSliced = false, kMx = false;
   typedef i32x8 Frag;
   typedef f32x16 Acc;
   static __device__ __forceinline__ Acc mfma(Frag x, Frag y, Acc c) {
@@ -85,7 +85,7 @@ template <> struct Geo<E4M3> {
 // power limit than 32x32x64, and its 16-wide blocks store 64-byte runs like the 16-bit types.
 struct GeoE4M3Rows {
   static constexpr int kBlk = 16, kGroups = 4, kCpl = 2;
-  static constexpr bool kRowSliced = true;
+  static constexpr bool kRowSliced = true, kMx = false;
   typedef i32x8 Frag;
   typedef f32x4 Acc;
   static __device__ __forceinline__ Acc mfma(Frag x, Frag y, Acc c) {
@@ -93,6 +93,23 @@ struct GeoE4M3Rows {
   }
   static __device__ __forceinline__ void mfma_inplace(Frag x, Frag y, Acc& c) {
     asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));
+  }
+};
+
+// The same shape with OCP MX block scaling: every lane passes, with its fragment, a register that
+// holds the E8M0 scale of its row for one 32-element block of K in the byte picked by kByteX /
+// kByteY (0..3), and the hardware multiplies each block's partial dot product by both scales.
+// Which block a lane's scale applies to fixes the order of K inside the MFMA (measured): the lanes
+// of group g = lane/16 supply bytes [16g, 16g+16) and [64+16g, 64+16g+16) of the 128-byte k-step,
+// and the scale of the lanes of group g applies to bytes [32g, 32g+32), whoever supplied them.
+struct GeoMxE4M3Rows : GeoE4M3Rows {
+  static constexpr bool kMx = true;
+  template <int kByteX, int kByteY>
+  static __device__ __forceinline__ void mfma_scaled_inplace(Frag x, Frag y, Acc& c, uint32_t sx, uint32_t sy) {
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[%5,%6,0] op_sel_hi:[%7,%8,0]"
+                 : "+a"(c)
+                 : "v"(x), "v"(y), "v"(sx), "v"(sy), "n"(kByteX & 1), "n"(kByteY & 1), "n"(kByteX >> 1),
+                   "n"(kByteY >> 1));
   }
 };
 

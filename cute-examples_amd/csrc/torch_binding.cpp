@@ -164,6 +164,82 @@ std::pair<torch::Tensor, torch::Tensor> quantize_e4m3(const torch::Tensor x) {
   return {q, sa[0]};
 }
 
+// Scale bytes of an MX operand: a uint8 (or float8_e8m0fnu) tensor (rows, K/32), rows contiguous.
+const uint8_t* mx_scale_ptr(const torch::Tensor& s, const torch::Tensor& x, const char* name) {
+  TORCH_CHECK(s.scalar_type() == at::kByte || s.scalar_type() == at::kFloat8_e8m0fnu, name,
+              " must be uint8 or float8_e8m0fnu (E8M0 scale bytes)");
+  TORCH_CHECK(s.dim() == 2 && s.size(0) == x.size(0) && s.size(1) * 32 == x.size(1), name,
+              " must have shape (rows, K/32) = (", x.size(0), ", ", x.size(1) / 32, ")");
+  TORCH_CHECK(s.device() == x.device(), "All tensors must be on the same device");
+  TORCH_CHECK(s.size(1) <= 1 || s.stride(1) == 1, name, " must be contiguous in its last dimension");
+  return (const uint8_t*)s.const_data_ptr();
+}
+
+// C = A · B^T for MX-quantised operands: A_q, B_q float8_e4m3fn (M,K), (N,K); scale_a, scale_b
+// E8M0 bytes (M,K/32), (N,K/32); C bf16 or fp16.
+torch::Tensor gemm_tn_mxfp8(const torch::Tensor A_q, const torch::Tensor B_q, const torch::Tensor scale_a,
+                            const torch::Tensor scale_b, torch::Tensor C) {
+  TORCH_CHECK(A_q.device() == B_q.device(), "All tensors must be on the same device");
+  TORCH_CHECK(A_q.is_contiguous() && B_q.is_contiguous(), "All tensors must be contiguous");
+  TORCH_CHECK(A_q.dim() == 2 && B_q.dim() == 2, "Both tensors must be 2D (matrix) tensors");
+  TORCH_CHECK(A_q.size(1) == B_q.size(1), "Inner dimensions of A and B must match (A: ", A_q.size(1),
+              ", B: ", B_q.size(1), ")");
+  TORCH_CHECK(A_q.scalar_type() == at::kFloat8_e4m3fn && B_q.scalar_type() == at::kFloat8_e4m3fn,
+              "Both tensors must be of type float8_e4m3fn");
+  const int64_t M = A_q.size(0), N = B_q.size(0), K = A_q.size(1);
+  TORCH_CHECK(K % 32 == 0, "K must be a multiple of the MX block (32); the kernel needs K % 128 == 0");
+  TORCH_CHECK(C.dim() == 2 && C.size(0) == M && C.size(1) == N, "C must have shape (", M, ", ", N, ")");
+  TORCH_CHECK(C.device() == A_q.device(), "All tensors must be on the same device");
+  const int out_dt = dtype_code(C.scalar_type());
+  TORCH_CHECK(out_dt == MI355_BF16 || out_dt == MI355_F16, "C must be bfloat16 or float16");
+  TORCH_CHECK(N <= 1 || C.stride(1) == 1, "C must be contiguous in its last dimension");
+  const int64_t ldc = M > 1 ? C.stride(0) : N;
+  const uint8_t* sa = mx_scale_ptr(scale_a, A_q, "scale_a");
+  const uint8_t* sb = mx_scale_ptr(scale_b, B_q, "scale_b");
+  int st = mi355_gemm_mx_check(M, N, K, K, K, ldc, out_dt);
+  TORCH_CHECK(st == MI355_OK, "gemm_kernels: ", mi355_gemm_strerror(st), " [mxfp8 M=", M, " N=", N, " K=", K, "]");
+  TORCH_CHECK(A_q.is_cuda(), "gemm_kernels runs on a HIP device only; got tensors on ", A_q.device());
+  if (M == 0 || N == 0) return C;
+  c10::DeviceGuard guard(A_q.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStream(A_q.device().index()).stream();
+  const size_t ws_bytes = mi355_gemm_mx_workspace_bytes(M, N, K, 0);
+  torch::Tensor ws;
+  void* ws_ptr = nullptr;
+  if (ws_bytes) {
+    ws = torch::empty({(int64_t)ws_bytes}, A_q.options().dtype(torch::kUInt8));
+    ws_ptr = ws.data_ptr();
+  }
+  st = mi355_gemm_tn_mxfp8(A_q.const_data_ptr(), B_q.const_data_ptr(), C.mutable_data_ptr(), M, N, K, K, K, ldc, sa,
+                           M > 1 ? scale_a.stride(0) : K / 32, sb, N > 1 ? scale_b.stride(0) : K / 32, 0, out_dt,
+                           ws_ptr, ws_bytes, (void*)stream);
+  TORCH_CHECK(st == MI355_OK, "gemm_kernels: ", mi355_gemm_strerror(st));
+  return C;
+}
+
+// (x_q, scales): x (rows, K) -> float8_e4m3fn (rows, K) and uint8 E8M0 scale bytes (rows, K/32),
+// one per 32 consecutive elements of a row, x ~= x_q * 2^(scales - 127).
+std::pair<torch::Tensor, torch::Tensor> quantize_mxfp8(const torch::Tensor x) {
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous(), "x must be a contiguous 2D tensor");
+  int dt;
+  switch (x.scalar_type()) {
+    case at::kBFloat16: dt = MI355_BF16; break;
+    case at::kHalf: dt = MI355_F16; break;
+    case at::kFloat: dt = MI355_F32; break;
+    default: TORCH_CHECK(false, "x must be bfloat16, float16 or float32");
+  }
+  const int64_t rows = x.size(0), K = x.size(1);
+  TORCH_CHECK(K % 32 == 0, "the last dimension must be a multiple of the MX block (32)");
+  TORCH_CHECK(x.is_cuda(), "gemm_kernels runs on a HIP device only; got a tensor on ", x.device());
+  c10::DeviceGuard guard(x.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+  torch::Tensor q = torch::empty({rows, K}, x.options().dtype(at::kFloat8_e4m3fn));
+  torch::Tensor sc = torch::empty({rows, K / 32}, x.options().dtype(at::kByte));
+  int st = mi355_quantize_mxfp8(x.const_data_ptr(), dt, rows, K, K, q.mutable_data_ptr(), sc.data_ptr<uint8_t>(),
+                                (void*)stream);
+  TORCH_CHECK(st == MI355_OK, "gemm_kernels: ", mi355_gemm_strerror(st));
+  return {q, sc};
+}
+
 std::string select_variant(int64_t M, int64_t N, int64_t K, at::ScalarType dtype) {
   const int dt = dtype_code(dtype);
   TORCH_CHECK(dt >= 0, "dtype must be bfloat16, float16 or float8_e4m3fn");
@@ -187,6 +263,11 @@ PYBIND11_MODULE(_C, m) {
   m.def("quantize_e4m3", &test::quantize_e4m3,
         "per-tensor fp8 quantisation on the device: returns (x_q float8_e4m3fn, scale 0-dim fp32 tensor)",
         py::arg("x"));
+  m.def("gemm_tn_mxfp8", &test::gemm_tn_mxfp8,
+        "C = A @ B.T for MX block-scaled float8_e4m3fn operands (one E8M0 scale byte per 32 elements of K)",
+        py::arg("A_q"), py::arg("B_q"), py::arg("scale_a"), py::arg("scale_b"), py::arg("C"));
+  m.def("quantize_mxfp8", &test::quantize_mxfp8,
+        "MX quantisation on the device: returns (x_q float8_e4m3fn, scales uint8 (rows, K/32))", py::arg("x"));
   m.def("select_variant", &test::select_variant, py::arg("M"), py::arg("N"), py::arg("K"),
         py::arg("dtype"));
   m.def("version", []() { return mi355_gemm_version(); });

@@ -8,6 +8,8 @@ Same package name and entry point as the reference (kernels/gemm_kernels/__init_
 plus the variant-selecting and fp8 entry points of the native module.  The native module is
 required: importing this package without a built gemm_kernels/_C*.so raises ImportError.
 """
-from ._C import gemm_tn, gemm_tn_fp8, gemm_tn_test, quantize_e4m3, select_variant, version
+from ._C import (gemm_tn, gemm_tn_fp8, gemm_tn_mxfp8, gemm_tn_test, quantize_e4m3, quantize_mxfp8,
+                 select_variant, version)
 
-__all__ = ["gemm_tn_test", "gemm_tn", "gemm_tn_fp8", "quantize_e4m3", "select_variant", "version"]
+__all__ = ["gemm_tn_test", "gemm_tn", "gemm_tn_fp8", "gemm_tn_mxfp8", "quantize_e4m3", "quantize_mxfp8",
+           "select_variant", "version"]

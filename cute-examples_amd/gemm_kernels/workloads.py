@@ -9,13 +9,14 @@ B (N,K).  Shapes and distributions:
   skinny        bf16, activations X (M,K) Normal(0,1), weights W (N,K) Normal(0,0.02),
                 M in {16,64,256}, (N,K) in {(14336,4096),(4096,14336),(6144,4096)}
   fp8_8192      e4m3, M=N=K=8192, quantised from Normal(0,1) with per-tensor scales amax/448
+  mxfp8_8192    e4m3 + E8M0 block scales (OCP MX), M=N=K=8192, quantised from Normal(0,1)
 
 The reference's own test draws unseeded torch.randn bf16 squares of side 4096/2048/1024
 (kernels/tests/gemm_test.py:15,23-24); `reference_test_shapes` keeps that list.
 """
 import torch
 
-from .quant import quantize_e4m3
+from .quant import quantize_e4m3, quantize_mxfp8
 
 reference_test_shapes = [(4096, 4096), (2048, 2048), (1024, 1024)]
 
@@ -68,3 +69,13 @@ def fp8_8192(seed=0, device="cpu", size=8192):
     b = normal((size, size), seed + 1, device, dtype=torch.float32)
     b_q, sb = quantize_e4m3(b)
     return a_q, b_q, sa, sb
+
+
+def mxfp8_8192(seed=0, device="cpu", size=8192):
+    """(A_q, scale_a, B_q, scale_b): float8_e4m3fn operands with uint8 E8M0 block scales (rows, K/32)."""
+    a = normal((size, size), seed, device, dtype=torch.float32)
+    a_q, sa = quantize_mxfp8(a)
+    del a
+    b = normal((size, size), seed + 1, device, dtype=torch.float32)
+    b_q, sb = quantize_mxfp8(b)
+    return a_q, sa, b_q, sb

@@ -111,6 +111,63 @@ int mi355_gemm_tn_scaled(const void *A, const void *B, void *C,
 int mi355_quantize_e4m3(const void *x, int x_dtype, int64_t n, void *x_q,
                         float *scale_amax, void *stream);
 
+/*
+ * OCP MX block scaling (MXFP8): C = A · B^T where every block of 32 consecutive elements of a row
+ * of A or of B shares one E8M0 scale byte (value 2^(byte-127)):
+ *   A[m,k] = A_q[m,k] * 2^(scale_a[m, k/32] - 127),  A_q e4m3; the same for B.
+ * The block scales are applied by the scaled matrix-core instruction of gfx950 inside the k loop.
+ *
+ *   scale_a, scale_b   device pointers to the scale bytes.  With scales_shuffled == 0 they are in
+ *                      the natural layout, (M, K/32) and (N, K/32) row-major with row strides
+ *                      ld_scale_a / ld_scale_b (bytes); the call then re-lays them into the
+ *                      workspace first (one small kernel per operand).  With scales_shuffled == 1
+ *                      they are the output of mi355_mx_shuffle_scales (ld_scale_* ignored) and no
+ *                      workspace is needed: do this once for weights.
+ *   workspace          at least mi355_gemm_mx_workspace_bytes(M, N, K, scales_shuffled) bytes,
+ *                      16-byte aligned.
+ * Constraints: K % 128 == 0; A, B 16-byte aligned with row strides that are multiples of 16;
+ * N % 4 == 0, ldc % 4 == 0, C 8-byte aligned; the size limits of the tiled variants.  Always runs
+ * the 256x256-tile kernel (MI355_VARIANT_BASIC) without a K split.
+ * Counterpart in the reference: none (it has no fp8 path); same launcher contract as
+ * mi355_gemm_tn (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92), block format per the OCP
+ * Microscaling Formats (MX) specification v1.0.
+ */
+int mi355_gemm_tn_mxfp8(const void *A_q, const void *B_q, void *C,
+                        int64_t M, int64_t N, int64_t K,
+                        int64_t lda, int64_t ldb, int64_t ldc,
+                        const uint8_t *scale_a, int64_t ld_scale_a,
+                        const uint8_t *scale_b, int64_t ld_scale_b,
+                        int scales_shuffled, int out_dtype,
+                        void *workspace, size_t workspace_bytes, void *stream);
+
+/* Workspace mi355_gemm_tn_mxfp8 needs (0 when the scales are already shuffled). */
+size_t mi355_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int scales_shuffled);
+
+/* Argument check of mi355_gemm_tn_mxfp8 without pointers; runs without a GPU. */
+int mi355_gemm_mx_check(int64_t M, int64_t N, int64_t K,
+                        int64_t lda, int64_t ldb, int64_t ldc, int out_dtype);
+
+/*
+ * Re-lay the scale bytes of one operand, (rows, K/32) row-major with row stride ld bytes, into
+ * the layout the kernel reads: `out` receives mi355_mx_shuffled_bytes(rows, K) bytes (rows padded
+ * to a multiple of 256 with the scale 1).  K % 128 == 0; out 8-byte aligned.
+ * Counterpart in the reference: none.
+ */
+int mi355_mx_shuffle_scales(const uint8_t *scales, int64_t rows, int64_t K, int64_t ld,
+                            uint8_t *out, void *stream);
+size_t mi355_mx_shuffled_bytes(int64_t rows, int64_t K);
+
+/*
+ * MX quantiser: x (rows, K) of x_dtype (BF16, F16 or F32), row stride ldx elements, K % 32 == 0
+ * -> x_q (rows, K) contiguous e4m3 and scales (rows, K/32) contiguous E8M0 bytes in the natural
+ * layout.  Per block: scale = 2^(floor(log2(amax)) - 8) (1 for a block of zeros), elements
+ * x/scale rounded to nearest even, saturated at +-448.  x 16-byte aligned with ldx*elem_bytes
+ * % 16 == 0, x_q 16-byte aligned.  NaN and infinity are not supported.
+ * Counterpart in the reference: none; OCP MX specification v1.0, section 6.3.
+ */
+int mi355_quantize_mxfp8(const void *x, int x_dtype, int64_t rows, int64_t K, int64_t ldx,
+                         void *x_q, uint8_t *scales, void *stream);
+
 /* Scratch bytes mi355_gemm_tn needs for this problem and variant (0 for most shapes).
  * Counterpart: none in the reference (it has no split-K); sizes the split-K partials that
  * replace the reference's single-pass accumulation (gemm.cuh:352-367) on skinny shapes. */

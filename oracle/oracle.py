@@ -132,3 +132,45 @@ def quantize_e4m3(x):
     scale = np.float32(amax) / np.float32(448.0) if amax > 0 else np.float32(1.0)
     q = c_round((x.numpy() / scale).astype(np.float32), E4M3)
     return torch.from_numpy(q).view(torch.float8_e4m3fn).reshape(x.shape), float(scale)
+
+
+# --- OCP MX block scaling (MXFP8) -----------------------------------------------------------------
+# The reference has no fp8 path; these restate the published format (OCP Microscaling Formats (MX)
+# specification v1.0: section 5.1 block = 32 elements sharing an E8M0 scale 2^(byte-127); section
+# 6.3 conversion: shared exponent floor(log2(amax)) - emax_elem, emax_elem = 8 for e4m3, elements
+# x / scale rounded to nearest even and saturated).  Pinned in tests/test_oracle.py by closed-form
+# blocks, torch's float8_e8m0fnu / float8_e4m3fn decoders and an exact rational brute force.
+
+MX_BLOCK = 32
+E4M3_EMAX = 8
+
+
+def quantize_mxfp8(x):
+    """x (rows, K) float tensor, K % 32 == 0 -> (x_q float8_e4m3fn (rows, K), scales uint8 (rows, K/32))."""
+    x = x.detach().cpu().float().contiguous()
+    rows, K = x.shape
+    assert K % MX_BLOCK == 0
+    blocks = x.numpy().reshape(rows, K // MX_BLOCK, MX_BLOCK).astype(np.float64)
+    amax = np.abs(blocks).max(axis=-1)
+    with np.errstate(divide="ignore"):
+        shared = np.floor(np.log2(amax)) - E4M3_EMAX          # -inf for a block of zeros
+    byte = np.where(amax > 0, np.clip(shared + 127, 0, 254), 127).astype(np.int64)
+    scaled = blocks * np.exp2(127.0 - byte)[..., None]          # exact: a power of two
+    q = c_round(scaled.astype(np.float32).reshape(rows, K), E4M3)
+    return (torch.from_numpy(q).view(torch.float8_e4m3fn).reshape(rows, K),
+            torch.from_numpy(byte.astype(np.uint8)))
+
+
+def dequantize_mxfp8(x_q, scales):
+    """(float8_e4m3fn (rows, K), uint8 (rows, K/32)) -> float32 (rows, K), exact."""
+    rows, K = x_q.shape
+    vals = c_decode(x_q.detach().cpu().contiguous().view(torch.uint8).numpy(), E4M3).astype(np.float64)
+    s = np.exp2(scales.detach().cpu().view(torch.uint8).numpy().astype(np.float64) - 127.0)
+    out = vals.reshape(rows, K // MX_BLOCK, MX_BLOCK) * s[..., None]
+    return torch.from_numpy(out.reshape(rows, K).astype(np.float32))
+
+
+def gemm_tn_mxfp8_fp32(A_q, scale_a, B_q, scale_b):
+    """Ground truth of the block-scaled GEMM: fp32 matmul of the dequantised operands
+    (the reference test's ground truth, gemm_test.py:36, applied to what the operands mean)."""
+    return torch.matmul(dequantize_mxfp8(A_q, scale_a), dequantize_mxfp8(B_q, scale_b).T)

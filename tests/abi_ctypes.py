@@ -31,6 +31,19 @@ def load():
     L.mi355_gemm_tn_scaled.restype = ci
     L.mi355_quantize_e4m3.argtypes = [vp, ci, i64, vp, vp, vp]
     L.mi355_quantize_e4m3.restype = ci
+    u8p = vp
+    L.mi355_gemm_tn_mxfp8.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, u8p, i64, u8p, i64, ci, ci, vp, sz, vp]
+    L.mi355_gemm_tn_mxfp8.restype = ci
+    L.mi355_gemm_mx_workspace_bytes.argtypes = [i64, i64, i64, ci]
+    L.mi355_gemm_mx_workspace_bytes.restype = sz
+    L.mi355_gemm_mx_check.argtypes = [i64, i64, i64, i64, i64, i64, ci]
+    L.mi355_gemm_mx_check.restype = ci
+    L.mi355_mx_shuffle_scales.argtypes = [u8p, i64, i64, i64, u8p, vp]
+    L.mi355_mx_shuffle_scales.restype = ci
+    L.mi355_mx_shuffled_bytes.argtypes = [i64, i64]
+    L.mi355_mx_shuffled_bytes.restype = sz
+    L.mi355_quantize_mxfp8.argtypes = [vp, ci, i64, i64, i64, vp, u8p, vp]
+    L.mi355_quantize_mxfp8.restype = ci
     L.mi355_gemm_workspace_bytes.argtypes = [i64, i64, i64, ci, ci]
     L.mi355_gemm_workspace_bytes.restype = sz
     L.mi355_gemm_select_variant.argtypes = [i64, i64, i64, ci]
@@ -64,3 +77,28 @@ def gemm_tn(L, A, B, C, scale=1.0, variant=AUTO, stream=None):
                          C.stride(0), in_dt, out_dt, scale, variant,
                          ws.data_ptr() if ws is not None else None, ws_bytes, s)
     return rc
+
+
+def gemm_tn_mxfp8(L, A_q, B_q, sa, sb, C, shuffled=False, stream=None):
+    """Call mi355_gemm_tn_mxfp8 on torch device tensors.  With shuffled=True the scales are first
+    re-laid with mi355_mx_shuffle_scales (as a caller would do once for weights)."""
+    import torch
+    M, K = A_q.shape
+    N = B_q.shape[0]
+    s = stream if stream is not None else torch.cuda.current_stream().cuda_stream
+    out_dt = torch_code(C.dtype)
+    if shuffled:
+        pa = torch.empty(max(L.mi355_mx_shuffled_bytes(M, K), 8), dtype=torch.uint8, device=A_q.device)
+        pb = torch.empty(max(L.mi355_mx_shuffled_bytes(N, K), 8), dtype=torch.uint8, device=A_q.device)
+        rc = L.mi355_mx_shuffle_scales(sa.data_ptr(), M, K, sa.stride(0), pa.data_ptr(), s)
+        rc = rc or L.mi355_mx_shuffle_scales(sb.data_ptr(), N, K, sb.stride(0), pb.data_ptr(), s)
+        if rc:
+            return rc
+        return L.mi355_gemm_tn_mxfp8(A_q.data_ptr(), B_q.data_ptr(), C.data_ptr(), M, N, K, A_q.stride(0),
+                                     B_q.stride(0), C.stride(0), pa.data_ptr(), 0, pb.data_ptr(), 0, 1, out_dt,
+                                     None, 0, s)
+    ws_bytes = L.mi355_gemm_mx_workspace_bytes(M, N, K, 0)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=A_q.device)
+    return L.mi355_gemm_tn_mxfp8(A_q.data_ptr(), B_q.data_ptr(), C.data_ptr(), M, N, K, A_q.stride(0),
+                                 B_q.stride(0), C.stride(0), sa.data_ptr(), sa.stride(0), sb.data_ptr(),
+                                 sb.stride(0), 0, out_dt, ws.data_ptr(), ws_bytes, s)

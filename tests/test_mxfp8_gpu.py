@@ -1,0 +1,199 @@
+"""MX block-scaled fp8 GEMM and its quantiser on the GPU, through the C ABI and the Python module,
+against the oracle's restatement of the OCP MX format.
+
+Tolerance: relative Frobenius error <= 3e-2 against the fp32 product of the dequantised operands
+(in practice ~2e-3: the products and block scales are exact, only the fp32 accumulation order and
+the bf16/fp16 output rounding differ); the quantiser, the power-of-two cases and the permutation
+case are bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle
+from tests import abi_ctypes as ac
+
+pytestmark = pytest.mark.gpu
+
+TOL = 3e-2
+
+
+def random_mx(rows, K, seed, scale_lo=112, scale_hi=142):
+    """Random e4m3 bytes (no NaN codes) and random scale bytes: every byte pattern, a wide range of scales."""
+    rng = np.random.default_rng(seed)
+    bits = rng.integers(0, 256, size=(rows, K), dtype=np.uint8)
+    bits[(bits & 0x7f) == 0x7f] ^= 0x08
+    sc = rng.integers(scale_lo, scale_hi, size=(rows, K // 32), dtype=np.uint8)
+    return torch.from_numpy(bits).view(torch.float8_e4m3fn), torch.from_numpy(sc)
+
+
+def run_mx(abi, A, sa, B, sb, out_dtype=torch.bfloat16, shuffled=False, ldc=None):
+    M, N = A.shape[0], B.shape[0]
+    guard = 8
+    Cfull = torch.full((M + guard, ldc or N), float("nan"), dtype=out_dtype, device="cuda")
+    C = Cfull[:M, :N]
+    rc = ac.gemm_tn_mxfp8(abi, A.cuda(), B.cuda(), sa.cuda(), sb.cuda(), C, shuffled)
+    assert rc == 0, abi.mi355_gemm_strerror(rc)
+    torch.cuda.synchronize()
+    assert torch.isnan(Cfull[M:].float()).all(), "wrote behind the M rows of C"
+    if ldc:
+        assert torch.isnan(Cfull[:M, N:].float()).all(), "wrote outside the N columns of C"
+    return C.cpu()
+
+
+def check(C, A, sa, B, sb):
+    ref = oracle.gemm_tn_mxfp8_fp32(A, sa, B, sb)
+    assert oracle.no_nan_left(C)
+    err = oracle.rel_frobenius(C, ref)
+    assert err <= TOL, err
+    return err, ref
+
+
+@pytest.mark.parametrize("shuffled", [False, True])
+@pytest.mark.parametrize("shape", [(256, 256, 128), (256, 256, 1024), (512, 768, 640), (1024, 1024, 2048)])
+def test_random_bytes_and_scales(abi, shape, shuffled):
+    M, N, K = shape
+    A, sa = random_mx(M, K, 1)
+    B, sb = random_mx(N, K, 2)
+    C = run_mx(abi, A, sa, B, sb, shuffled=shuffled)
+    err, _ = check(C, A, sa, B, sb)
+    assert err < 5e-3
+
+
+@pytest.mark.parametrize("shape", [(100, 260, 256), (257, 255 * 4, 384), (1, 4, 128), (300, 516, 128), (640, 128, 1152),
+                                   (129, 132, 512)])
+def test_ragged_tiles(abi, shape):
+    """M and N that do not fill the 256-row tiles or the 128-row scale groups; padded C rows."""
+    M, N, K = shape
+    A, sa = random_mx(M, K, 3)
+    B, sb = random_mx(N, K, 4)
+    C = run_mx(abi, A, sa, B, sb, ldc=N + 12)
+    check(C, A, sa, B, sb)
+
+
+def test_each_scale_byte_reaches_its_block_only(abi):
+    """All elements 1, all scales 1 except ONE (row, block) of A doubled: exactly row m changes, by
+    exactly +32 per column, for every position of the block in the k-step, the scale group and the
+    k-step.  Pins the shuffle and which lane's byte the matrix core applies to which 32 elements."""
+    M = N = 256
+    K = 384
+    ones = torch.ones(M, K).to(torch.float8_e4m3fn)
+    base = torch.full((M, K // 32), 127, dtype=torch.uint8)
+    for m, blk in [(0, 0), (5, 1), (17, 2), (130, 3), (255, 11), (64, 6), (127, 9), (200, 4)]:
+        sa = base.clone()
+        sa[m, blk] = 128
+        C = run_mx(abi, ones, sa, ones, base).float()
+        want = torch.full((M, N), float(K))
+        want[m, :] += 32.0
+        assert torch.equal(C, want), (m, blk)
+        C = run_mx(abi, ones, base, ones, sa).float()      # and on the B side: column m
+        assert torch.equal(C, want.t()), (m, blk)
+
+
+def test_block_order_inside_a_k_step(abi):
+    """Elements of ONE 32-element block are 1, the rest 0, and that block's scale is 2^3: the result
+    is 32*8 only if the kernel pairs the block's elements with the block's own scale."""
+    M = N = 256
+    K = 256
+    base = torch.full((M, K // 32), 127, dtype=torch.uint8)
+    ones = torch.ones(N, K).to(torch.float8_e4m3fn)
+    for blk in range(K // 32):
+        A = torch.zeros(M, K)
+        A[:, 32 * blk:32 * blk + 32] = 1.0
+        sa = base.clone()
+        sa[:, blk] = 130
+        C = run_mx(abi, A.to(torch.float8_e4m3fn), sa, ones, base).float()
+        assert torch.all(C == 256.0), blk
+
+
+def test_permutation_is_exact(abi):
+    """B = permutation with power-of-two block scales: C[m][n] = A[m][perm[n]] * scales, exactly."""
+    M = N = K = 512
+    A, sa = random_mx(M, K, 5, 125, 130)
+    perm = torch.randperm(K, generator=torch.Generator().manual_seed(6))
+    P = torch.zeros(N, K)
+    P[torch.arange(N), perm] = 1.0
+    sb = torch.from_numpy(np.random.default_rng(7).integers(125, 130, size=(N, K // 32), dtype=np.uint8))
+    C = run_mx(abi, A, sa, P.to(torch.float8_e4m3fn), sb)
+    want = oracle.gemm_tn_mxfp8_fp32(A, sa, P.to(torch.float8_e4m3fn), sb)
+    assert torch.equal(C.view(torch.int16), (want + 0.0).to(torch.bfloat16).view(torch.int16))
+
+
+def test_scale_shift_is_exact(abi):
+    """Adding 1 to every scale byte of A doubles C exactly (bf16 scaling by 2 is exact)."""
+    M, N, K = 512, 512, 1024
+    A, sa = random_mx(M, K, 8, 120, 130)
+    B, sb = random_mx(N, K, 9, 120, 130)
+    C1 = run_mx(abi, A, sa, B, sb).float()
+    C2 = run_mx(abi, A, sa + 1, B, sb).float()
+    assert torch.equal(C2, 2 * C1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_quantizer_is_bit_exact(abi, dtype):
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(300, 1024, generator=g) * torch.exp2(torch.randint(-12, 12, (300, 1), generator=g).float())
+    x[7, 64:96] = 0.0                       # a block of zeros
+    x[8, :32] = 448.0
+    x[9, 32:64] = torch.linspace(-500, 500, 32)
+    x = x.to(dtype)
+    q = torch.empty(x.shape, dtype=torch.uint8, device="cuda")
+    sc = torch.empty(x.shape[0], x.shape[1] // 32, dtype=torch.uint8, device="cuda")
+    xd = x.cuda()
+    code = {torch.bfloat16: ac.BF16, torch.float16: ac.F16, torch.float32: ac.F32}[dtype]
+    rc = abi.mi355_quantize_mxfp8(xd.data_ptr(), code, x.shape[0], x.shape[1], xd.stride(0), q.data_ptr(), sc.data_ptr(),
+                                  torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    want_q, want_s = oracle.quantize_mxfp8(x)
+    assert torch.equal(sc.cpu(), want_s)
+    assert torch.equal(q.cpu(), want_q.view(torch.uint8))
+
+
+def test_end_to_end_from_bf16(abi):
+    """quantise -> block-scaled GEMM against the fp32 product of the ORIGINAL operands: the error is
+    the quantisation's (e4m3 keeps 4 significant bits: ~2.7e-2 per element, averaging down over K)."""
+    import gemm_kernels
+    g = torch.Generator().manual_seed(20)
+    # per-row magnitudes spread over 2^+-6: what block scaling is for
+    A = (torch.randn(512, 2048, generator=g) * torch.exp2(torch.randint(-6, 6, (512, 1), generator=g).float())).bfloat16()
+    B = (torch.randn(768, 2048, generator=g) * torch.exp2(torch.randint(-6, 6, (768, 1), generator=g).float())).bfloat16()
+    Aq, sa = gemm_kernels.quantize_mxfp8(A.cuda())
+    Bq, sb = gemm_kernels.quantize_mxfp8(B.cuda())
+    C = torch.full((512, 768), float("nan"), dtype=torch.bfloat16, device="cuda")
+    out = gemm_kernels.gemm_tn_mxfp8(Aq, Bq, sa, sb, C)
+    assert out.data_ptr() == C.data_ptr()
+    torch.cuda.synchronize()
+    check(C.cpu(), Aq.cpu(), sa.cpu(), Bq.cpu(), sb.cpu())
+    err = oracle.rel_frobenius(C.cpu(), oracle.gemm_tn_fp32(A, B))
+    assert err <= 5e-2, err
+
+
+def test_full_size_properties(abi):
+    """8192^3: the sampled rows against the oracle, and linearity in the scales."""
+    from gemm_kernels import workloads
+    A, sa, B, sb = workloads.mxfp8_8192(seed=0, device="cuda")
+    C = torch.full((8192, 8192), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert ac.gemm_tn_mxfp8(abi, A, B, sa, sb, C) == 0
+    torch.cuda.synchronize()
+    assert not torch.isnan(C.float()).any()
+    rows = torch.tensor([0, 1, 127, 128, 255, 256, 4095, 4096, 8191])
+    ref = oracle.gemm_tn_mxfp8_fp32(A[rows].cpu(), sa[rows].cpu(), B.cpu(), sb.cpu())
+    assert oracle.rel_frobenius(C[rows].cpu(), ref) <= TOL
+    C2 = torch.empty_like(C)
+    assert ac.gemm_tn_mxfp8(abi, A, B, sa + 2, sb - 1, C2) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(C2.float(), 2 * C.float())
+
+
+def test_rejects_bad_arguments(abi):
+    assert abi.mi355_gemm_mx_check(256, 256, 64, 64, 64, 256, ac.BF16) == ac.ERR_SHAPE      # K % 128
+    A, sa = random_mx(256, 128, 1)
+    C = torch.empty(256, 256, dtype=torch.bfloat16, device="cuda")
+    Ad, sad = A.cuda(), sa.cuda()
+    s = torch.cuda.current_stream().cuda_stream
+    rc = abi.mi355_gemm_tn_mxfp8(Ad.data_ptr(), Ad.data_ptr(), C.data_ptr(), 256, 256, 128, 128, 128, 256, sad.data_ptr(), 4,
+                                 sad.data_ptr(), 4, 0, ac.BF16, None, 0, s)
+    assert rc == ac.ERR_WORKSPACE
+    rc = abi.mi355_gemm_tn_mxfp8(Ad.data_ptr(), Ad.data_ptr(), C.data_ptr(), 256, 256, 128, 128, 128, 256, None, 4,
+                                 sad.data_ptr(), 4, 0, ac.BF16, None, 0, s)
+    assert rc == ac.ERR_NULL

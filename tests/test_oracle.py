@@ -154,3 +154,94 @@ def test_metrics():
     assert oracle.reference_accepts(label + 0.009, label)
     assert not oracle.reference_accepts(label + 0.2, label)
     assert oracle.no_nan_left(label) and not oracle.no_nan_left(label / torch.tensor(0.0) * 0)
+
+
+# --- MX block scaling ------------------------------------------------------------------------------
+
+def test_mx_quantizer_closed_forms():
+    """Blocks whose quantisation the format fixes by hand (OCP MX v1.0, 6.3)."""
+    x = torch.zeros(4, 64)
+    x[0, :32] = torch.tensor([2.0 ** k for k in range(-10, 22)])       # amax 2^21 -> shared exp 13
+    x[0, 32:] = 0.0                                                     # zeros -> scale 1
+    x[1, :32] = 448.0                                                   # amax 448 -> 2^0, elements 448
+    x[1, 32:] = torch.linspace(-500.0, 500.0, 32)                       # amax 500 -> 2^0, |x|>448 saturates
+    x[2, :32] = 1.0
+    x[2, 32] = 3.0e-5                                                   # floor(log2)=-16 -> shared -24
+    x[3, 0] = -255.9999                                                 # amax in [128,256) -> 2^-1
+    q, s = oracle.quantize_mxfp8(x)
+    qf = q.float()
+    assert s[0, 0] == 127 + 13 and s[0, 1] == 127
+    # elements 2^k / 2^13 for k = -10..21: below 2^-9 they vanish or hit the subnormal grid
+    want = torch.tensor([2.0 ** (k - 13) for k in range(-10, 22)])
+    want[want < 2.0 ** -10] = 0.0
+    want[(want >= 2.0 ** -10) & (want < 2.0 ** -9)] = 0.0              # 2^-10 is a tie between 0 and 2^-9 -> even (0)
+    assert torch.equal(qf[0, :32], want)
+    assert s[1, 0] == 127 and torch.all(qf[1, :32] == 448.0)
+    assert s[1, 1] == 127 and qf[1, 32] == -448.0 and qf[1, 63] == 448.0
+    assert s[2, 0] == 127 - 8 and torch.all(qf[2, :32] == 256.0)
+    assert s[2, 1] == 127 - 24 and qf[2, 32] == 448.0                  # 3e-5 * 2^24 = 503.3 saturates
+    assert s[3, 0] == 127 - 1 and qf[3, 0] == -448.0                   # 511.9998 saturates
+
+
+def test_mx_scale_and_element_decoders_match_torch():
+    """The byte -> value maps against torch's own float8_e8m0fnu and float8_e4m3fn decoders."""
+    b = torch.arange(0, 255, dtype=torch.uint8)                         # 255 is NaN in E8M0
+    want = b.view(torch.float8_e8m0fnu).float().double()
+    q = torch.full((255, 32), 1.0).to(torch.float8_e4m3fn)
+    got = oracle.dequantize_mxfp8(q, b.reshape(255, 1)).double()[:, 0]
+    ok = want >= 2.0 ** -126                                            # fp32 output: the smallest scales are subnormal
+    assert torch.equal(got[ok], want[ok])
+    rng = np.random.default_rng(3)
+    bits = rng.integers(0, 256, size=(8, 64), dtype=np.uint8)
+    bits[(bits & 0x7f) == 0x7f] = 0
+    qq = torch.from_numpy(bits).view(torch.float8_e4m3fn)
+    sc = torch.from_numpy(rng.integers(110, 140, size=(8, 2), dtype=np.uint8))
+    want = qq.float().reshape(8, 2, 32) * sc.view(torch.float8_e8m0fnu).float()[..., None]
+    assert torch.equal(oracle.dequantize_mxfp8(qq, sc), want.reshape(8, 64))
+
+
+def test_mx_quantizer_invariants():
+    """Properties the conversion must have whatever the data: the largest element of every block
+    lands in the top binade [256, 448], scaling a block by 2^k moves only the scale byte, and the
+    round trip stays within half an e4m3 ulp of the block's top binade (2^-4 of 2^(e+8)... ) except
+    where saturation (amax in (448, 512) * 2^e) applies."""
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(64, 256, generator=g) * torch.exp2(torch.randint(-20, 20, (64, 1), generator=g).float())
+    q, s = oracle.quantize_mxfp8(x)
+    top = q.float().abs().reshape(64, 8, 32).amax(-1)
+    assert torch.all((top >= 256.0) & (top <= 448.0))
+    q2, s2 = oracle.quantize_mxfp8(x * 8.0)
+    assert torch.equal(q2.view(torch.uint8), q.view(torch.uint8)) and torch.equal(s2, s + 3)
+    back = oracle.dequantize_mxfp8(q, s)
+    unit = torch.exp2(s.float() - 127.0).repeat_interleave(32, dim=1)    # value of one unit of x/scale
+    err = (back - x).abs() / unit
+    scaled = (x / unit).abs()
+    assert torch.all(err[scaled <= 448.0] <= 16.0 + 1e-3)                # half an ulp of [256, 512): 32/2
+    assert torch.all(err[scaled > 448.0] <= 64.0)                        # saturated from below 512
+    # e4m3 keeps 4 significant bits: relative error of normal values <= 2^-4
+    normal = scaled >= 2.0 ** -6
+    assert torch.all(((back - x).abs() / x.abs())[normal & (scaled <= 448.0)] <= 2.0 ** -4 + 1e-6)
+
+
+def test_mx_gemm_bruteforce_exact():
+    """The block-scaled product against exact rational arithmetic on a tiny case."""
+    from fractions import Fraction
+    rng = np.random.default_rng(11)
+    M, N, K = 3, 4, 64
+    def operand(rows):
+        bits = rng.integers(0, 256, size=(rows, K), dtype=np.uint8)
+        bits[(bits & 0x7f) == 0x7f] = 0x30
+        bits[(bits & 0x78) > 0x50] &= 0x3f                                # keep products exact in fp32 sums
+        return torch.from_numpy(bits).view(torch.float8_e4m3fn), \
+            torch.from_numpy(rng.integers(120, 134, size=(rows, K // 32), dtype=np.uint8))
+    A, sa = operand(M)
+    B, sb = operand(N)
+    got = oracle.gemm_tn_mxfp8_fp32(A, sa, B, sb).double()
+    Af, Bf = A.float().numpy(), B.float().numpy()
+    for m in range(M):
+        for n in range(N):
+            acc = Fraction(0)
+            for k in range(K):
+                acc += Fraction(float(Af[m, k])) * Fraction(float(Bf[n, k])) * \
+                    Fraction(2) ** (int(sa[m, k // 32]) - 127) * Fraction(2) ** (int(sb[n, k // 32]) - 127)
+            assert abs(float(acc) - float(got[m, n])) <= 1e-5 * max(1.0, abs(float(acc))), (m, n)
