@@ -5,8 +5,8 @@
 
 A step is one gemm launch over one set of synthetic operands already resident in HBM.  The
 headline workload is bf16 M=N=K=8192, Normal(0,1) operands (the configuration the metric is
-quoted on); fp8 8192^3, bf16 4096^3, fp16 512^3 and the skinny projection shapes are timed with
-fewer steps and reported under "extras".  Prints ONE JSON line.
+quoted on); fp8 8192^3 (per-tensor scales and MX block scales), bf16 4096^3, fp16 512^3 and the
+skinny projection shapes are timed with fewer steps and reported under "extras".  Prints ONE JSON line.
 
 Protocol follows the reference's benchmark (kernels/tests/gemm_bench.py:285-295, :502-506):
 warm-up, then timed launches, TFLOP/s = 2*M*N*K / t — with HIP events on the launch stream
@@ -28,7 +28,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs of this script
 # (FETCH_SIZE, then WRITE_SIZE, each with --copy-calibration and scaled by what the same counter
 # reads for the 1 GiB copy: x2.000 and x1.000).  Workloads without a counter run report null.
-MEASURED_TRAFFIC_BYTES = {"bf16_8192": 1.887e9, "fp8_8192": 0.979e9, "skinny_16_14336_4096": 1.265e8}
+MEASURED_TRAFFIC_BYTES = {"bf16_8192": 1.887e9, "fp8_8192": 0.979e9, "mxfp8_8192": 0.965e9, "skinny_16_14336_4096": 1.265e8}
 
 
 def parse():
@@ -82,6 +82,10 @@ def build_case(name, variant, device="cuda", seed=0):
     elif name == "fp8_8192":
         A, B, sa, sb = w.fp8_8192(seed, device)
         sets, tag, fp8 = [(A, B)], "e4m3", (float(sa), float(sb))
+    elif name == "mxfp8_8192":
+        A, sa, B, sb = w.mxfp8_8192(seed, device)
+        # weights-style call: the block scales are re-laid once, outside the timed launches
+        sets, tag, fp8 = [(A, B)], "e4m3", ("mx", gemm_kernels.shuffle_mx_scales(sa), gemm_kernels.shuffle_mx_scales(sb))
     elif name.startswith("skinny_"):
         M, N, K = (int(x) for x in name.split("_")[1:])
         # rotate operand sets so weights come from HBM, not the Infinity Cache (256 MB)
@@ -98,13 +102,17 @@ def build_case(name, variant, device="cuda", seed=0):
     def call():
         A, B = sets[state["i"] % len(sets)]
         state["i"] += 1
-        if fp8:
+        if fp8 and fp8[0] == "mx":
+            gemm_kernels.gemm_tn_mxfp8(A, B, fp8[1], fp8[2], C, True)
+        elif fp8:
             gemm_kernels.gemm_tn_fp8(A, B, fp8[0], fp8[1], C, variant)
         else:
             gemm_kernels.gemm_tn(A, B, C, variant)
 
     es = sets[0][0].element_size()
     nbytes = (M * K + N * K) * es + M * N * C.element_size()
+    if fp8 and fp8[0] == "mx":
+        nbytes += (M + N) * (K // 32)
     return call, 2.0 * M * N * K, nbytes, tag, (M, N, K), sets, C, fp8
 
 
@@ -187,7 +195,7 @@ def main():
 
     extras = []
     if not a.no_extras:
-        names = ["bf16_8192", "fp8_8192", "bf16_4096", "fp16_512"] + \
+        names = ["bf16_8192", "fp8_8192", "mxfp8_8192", "bf16_4096", "fp16_512"] + \
                 ["skinny_%d_%d_%d" % (m, n, k) for (n, k) in ((14336, 4096), (4096, 14336), (6144, 4096))
                  for m in (16, 64, 256)]
         for n in names:

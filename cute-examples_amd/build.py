@@ -19,6 +19,8 @@ LIB = os.path.join(OUT, "libmi355gemm.so")
 
 HIP_SOURCES = ["gemm_api.hip", "gemm_tn_simple.hip", "gemm_tn_ring.hip", "gemm_tn_pingpong.hip", "gemm_tn_stream.hip", "quantize_e4m3.hip", "mx_scales.hip"]
 
+CHECKED_SOURCE = "gemm_tn_ring.hip"   # its device assembly is verified after compilation
+
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -38,8 +40,30 @@ def _run(cmd):
 
 
 def build_lib():
+    """Compile every source to an object (in parallel), check the generated assembly of the
+    block-scaled kernel (check_async_loads.py), link."""
+    import glob
+    import tempfile
+    from concurrent.futures import ThreadPoolExecutor
+
+    sys.path.insert(0, HERE)
+    import check_async_loads
+
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    _run([hipcc] + HIPCC_FLAGS + ["-o", LIB] + [os.path.join(CSRC, s) for s in HIP_SOURCES])
+    with tempfile.TemporaryDirectory() as tmp:
+        def compile_one(src):
+            obj = os.path.join(tmp, src.replace(".hip", ".o"))
+            extra = ["-save-temps=obj"] if src == CHECKED_SOURCE else []
+            _run([hipcc] + HIPCC_FLAGS + ["-c"] + extra + ["-o", obj, os.path.join(CSRC, src)])
+            return obj
+
+        with ThreadPoolExecutor(max_workers=min(len(HIP_SOURCES), os.cpu_count() or 1)) as pool:
+            objs = list(pool.map(compile_one, HIP_SOURCES))
+        asm = glob.glob(os.path.join(tmp, CHECKED_SOURCE.replace(".hip", "") + "-hip-amdgcn-*gfx950.s"))
+        if len(asm) != 1:
+            raise RuntimeError("expected one device assembly file for %s, found %r" % (CHECKED_SOURCE, asm))
+        print("check_async_loads: %d scale operands ok" % check_async_loads.check(asm[0]), flush=True)
+        _run([hipcc] + HIPCC_FLAGS + ["-o", LIB] + objs)
     return LIB
 
 

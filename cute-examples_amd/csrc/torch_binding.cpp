@@ -177,8 +177,9 @@ const uint8_t* mx_scale_ptr(const torch::Tensor& s, const torch::Tensor& x, cons
 
 // C = A · B^T for MX-quantised operands: A_q, B_q float8_e4m3fn (M,K), (N,K); scale_a, scale_b
 // E8M0 bytes (M,K/32), (N,K/32); C bf16 or fp16.
+// With scales_shuffled the scale tensors are outputs of shuffle_mx_scales (flat uint8).
 torch::Tensor gemm_tn_mxfp8(const torch::Tensor A_q, const torch::Tensor B_q, const torch::Tensor scale_a,
-                            const torch::Tensor scale_b, torch::Tensor C) {
+                            const torch::Tensor scale_b, torch::Tensor C, bool scales_shuffled) {
   TORCH_CHECK(A_q.device() == B_q.device(), "All tensors must be on the same device");
   TORCH_CHECK(A_q.is_contiguous() && B_q.is_contiguous(), "All tensors must be contiguous");
   TORCH_CHECK(A_q.dim() == 2 && B_q.dim() == 2, "Both tensors must be 2D (matrix) tensors");
@@ -194,15 +195,27 @@ torch::Tensor gemm_tn_mxfp8(const torch::Tensor A_q, const torch::Tensor B_q, co
   TORCH_CHECK(out_dt == MI355_BF16 || out_dt == MI355_F16, "C must be bfloat16 or float16");
   TORCH_CHECK(N <= 1 || C.stride(1) == 1, "C must be contiguous in its last dimension");
   const int64_t ldc = M > 1 ? C.stride(0) : N;
-  const uint8_t* sa = mx_scale_ptr(scale_a, A_q, "scale_a");
-  const uint8_t* sb = mx_scale_ptr(scale_b, B_q, "scale_b");
   int st = mi355_gemm_mx_check(M, N, K, K, K, ldc, out_dt);
   TORCH_CHECK(st == MI355_OK, "gemm_kernels: ", mi355_gemm_strerror(st), " [mxfp8 M=", M, " N=", N, " K=", K, "]");
   TORCH_CHECK(A_q.is_cuda(), "gemm_kernels runs on a HIP device only; got tensors on ", A_q.device());
   if (M == 0 || N == 0) return C;
   c10::DeviceGuard guard(A_q.device());
   hipStream_t stream = c10::hip::getCurrentHIPStream(A_q.device().index()).stream();
-  const size_t ws_bytes = mi355_gemm_mx_workspace_bytes(M, N, K, 0);
+  const uint8_t *sa, *sb;
+  if (scales_shuffled) {
+    auto shuffled = [&](const torch::Tensor& t, int64_t rows, const char* name) {
+      TORCH_CHECK(t.scalar_type() == at::kByte && t.dim() == 1 && t.is_contiguous() && t.device() == A_q.device() &&
+                      (size_t)t.numel() == mi355_mx_shuffled_bytes(rows, K),
+                  name, " must be the output of shuffle_mx_scales for this operand");
+      return (const uint8_t*)t.const_data_ptr();
+    };
+    sa = shuffled(scale_a, M, "scale_a");
+    sb = shuffled(scale_b, N, "scale_b");
+  } else {
+    sa = mx_scale_ptr(scale_a, A_q, "scale_a");
+    sb = mx_scale_ptr(scale_b, B_q, "scale_b");
+  }
+  const size_t ws_bytes = mi355_gemm_mx_workspace_bytes(M, N, K, scales_shuffled ? 1 : 0);
   torch::Tensor ws;
   void* ws_ptr = nullptr;
   if (ws_bytes) {
@@ -210,10 +223,29 @@ torch::Tensor gemm_tn_mxfp8(const torch::Tensor A_q, const torch::Tensor B_q, co
     ws_ptr = ws.data_ptr();
   }
   st = mi355_gemm_tn_mxfp8(A_q.const_data_ptr(), B_q.const_data_ptr(), C.mutable_data_ptr(), M, N, K, K, K, ldc, sa,
-                           M > 1 ? scale_a.stride(0) : K / 32, sb, N > 1 ? scale_b.stride(0) : K / 32, 0, out_dt,
+                           !scales_shuffled && M > 1 ? scale_a.stride(0) : K / 32, sb,
+                           !scales_shuffled && N > 1 ? scale_b.stride(0) : K / 32, scales_shuffled ? 1 : 0, out_dt,
                            ws_ptr, ws_bytes, (void*)stream);
   TORCH_CHECK(st == MI355_OK, "gemm_kernels: ", mi355_gemm_strerror(st));
   return C;
+}
+
+// Scale bytes (rows, K/32) of one operand -> the layout the kernel reads (a flat uint8 tensor); do
+// it once for weights and pass scales_shuffled=True to gemm_tn_mxfp8.
+torch::Tensor shuffle_mx_scales(const torch::Tensor scales) {
+  TORCH_CHECK(scales.scalar_type() == at::kByte || scales.scalar_type() == at::kFloat8_e8m0fnu,
+              "scales must be uint8 or float8_e8m0fnu");
+  TORCH_CHECK(scales.dim() == 2 && (scales.size(1) <= 1 || scales.stride(1) == 1), "scales must be (rows, K/32), rows contiguous");
+  const int64_t rows = scales.size(0), K = scales.size(1) * 32;
+  TORCH_CHECK(K % 128 == 0, "K must be a multiple of 128");
+  TORCH_CHECK(scales.is_cuda(), "gemm_kernels runs on a HIP device only; got a tensor on ", scales.device());
+  c10::DeviceGuard guard(scales.device());
+  hipStream_t stream = c10::hip::getCurrentHIPStream(scales.device().index()).stream();
+  torch::Tensor out = torch::empty({(int64_t)mi355_mx_shuffled_bytes(rows, K)}, scales.options().dtype(at::kByte));
+  int st = mi355_mx_shuffle_scales((const uint8_t*)scales.const_data_ptr(), rows, K, rows > 1 ? scales.stride(0) : K / 32,
+                                   out.data_ptr<uint8_t>(), (void*)stream);
+  TORCH_CHECK(st == MI355_OK, "gemm_kernels: ", mi355_gemm_strerror(st));
+  return out;
 }
 
 // (x_q, scales): x (rows, K) -> float8_e4m3fn (rows, K) and uint8 E8M0 scale bytes (rows, K/32),
@@ -265,7 +297,10 @@ PYBIND11_MODULE(_C, m) {
         py::arg("x"));
   m.def("gemm_tn_mxfp8", &test::gemm_tn_mxfp8,
         "C = A @ B.T for MX block-scaled float8_e4m3fn operands (one E8M0 scale byte per 32 elements of K)",
-        py::arg("A_q"), py::arg("B_q"), py::arg("scale_a"), py::arg("scale_b"), py::arg("C"));
+        py::arg("A_q"), py::arg("B_q"), py::arg("scale_a"), py::arg("scale_b"), py::arg("C"),
+        py::arg("scales_shuffled") = false);
+  m.def("shuffle_mx_scales", &test::shuffle_mx_scales,
+        "re-lay MX scale bytes (rows, K/32) into the layout the kernel reads", py::arg("scales"));
   m.def("quantize_mxfp8", &test::quantize_mxfp8,
         "MX quantisation on the device: returns (x_q float8_e4m3fn, scales uint8 (rows, K/32))", py::arg("x"));
   m.def("select_variant", &test::select_variant, py::arg("M"), py::arg("N"), py::arg("K"),

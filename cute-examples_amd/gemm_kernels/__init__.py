@@ -9,7 +9,7 @@ plus the variant-selecting and fp8 entry points of the native module.  The nativ
 required: importing this package without a built gemm_kernels/_C*.so raises ImportError.
 """
 from ._C import (gemm_tn, gemm_tn_fp8, gemm_tn_mxfp8, gemm_tn_test, quantize_e4m3, quantize_mxfp8,
-                 select_variant, version)
+                 select_variant, shuffle_mx_scales, version)
 
 __all__ = ["gemm_tn_test", "gemm_tn", "gemm_tn_fp8", "gemm_tn_mxfp8", "quantize_e4m3", "quantize_mxfp8",
-           "select_variant", "version"]
+           "shuffle_mx_scales", "select_variant", "version"]

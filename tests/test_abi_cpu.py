@@ -11,7 +11,8 @@ from tests import abi_ctypes as ac
 
 def test_exports_every_declared_symbol(abi):
     names = ac.declared_symbols()
-    assert {"mi355_gemm_tn", "mi355_gemm_tn_scaled", "mi355_quantize_e4m3"} <= set(names) and len(names) >= 9
+    assert {"mi355_gemm_tn", "mi355_gemm_tn_scaled", "mi355_quantize_e4m3", "mi355_gemm_tn_mxfp8",
+            "mi355_quantize_mxfp8", "mi355_mx_shuffle_scales"} <= set(names) and len(names) >= 15
     for n in names:
         assert hasattr(abi, n), n
     dyn = subprocess.run(["nm", "-D", "--defined-only", ac.LIB], capture_output=True, text=True).stdout
@@ -72,6 +73,41 @@ def test_quantize_rejects_before_any_device_access(abi):
     assert f(None, ac.E4M3, 16, None, None, None) == ac.ERR_DTYPE
     assert f(None, ac.F32, -1, None, None, None) == ac.ERR_SHAPE
     assert f(17, ac.F32, 16, 8, 12, None) == ac.ERR_ALIGN
+
+
+@pytest.mark.parametrize("args,want", [
+    ((256, 256, 128, 128, 128, 256, ac.BF16), ac.OK),
+    ((100, 260, 1024, 1024, 1040, 264, ac.F16), ac.OK),
+    ((256, 256, 64, 64, 64, 256, ac.BF16), ac.ERR_SHAPE),            # K % 128
+    ((256, 256, 128, 120, 128, 256, ac.BF16), ac.ERR_SHAPE),         # lda < K
+    ((256, 258, 128, 128, 128, 258, ac.BF16), ac.ERR_SHAPE),         # N % 4
+    ((256, 256, 128, 128, 128, 256, ac.E4M3), ac.ERR_DTYPE),
+    ((0, 256, 128, 128, 128, 256, ac.BF16), ac.OK),
+    ((1 << 20, 256, 1 << 17, 1 << 17, 1 << 17, 256, ac.BF16), ac.ERR_SHAPE),   # 4 GiB of scales for A
+])
+def test_mx_check(abi, args, want):
+    assert abi.mi355_gemm_mx_check(*args) == want
+
+
+def test_mx_sizes_and_rejections_before_any_device_access(abi):
+    assert abi.mi355_mx_shuffled_bytes(256, 128) == 256 * 4
+    assert abi.mi355_mx_shuffled_bytes(257, 1024) == 512 * 32       # rows padded to whole 256-row tiles
+    assert abi.mi355_mx_shuffled_bytes(256, 96) == 0                 # K % 128
+    assert abi.mi355_gemm_mx_workspace_bytes(300, 100, 256, 0) == (512 + 256) * 8
+    assert abi.mi355_gemm_mx_workspace_bytes(300, 100, 256, 1) == 0
+    f = abi.mi355_gemm_tn_mxfp8
+    assert f(None, None, None, 256, 256, 128, 128, 128, 256, None, 4, None, 4, 0, ac.BF16, None, 0, None) == ac.ERR_NULL
+    assert f(None, None, None, 256, 256, 100, 128, 128, 256, None, 4, None, 4, 0, ac.BF16, None, 0, None) == ac.ERR_SHAPE
+    assert f(None, None, None, 0, 256, 128, 128, 128, 256, None, 4, None, 4, 0, ac.BF16, None, 0, None) == ac.OK
+    assert f(16, 16, 16, 256, 256, 128, 128, 128, 256, 16, 2, 16, 4, 0, ac.BF16, 16, 1 << 20, None) == ac.ERR_SHAPE  # ld_scale < K/32
+    assert f(16, 16, 16, 256, 256, 128, 128, 128, 256, 16, 4, 16, 4, 0, ac.BF16, 16, 100, None) == ac.ERR_WORKSPACE
+    assert f(24, 16, 16, 256, 256, 128, 128, 128, 256, 16, 4, 16, 4, 1, ac.BF16, None, 0, None) == ac.ERR_ALIGN
+    assert abi.mi355_mx_shuffle_scales(None, 256, 128, 4, None, None) == ac.ERR_NULL
+    assert abi.mi355_mx_shuffle_scales(None, 256, 96, 4, None, None) == ac.ERR_SHAPE
+    assert abi.mi355_quantize_mxfp8(None, ac.BF16, 4, 64, 64, None, None, None) == ac.ERR_NULL
+    assert abi.mi355_quantize_mxfp8(None, ac.E4M3, 4, 64, 64, None, None, None) == ac.ERR_DTYPE
+    assert abi.mi355_quantize_mxfp8(None, ac.BF16, 4, 48, 48, None, None, None) == ac.ERR_SHAPE
+    assert abi.mi355_quantize_mxfp8(16, ac.BF16, 4, 64, 68, 16, 16, None) == ac.ERR_ALIGN
 
 
 def test_workspace_bytes(abi):

@@ -69,6 +69,40 @@ def test_fp8_contract():
         gemm_kernels.gemm_tn_fp8(A, A, torch.ones(2), 1.0, C)
 
 
+def test_mxfp8_contract():
+    A = torch.zeros(256, 256, dtype=torch.float8_e4m3fn)
+    s = torch.full((256, 8), 127, dtype=torch.uint8)
+    C = torch.zeros(256, 256, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        gemm_kernels.gemm_tn_mxfp8(A_q=A, B_q=A, scale_a=s, scale_b=s.view(torch.float8_e8m0fnu), C=C)
+    with pytest.raises(RuntimeError, match="float8_e4m3fn"):
+        gemm_kernels.gemm_tn_mxfp8(A.view(torch.uint8), A.view(torch.uint8), s, s, C)
+    with pytest.raises(RuntimeError, match="bfloat16 or float16"):
+        gemm_kernels.gemm_tn_mxfp8(A, A, s, s, C.float())
+    with pytest.raises(RuntimeError, match="constraint"):                 # K % 128
+        gemm_kernels.gemm_tn_mxfp8(A[:, :160].contiguous(), A[:, :160].contiguous(), s[:, :5], s[:, :5], C)
+    with pytest.raises(RuntimeError, match="multiple of the MX block"):
+        gemm_kernels.gemm_tn_mxfp8(A[:, :48].contiguous(), A[:, :48].contiguous(), s, s, C)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        gemm_kernels.quantize_mxfp8(torch.zeros(4, 64))
+    with pytest.raises(RuntimeError, match="multiple of the MX block"):
+        gemm_kernels.quantize_mxfp8(torch.zeros(4, 48))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        gemm_kernels.shuffle_mx_scales(s)
+
+
+def test_mx_quantizer_in_torch_ops_matches_the_oracle():
+    """The package's torch-op MX quantiser (used for CPU tensors) against the oracle's restatement."""
+    from gemm_kernels import quant
+    from oracle import oracle
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(40, 256, generator=g) * torch.exp2(torch.randint(-15, 15, (40, 1), generator=g).float())
+    x[3, 32:64] = 0
+    q, s = quant.quantize_mxfp8(x)
+    wq, ws = oracle.quantize_mxfp8(x)
+    assert torch.equal(s, ws) and torch.equal(q.view(torch.uint8), wq.view(torch.uint8))
+
+
 def test_select_variant():
     assert gemm_kernels.select_variant(8192, 8192, 8192, torch.bfloat16) in ("basic", "pingpong")
     assert gemm_kernels.select_variant(100, 30, 77, torch.float16) == "simple"

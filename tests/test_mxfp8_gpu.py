@@ -168,6 +168,25 @@ def test_end_to_end_from_bf16(abi):
     assert err <= 5e-2, err
 
 
+def test_python_module_with_preshuffled_scales(abi):
+    import gemm_kernels
+    A, sa = random_mx(384, 512, 30, 116, 124)     # small scales: the fp16 output must not overflow
+    B, sb = random_mx(520, 512, 31, 116, 124)
+    Ad, Bd, sad, sbd = A.cuda(), B.cuda(), sa.cuda(), sb.cuda()
+    C1 = torch.full((384, 520), float("nan"), dtype=torch.float16, device="cuda")
+    C2 = torch.full((384, 520), float("nan"), dtype=torch.float16, device="cuda")
+    gemm_kernels.gemm_tn_mxfp8(Ad, Bd, sad.view(torch.float8_e8m0fnu), sbd, C1)
+    pa, pb = gemm_kernels.shuffle_mx_scales(sad), gemm_kernels.shuffle_mx_scales(sbd)
+    gemm_kernels.gemm_tn_mxfp8(Ad, Bd, pa, pb, C2, scales_shuffled=True)
+    torch.cuda.synchronize()
+    assert torch.equal(C1.view(torch.int16), C2.view(torch.int16))
+    ref = oracle.gemm_tn_mxfp8_fp32(A, sa, B, sb)
+    assert torch.isfinite(C1.cpu().float()).all()
+    assert oracle.rel_frobenius(C1.cpu(), ref) <= TOL
+    with pytest.raises(RuntimeError, match="shuffle_mx_scales"):
+        gemm_kernels.gemm_tn_mxfp8(Ad, Bd, sad, sbd, C2, scales_shuffled=True)
+
+
 def test_full_size_properties(abi):
     """8192^3: the sampled rows against the oracle, and linearity in the scales."""
     from gemm_kernels import workloads
