@@ -66,6 +66,20 @@ def time_calls(call, steps, warmup):
     return e0.elapsed_time(e1) / steps, wall_ms
 
 
+def per_launch_ms(call, steps):
+    """A second pass with an event pair around every launch -> (median, min) ms.  Includes the gap
+    between launches, so it is not the figure `value` is computed from."""
+    import torch
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    ev[0].record()
+    for i in range(steps):
+        call()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    t = sorted(ev[i].elapsed_time(ev[i + 1]) for i in range(steps))
+    return t[len(t) // 2], t[0]
+
+
 def build_case(name, variant, device="cuda", seed=0):
     import torch
     import gemm_kernels
@@ -119,15 +133,17 @@ def build_case(name, variant, device="cuda", seed=0):
 def measure(name, variant, steps, warmup):
     call, flops, nbytes, tag, mnk, sets, C, fp8 = build_case(name, variant)
     ms, wall_ms = time_calls(call, steps, warmup)
+    med, mn = per_launch_ms(call, steps)
     tflops = flops / ms / 1e9
     row = {"workload": name, "M": mnk[0], "N": mnk[1], "K": mnk[2], "dtype": tag, "steps": steps,
-           "ms": round(ms, 5), "wall_ms": round(wall_ms, 5), "tflops": round(tflops, 2),
+           "ms": round(ms, 5), "wall_ms": round(wall_ms, 5), "launch_ms_median": round(med, 5),
+           "launch_ms_min": round(mn, 5), "tflops": round(tflops, 2),
            "pct_mfma_peak": round(100 * tflops / PEAK_TFLOPS[tag], 2),
            "gbs": round(nbytes / ms / 1e6, 1), "pct_hbm_peak": round(100 * nbytes / ms / 1e6 / PEAK_HBM_GBS, 2)}
     return row, (sets, C, fp8, flops, nbytes)
 
 
-def cpu_baseline(A, B, total_rows, budget_s=12.0):
+def cpu_baseline(A, B, total_rows, budget_s=12.0, native_budget_s=5.0):
     """The oracle's fp32 matmul (the reference's ground truth, gemm_test.py:36) timed on the host
     cores on a bounded sample: as many row blocks of A against all of B as fit the budget."""
     import torch
@@ -146,8 +162,23 @@ def cpu_baseline(A, B, total_rows, budget_s=12.0):
         if el > budget_s or done >= 16 * total_rows:
             break
     tflops = 2.0 * done * N * K / el / 1e12
+    # The same product in the operands' own 16-bit type, where torch has a CPU kernel for it.
+    native = None
+    if Ac.dtype in (torch.bfloat16, torch.float16):
+        try:
+            torch.matmul(Ac[:64], Bc.T)
+            t0, n_done = time.perf_counter(), 0
+            while True:
+                torch.matmul(Ac, Bc.T)
+                n_done += rows
+                el_n = time.perf_counter() - t0
+                if el_n > native_budget_s or n_done >= 16 * total_rows:
+                    break
+            native = round(2.0 * n_done * N * K / el_n / 1e12, 4)
+        except RuntimeError:
+            native = None
     return {"value": round(tflops, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
-            "kind": "port",
+            "kind": "port", "native_16bit_value": native,
             "sample": "torch.matmul fp32 (incl. bf16->fp32 casts) of %d-row blocks of A against all of B "
                       "(N=%d, K=%d), %d rows in %.1f s; host has %d logical cpus"
                       % (rows, N, K, done, el, os.cpu_count())}
@@ -188,6 +219,7 @@ def main():
     roof["flops_per_launch"] = flops
     roof["algorithmic_bytes_per_launch"] = nbytes
     roof["avg_launch_ms"] = head["ms"]
+    roof["launch_ms_median"], roof["launch_ms_min"] = head["launch_ms_median"], head["launch_ms_min"]
 
     cpu_operands = (sets[0][0][:1024].cpu(), sets[0][1].cpu(), sets[0][0].shape[0]) if not a.no_cpu else None
     del sets, C, keep
