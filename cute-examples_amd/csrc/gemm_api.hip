@@ -113,7 +113,12 @@ size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int in_dtype,
   int splits = 1;
   if (v == MI355_VARIANT_SKINNY) splits = mi355::stream_splits(M, N, K, elem_bytes(in_dtype));
   else if (v == MI355_VARIANT_BASIC) splits = mi355::ring_splits(M, N, K, elem_bytes(in_dtype));
-  return splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0;
+  if (splits > 1) return (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
+  if (v == MI355_VARIANT_BASIC) {
+    int tail_tiles, tail_splits;
+    return mi355::ring_tail(M, N, K, elem_bytes(in_dtype), &tail_tiles, &tail_splits);
+  }
+  return 0;
 }
 
 int mi355_quantize_e4m3(const void* x, int x_dtype, int64_t n, void* x_q, float* scale_amax, void* stream) {
@@ -184,6 +189,8 @@ int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, in
   g.scale = 1.0f;
   g.splits = 1;
   g.partial = nullptr;
+  g.tail_tiles = 0;
+  g.tail_splits = 1;
   g.scale_a = g.scale_b = nullptr;
   g.mx_a = g.mx_b = nullptr;
   if (K == 0) {  // an empty sum: zeros, written by the generic kernel
@@ -237,6 +244,8 @@ int mi355_gemm_tn_scaled(const void* A, const void* B, void* C, int64_t M, int64
   g.scale = scale;
   g.splits = 1;
   g.partial = nullptr;
+  g.tail_tiles = 0;
+  g.tail_splits = 1;
   g.scale_a = scale_a;
   g.scale_b = scale_b;
   g.mx_a = g.mx_b = nullptr;
@@ -259,13 +268,22 @@ int mi355_gemm_tn_scaled(const void* A, const void* B, void* C, int64_t M, int64
     g.tiles_m = g.tiles_n = 0;
     rc = mi355::launch_stream(g, in_dtype, out_dtype, splits, workspace, s);
   } else if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG) {
-    const int tile = v == MI355_VARIANT_PINGPONG ? 256 : mi355::ring_tile_edge(M, N);
+    const int tile = v == MI355_VARIANT_PINGPONG ? 256 : mi355::ring_tile_edge(M, N, K, elem_bytes(in_dtype));
     if (v == MI355_VARIANT_BASIC) {
       const int splits = mi355::ring_splits(M, N, K, elem_bytes(in_dtype));
       const size_t need = splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0;
       if (need && (!workspace || workspace_bytes < need || (uintptr_t)workspace % 16 != 0)) return MI355_ERR_WORKSPACE;
       g.splits = splits;
       g.partial = (float*)workspace;
+      if (splits == 1) {
+        // Optional: without a workspace the tiles of the last round simply run unsplit.
+        int tail_tiles, tail_splits;
+        const size_t tail_bytes = mi355::ring_tail(M, N, K, elem_bytes(in_dtype), &tail_tiles, &tail_splits);
+        if (tail_bytes && workspace && workspace_bytes >= tail_bytes && (uintptr_t)workspace % 16 == 0) {
+          g.tail_tiles = tail_tiles;
+          g.tail_splits = tail_splits;
+        }
+      }
     }
     g.tiles_m = (M + tile - 1) / tile;
     g.tiles_n = (N + tile - 1) / tile;

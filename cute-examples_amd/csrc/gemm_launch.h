@@ -19,6 +19,11 @@ struct GemmArgs {
   // partial[split][M][N]; launch_splitk_reduce then adds the splits in order, scales and rounds.
   int32_t splits;
   float* partial;
+  // Tail split (single-group tile kernel only, splits == 1): the last tail_tiles tiles in tile-map
+  // order are cut tail_splits ways along K, so that the last, partly filled round of workgroups
+  // takes 1/tail_splits of a tile's time.  Their fp32 partial tiles go to
+  // partial[split][tail tile][tile edge][tile edge] and launch_tail_reduce writes those tiles of C.
+  int32_t tail_tiles, tail_splits;
   // Optional device-resident factors (one float each, or null) multiplied into scale by the
   // kernel that writes C, so that per-tensor fp8 scales never have to visit the host.
   const float* scale_a;
@@ -43,11 +48,14 @@ __device__ __forceinline__ float output_scale(const GemmArgs& g) {
 int launch_tile256_pingpong(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
 // Single-wave-group ring kernel; tile is 256 or 128 (ring_tile_edge and ring_splits are pure host
 // heuristics).
-int ring_tile_edge(int64_t M, int64_t N);
+int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes);
 int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes);
 // C = rne(scale * sum_s partial[s]) for partial laid out [splits][M][N] in fp32.
 int launch_splitk_reduce(const float* partial, const GemmArgs& g, int out_dtype, hipStream_t stream);
 int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, hipStream_t stream);
+// Tail split the single-group kernel would use for this problem (pure host heuristic): returns the
+// workspace bytes it needs (0 = no tail split) and sets *tail_tiles, *tail_splits.
+size_t ring_tail(int64_t M, int64_t N, int64_t K, int elem_bytes, int* tail_tiles, int* tail_splits);
 int launch_tile_ring_mx(const GemmArgs& g, int out_dtype, hipStream_t stream);
 // Block scales: bytes of the shuffled layout for `rows` rows and K elements per row; the shuffle
 // itself (natural (rows, K/32) row-major bytes -> shuffled); and the MX quantiser

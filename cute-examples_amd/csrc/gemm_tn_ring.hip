@@ -129,9 +129,34 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   const uint32_t tiles_m = (uint32_t)g.tiles_m, tiles_n = (uint32_t)g.tiles_n;
   const uint32_t total_tiles = tiles_m * tiles_n;  // the launcher keeps items below 2^31
   // Work items are (tile, split) pairs, split-major, so that workgroups running together read the
-  // same range of K.  steps is the number of k-steps of one item.
-  const uint32_t total_items = total_tiles * (uint32_t)g.splits;
-  const uint32_t steps = __builtin_amdgcn_readfirstlane(k_steps / (uint32_t)g.splits);
+  // same range of K.  With a uniform K split every tile has g.splits items; with a tail split only
+  // the last g.tail_tiles tiles are cut (g.tail_splits ways) and come after all whole tiles.
+  // steps is the number of k-steps of the current item.
+  const uint32_t tail_tiles = (uint32_t)g.tail_tiles, tail_splits = (uint32_t)g.tail_splits;
+  const uint32_t whole_tiles = total_tiles - tail_tiles;  // tail_tiles == 0 unless g.splits == 1
+  const uint32_t total_items = tail_tiles ? whole_tiles + tail_tiles * tail_splits : total_tiles * (uint32_t)g.splits;
+  const uint32_t steps_split = __builtin_amdgcn_readfirstlane(k_steps / (uint32_t)(tail_tiles ? tail_splits : g.splits));
+  uint32_t steps = 0;
+  // item -> (tile number in tile-map order, split, whether it writes fp32 partials); sets steps.
+  auto decode_item = [&](uint32_t it, uint32_t* tile, uint32_t* split_of) __attribute__((always_inline)) -> bool {
+    if (tail_tiles) {
+      if (it < whole_tiles) {
+        *tile = it;
+        *split_of = 0;
+        steps = k_steps;
+        return false;
+      }
+      const uint32_t j = it - whole_tiles;
+      *tile = whole_tiles + j % tail_tiles;
+      *split_of = j / tail_tiles;
+      steps = steps_split;
+      return true;
+    }
+    *tile = it % total_tiles;
+    *split_of = it / total_tiles;
+    steps = steps_split;
+    return g.splits > 1;
+  };
 
   // Descriptors of the A and B row panels of a tile; rows past the matrix edge are out of range.
   auto panel_a = [&](int64_t m0) __attribute__((always_inline)) {
@@ -283,14 +308,24 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   auto epilogue = [&](int64_t m0, int64_t n0) __attribute__((always_inline)) {
     store_output_tile<G, OutT, kNbM, kNbN, kAsmMfma>(acc, g, m0, n0, kTile, wm * kWaveTileM, wn * kWaveTileN, lane, scale);
   };
-  auto store_partial = [&](int64_t m0, int64_t n0, uint32_t split) __attribute__((always_inline)) {
-    store_partial_tile<G, kNbM, kNbN, kAsmMfma>(acc, g, m0, n0, kTile, split, wm * kWaveTileM, wn * kWaveTileN, lane);
+  auto store_partial = [&](int64_t m0, int64_t n0, uint32_t split, uint32_t tile_no) __attribute__((always_inline)) {
+    if (tail_tiles) {
+      // a whole tile of the compact tail workspace (rows past M hold zeros: their operands read as 0)
+      float* base = g.partial + ((int64_t)split * tail_tiles + (tile_no - whole_tiles)) * (kTile * kTile);
+      store_partial_tile<G, kNbM, kNbN, kAsmMfma>(acc, base, kTile, kTile, kTile, wm * kWaveTileM, wn * kWaveTileN, lane);
+    } else {
+      // plane `split` of M x N floats, clipped at the matrix edge
+      const int64_t rows = g.M - m0 < kTile ? g.M - m0 : kTile;
+      const uint32_t cols = (uint32_t)(g.N - n0 < kTile ? g.N - n0 : kTile);
+      float* base = g.partial + ((int64_t)split * g.M + m0) * g.N + n0;
+      store_partial_tile<G, kNbM, kNbN, kAsmMfma>(acc, base, (uint32_t)g.N, rows, cols, wm * kWaveTileM, wn * kWaveTileN, lane);
+    }
   };
 
   uint32_t item = blockIdx.x;
-  uint32_t tile_m, tile_n;
-  tile_coord_t<uint32_t>(item % total_tiles, tiles_m, tiles_n, &tile_m, &tile_n);
-  uint32_t split = item / total_tiles;
+  uint32_t tile_m, tile_n, tile_no, split;
+  bool partial_item = decode_item(item, &tile_no, &split);
+  tile_coord_t<uint32_t>(tile_no, tiles_m, tiles_n, &tile_m, &tile_n);
   uint32_t step0 = __builtin_amdgcn_readfirstlane(split * steps);  // first k-step of the current item
   __amdgpu_buffer_rsrc_t rsrc_a = panel_a((int64_t)tile_m * kTile), rsrc_b = panel_b((int64_t)tile_n * kTile);
   if constexpr (kMx) mx_open_tile(tile_m, tile_n, step0);  // before the copies: see the waits
@@ -422,27 +457,51 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     __builtin_amdgcn_s_barrier();
 
     const int64_t done_m0 = (int64_t)tile_m * kTile, done_n0 = (int64_t)tile_n * kTile;
-    const uint32_t done_split = split;
+    const uint32_t done_split = split, done_tile = tile_no;
+    const bool done_partial = partial_item;
     item += gridDim.x;
     const bool more = item < total_items;
     if (more) {
-      tile_coord_t<uint32_t>(item % total_tiles, tiles_m, tiles_n, &tile_m, &tile_n);
-      split = item / total_tiles;
+      partial_item = decode_item(item, &tile_no, &split);
+      tile_coord_t<uint32_t>(tile_no, tiles_m, tiles_n, &tile_m, &tile_n);
       step0 = __builtin_amdgcn_readfirstlane(split * steps);
       rsrc_a = panel_a((int64_t)tile_m * kTile);
       rsrc_b = panel_b((int64_t)tile_n * kTile);
       if constexpr (kMx) mx_open_tile(tile_m, tile_n, step0);
       open_tile(rsrc_a, rsrc_b, step0);  // in flight while the finished tile is stored
     }
-    if (g.splits > 1) store_partial(done_m0, done_n0, done_split);
+    if (done_partial) store_partial(done_m0, done_n0, done_split, done_tile);
     else epilogue(done_m0, done_n0);
     if (!more) break;
   }
 }
 
+// C tiles of a tail split: rne(scale * (partial[0] + ... + partial[S-1])) in that order, for the
+// last g.tail_tiles tiles in tile-map order; one thread per 4 consecutive columns.
+template <class OutT, int kTileT>
+__global__ __launch_bounds__(256) void tail_reduce(GemmArgs g) {
+  constexpr uint32_t kQuadsPerTile = kTileT * kTileT / 4;
+  const uint32_t q = blockIdx.x * 256u + threadIdx.x;
+  const uint32_t t = q / kQuadsPerTile, in_tile = q % kQuadsPerTile;
+  if (t >= (uint32_t)g.tail_tiles) return;
+  const uint32_t r = in_tile / (kTileT / 4), c = (in_tile % (kTileT / 4)) * 4;
+  uint32_t tile_m, tile_n;
+  tile_coord_t<uint32_t>((uint32_t)(g.tiles_m * g.tiles_n) - (uint32_t)g.tail_tiles + t, (uint32_t)g.tiles_m,
+                         (uint32_t)g.tiles_n, &tile_m, &tile_n);
+  const int64_t m = (int64_t)tile_m * kTileT + r, n = (int64_t)tile_n * kTileT + c;
+  if (m >= g.M || n >= g.N) return;  // N % 4 == 0: a quad is in or out as a whole
+  const float* p = g.partial + (int64_t)t * (kTileT * kTileT) + r * kTileT + c;
+  const int64_t split_stride = (int64_t)g.tail_tiles * (kTileT * kTileT);
+  f32x4 sum = *(const f32x4*)p;
+  for (int s = 1; s < g.tail_splits; ++s) sum += *(const f32x4*)(p + s * split_stride);
+  const float scale = output_scale(g);
+  *(u32x2*)((uint16_t*)g.C + m * g.ldc + n) = Pack4<OutT>::run(sum[0] * scale, sum[1] * scale, sum[2] * scale, sum[3] * scale);
+}
+
 template <class T, class OutT, int kTileT>
 int launch_tile(const GemmArgs& g, hipStream_t stream) {
-  const int64_t items = g.tiles_m * g.tiles_n * g.splits;
+  const int64_t items = g.tail_tiles ? g.tiles_m * g.tiles_n + (int64_t)g.tail_tiles * (g.tail_splits - 1)
+                                     : g.tiles_m * g.tiles_n * g.splits;
   if (items >= ((int64_t)1 << 31)) return -1;  // the kernel counts items in 32 bits
   const int64_t slots = (int64_t)compute_units() * (kTileT == 256 ? 1 : 2);  // resident workgroups (LDS-bound)
   const int64_t blocks = items < slots ? items : slots;
@@ -456,6 +515,11 @@ int launch_tile(const GemmArgs& g, hipStream_t stream) {
   if (hipGetLastError() != hipSuccess) return -1;
   if (g.splits > 1)
     return launch_splitk_reduce(g.partial, g, std::is_same<OutT, BF16>::value ? 0 : 1, stream);
+  if (g.tail_tiles) {
+    const int64_t quads = (int64_t)g.tail_tiles * (kTileT * kTileT / 4);
+    hipLaunchKernelGGL((tail_reduce<OutT, kTileT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, g);
+    if (hipGetLastError() != hipSuccess) return -1;
+  }
   return 0;
 }
 
@@ -466,14 +530,51 @@ int launch(const GemmArgs& g, int tile, hipStream_t stream) {
 
 }  // namespace
 
+namespace {
+
+constexpr int64_t kSlots256 = 256;  // resident workgroups of 256x256 tiles on an MI355X (one per CU);
+                                    // heuristics only, so no device query here
+
+// Tail split of `tiles` 256x256 tiles with `steps` k-steps each.  When the tiles fill one or two
+// rounds of workgroups plus a last round that is at most half full, the tiles of that round are cut
+// along K so that they occupy (almost) all workgroup slots and the round takes 1/S of a tile's
+// time; every item keeps at least 16 k-steps and the k-steps divide evenly, as in ring_splits.
+// Measured at bf16: +5..+10 % for one or two full rounds (4096x6144x4096, 6144^3); with three
+// full rounds (4096x14336x4096) the partly filled round, which runs at a higher clock, costs no
+// more than the partial tiles' extra traffic and second launch (-1 %), and on 128x128 tiles the
+// split loses (-8 % at 4352^2x4096), so those are never cut.
+void tail_plan(int64_t tiles, int64_t steps, int* tail_tiles, int* tail_splits) {
+  *tail_tiles = 0;
+  *tail_splits = 1;
+  const int64_t rest = tiles % kSlots256;
+  if (tiles < kSlots256 || tiles > 3 * kSlots256 || rest == 0) return;
+  int best = 1;
+  for (int s = 2; s <= 16; ++s) {
+    if (rest * s > kSlots256) break;
+    if (steps % s != 0 || steps / s < 16) continue;
+    best = s;
+  }
+  if (best == 1) return;
+  *tail_tiles = (int)rest;
+  *tail_splits = best;
+}
+
+int64_t k_steps_of(int64_t K, int elem_bytes) { return (K * elem_bytes + kRowBytes - 1) / kRowBytes; }
+
+}  // namespace
+
 // Tile edge the single-group kernel should use: 256 unless that leaves most CUs idle and the
 // 128x128 variant (about 0.36 of a 256-tile's time per tile, up to two per CU) finishes sooner.
-int ring_tile_edge(int64_t M, int64_t N) {
-  const int64_t cus = 256;  // MI355X; a heuristic only, so no device query here
+// A last round of 256-tiles that gets a tail split counts as 1/S of a round plus 0.2 for the
+// partial tiles' traffic and the second launch (measured 0.12..0.25).
+int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes) {
   const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
   const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
-  const double time256 = (double)((t256 + cus - 1) / cus);
-  const double time128 = (double)((t128 + cus - 1) / cus) * 0.36;
+  int tail_tiles, tail_splits;
+  tail_plan(t256, k_steps_of(K, elem_bytes), &tail_tiles, &tail_splits);
+  const double time256 = tail_tiles ? (double)(t256 / kSlots256) + 1.0 / tail_splits + 0.2
+                                    : (double)((t256 + kSlots256 - 1) / kSlots256);
+  const double time128 = (double)((t128 + kSlots256 - 1) / kSlots256) * 0.36;
   return time128 < time256 ? 128 : 256;
 }
 
@@ -481,10 +582,10 @@ int ring_tile_edge(int64_t M, int64_t N) {
 // idle (the partial tiles cost S*M*N*8 bytes of extra traffic and a second launch), the k-steps
 // divide evenly and every item keeps at least 16 k-steps.
 int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
-  const int tile = ring_tile_edge(M, N);
+  const int tile = ring_tile_edge(M, N, K, elem_bytes);
   const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile);
   const int64_t slots = 256;  // one item per CU of an MI355X
-  const int64_t steps = (K * elem_bytes + kRowBytes - 1) / kRowBytes;
+  const int64_t steps = k_steps_of(K, elem_bytes);
   int best = 1;
   for (int s = 2; s <= 16; ++s) {
     if (tiles * s > slots) break;
@@ -492,6 +593,16 @@ int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
     best = s;
   }
   return best;
+}
+
+// The tail split (tail_plan) of this problem, if it runs on 256x256 tiles without a uniform K
+// split: returns the workspace bytes of its partial tiles.
+size_t ring_tail(int64_t M, int64_t N, int64_t K, int elem_bytes, int* tail_tiles, int* tail_splits) {
+  *tail_tiles = 0;
+  *tail_splits = 1;
+  if (M <= 0 || N <= 0 || K <= 0 || ring_tile_edge(M, N, K, elem_bytes) != 256) return 0;
+  tail_plan(((M + 255) / 256) * ((N + 255) / 256), k_steps_of(K, elem_bytes), tail_tiles, tail_splits);
+  return (size_t)*tail_tiles * (size_t)*tail_splits * 256 * 256 * sizeof(float);
 }
 
 int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, hipStream_t stream) {

@@ -123,20 +123,18 @@ __device__ __forceinline__ void store_output_tile(typename G::Acc (&acc)[kNbM][k
   }
 }
 
-// The same part of the tile as raw fp32 accumulators into plane `split` (M x N floats, row stride
-// N) of the split-K workspace: 4 consecutive columns per register quad, no lane exchange.
+// The same part of the tile as raw fp32 accumulators into the split-K workspace: `rows` x `cols`
+// floats at `base` with row stride `ld` floats; 4 consecutive columns per register quad, no lane
+// exchange.
 template <class G, int kNbM, int kNbN, bool kAsmRead>
-__device__ __forceinline__ void store_partial_tile(typename G::Acc (&acc)[kNbM][kNbN], const GemmArgs& g,
-                                                   int64_t m0, int64_t n0, int tile_edge, uint32_t split,
-                                                   uint32_t wave_row, uint32_t wave_col, uint32_t lane) {
+__device__ __forceinline__ void store_partial_tile(typename G::Acc (&acc)[kNbM][kNbN], float* base, uint32_t ld,
+                                                   int64_t rows, uint32_t cols, uint32_t wave_row,
+                                                   uint32_t wave_col, uint32_t lane) {
   constexpr int kBlk = G::kBlk;
   constexpr int kQuads = kBlk * kBlk / 64 / 4;
   const uint32_t rblk = lane & (kBlk - 1), grp = lane / kBlk;
-  const int64_t rows = g.M - m0 < tile_edge ? g.M - m0 : tile_edge;
-  const uint32_t cols = (uint32_t)(g.N - n0 < tile_edge ? g.N - n0 : tile_edge);
-  const uint32_t ldp_b = (uint32_t)g.N * 4;
-  const __amdgpu_buffer_rsrc_t rp = make_raw_buffer(g.partial + ((int64_t)split * g.M + m0) * g.N + n0,
-                                                    (uint32_t)(((rows - 1) * g.N + cols) * 4));
+  const uint32_t ldp_b = ld * 4;
+  const __amdgpu_buffer_rsrc_t rp = make_raw_buffer(base, (uint32_t)(((rows - 1) * ld + cols) * 4));
   const uint32_t col0 = wave_col + grp * 4;
   const uint32_t v0 = (wave_row + rblk) * ldp_b + col0 * 4;
   const uint32_t block_step = __builtin_amdgcn_readfirstlane(kBlk * ldp_b);

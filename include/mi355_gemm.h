@@ -65,7 +65,9 @@ enum mi355_status {
  *             (1.0f for bf16/fp16; scale_a*scale_b for per-tensor-scaled fp8)
  *   variant   enum mi355_variant
  *   workspace device scratch of at least mi355_gemm_workspace_bytes(...) bytes, or NULL when
- *             that function returns 0; contents need not be initialised
+ *             that function returns 0; contents need not be initialised.  A K split needs it
+ *             (MI355_ERR_WORKSPACE otherwise); the tail split of the tiled kernel (the tiles of
+ *             a partly filled last round of workgroups cut along K) is skipped without it
  *   stream    hipStream_t on which the kernels are enqueued (NULL = the null stream)
  *
  * Replaces test::gemm_tn_test (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92): same operand
@@ -168,9 +170,10 @@ size_t mi355_mx_shuffled_bytes(int64_t rows, int64_t K);
 int mi355_quantize_mxfp8(const void *x, int x_dtype, int64_t rows, int64_t K, int64_t ldx,
                          void *x_q, uint8_t *scales, void *stream);
 
-/* Scratch bytes mi355_gemm_tn needs for this problem and variant (0 for most shapes).
+/* Scratch bytes mi355_gemm_tn wants for this problem and variant (0 for most shapes).
  * Counterpart: none in the reference (it has no split-K); sizes the split-K partials that
- * replace the reference's single-pass accumulation (gemm.cuh:352-367) on skinny shapes. */
+ * replace the reference's single-pass accumulation (gemm.cuh:352-367) on skinny shapes and in
+ * the last round of tiles when that round would leave more than half of the CUs idle. */
 size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K,
                                   int in_dtype, int variant);
 

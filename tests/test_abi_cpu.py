@@ -122,6 +122,15 @@ def test_workspace_bytes(abi):
     assert f(16, 4096, 14336, ac.BF16, ac.PINGPONG) == 0
     assert f(16, 4096, 14336, ac.E4M3, ac.AUTO) == f(16, 4096, 14336, ac.E4M3, ac.BASIC) > 0   # fp8: tiled kernel + K splits
     assert f(-1, 4096, 14336, ac.BF16, ac.AUTO) == 0 and f(16, 4096, 14336, 9, ac.AUTO) == 0
+    # tail split: 384 tiles of 256 -> the 128 of the second round are cut in two along K
+    assert f(4096, 6144, 4096, ac.BF16, ac.BASIC) == f(4096, 6144, 4096, ac.BF16, ac.AUTO) == 2 * 128 * 256 * 256 * 4
+    assert f(4096, 6144, 1024, ac.BF16, ac.BASIC) == 0          # 16 k-steps: too short to cut
+    assert f(4096, 7168, 4096, ac.BF16, ac.BASIC) == 0          # 448 tiles: the last round is 3/4 full
+    assert f(4352, 4352, 4096, ac.BF16, ac.BASIC) == 4 * 33 * 256 * 256 * 4    # 289 tiles: 33 cut in four
+    assert f(4352, 4352, 1024, ac.BF16, ac.BASIC) == 0          # too short to cut: runs on 128x128 tiles
+    assert f(6144, 6144, 6144, ac.BF16, ac.BASIC) == 4 * 64 * 256 * 256 * 4    # two full rounds + 64 tiles cut in four
+    assert f(4096, 14336, 4096, ac.BF16, ac.BASIC) == 0         # three full rounds: not worth it
+    assert f(4096, 6144, 4096, ac.BF16, ac.PINGPONG) == 0
 
 
 def test_select_variant(abi):

@@ -215,6 +215,43 @@ def test_basic_kernel_with_128_tiles_and_k_splits(abi, dt, M, N, K):
     assert torch.equal(C.view(torch.int16), C2.view(torch.int16))   # fixed summation order
 
 
+@pytest.mark.parametrize("dt,M,N,K", [
+    (torch.bfloat16, 4096, 6144, 4096),        # 384 tiles of 256: one full round + 128 tiles cut in two
+    (torch.bfloat16, 6144, 6144, 6144),        # two full rounds + 64 tiles cut in four
+    (torch.bfloat16, 4352, 4352, 4096),        # 289 tiles: one full round + 33 tiles cut in four
+    (torch.float8_e4m3fn, 4096, 6144, 8192),
+    (torch.float16, 4000, 6100, 4200),         # ragged M, N and last k-step: 384 tiles of 256, 66 k-steps cut in two
+])
+def test_tail_split(abi, dt, M, N, K):
+    """More tiles than workgroup slots with a last round at most half full: the tiles of that round
+    are cut along K.  Checked against the oracle, element by element against the one-thread-per-
+    output kernel, for determinism, and without a workspace (the split is then skipped)."""
+    assert abi.mi355_gemm_workspace_bytes(M, N, K, ac.torch_code(dt), ac.BASIC) > 0
+    A = rand((M, K), M, torch.float32).clamp_(-50, 50).to(dt)
+    B = rand((N, K), N, torch.float32).clamp_(-50, 50).to(dt)
+    scale = 2.0 ** -4
+    C = run_abi(abi, A, B, ac.BASIC, scale)
+    check(C, A, B, scale)
+    Ad, Bd = A.cuda(), B.cuda()
+    S = torch.empty((M, N), dtype=out_dtype_of(dt), device="cuda")
+    assert ac.gemm_tn(abi, Ad, Bd, S, scale, ac.SIMPLE) == 0
+    torch.cuda.synchronize()
+    d = (C.float() - S.cpu().float()).abs()
+    bad = d > 2e-2 * S.cpu().float().abs() + 2e-2 * (K ** 0.5) * scale
+    assert int(bad.sum()) == 0, (int(bad.sum()), float(d.max()))
+    C2 = run_abi(abi, A, B, ac.AUTO, scale)
+    assert torch.equal(C.view(torch.int16), C2.view(torch.int16))
+    # no workspace: same tiles, no split; differs from C only by the summation order inside the tail tiles
+    C3 = torch.full((M, N), float("nan"), dtype=out_dtype_of(dt), device="cuda")
+    rc = abi.mi355_gemm_tn(Ad.data_ptr(), Bd.data_ptr(), C3.data_ptr(), M, N, K, K, K, N, ac.torch_code(dt),
+                           ac.torch_code(C3.dtype), scale, ac.BASIC, None, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    check(C3.cpu(), A, B, scale)
+    same = (C3.cpu().view(torch.int16) == C.view(torch.int16)).float().mean()
+    assert 0.5 < same < 1.0 or dt == torch.float8_e4m3fn, same
+
+
 def test_k_zero_and_empty(abi):
     A, B = torch.zeros(8, 0, dtype=torch.bfloat16), torch.zeros(4, 0, dtype=torch.bfloat16)
     C = run_abi(abi, A, B)
