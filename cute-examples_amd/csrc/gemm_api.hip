@@ -32,7 +32,6 @@ bool tile256_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64
 // 128x128-tile kernel with K splits is faster (measured on the LLM projection shapes).
 constexpr int64_t kSkinnyAutoMaxM = 64;
 bool skinny_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int in_dtype) {
-  if (in_dtype == MI355_E4M3) return false;
   if (M > 256) return false;
   return tile256_ok(M, N, K, lda, ldb, ldc, in_dtype);
 }
@@ -75,7 +74,7 @@ const char* mi355_gemm_strerror(int status) {
     case MI355_ERR_SHAPE:
       return "shape or leading dimension violates a constraint of the requested variant "
              "(need M,N,K >= 0, lda,ldb >= K, ldc >= N; tiled variants need K*elem_bytes % 16 == 0, "
-             "16-byte aligned rows and N % 4 == 0; skinny needs M <= 256 and 16-bit inputs)";
+             "16-byte aligned rows and N % 4 == 0; skinny needs M <= 256)";
     case MI355_ERR_VARIANT: return "unknown variant, or variant not available for this shape/dtype";
     case MI355_ERR_WORKSPACE: return "workspace is NULL or smaller than mi355_gemm_workspace_bytes()";
     case MI355_ERR_LAUNCH: return "HIP runtime rejected the kernel launch";

@@ -8,8 +8,9 @@
 //   * per k-step (128 B of K per row) the TM rows of X and 64 rows of W go global -> LDS with
 //     full-cache-line direct-to-LDS loads into a ring of kDepth stages, kDepth-1 k-steps ahead;
 //   * the four waves read MFMA fragments from LDS (same 16-byte-chunk swizzle as the big-tile
-//     kernels) and run v_mfma_f32_16x16x32; W blocks are the MFMA rows, so every lane ends up
-//     with four consecutive n of one m;
+//     kernels) and run v_mfma_f32_16x16x32 (two per k-step and block pair) or, for fp8,
+//     v_mfma_f32_16x16x128_f8f6f4 (one); W blocks are the MFMA rows, so every lane ends up with
+//     four consecutive n of one m;
 //   * with K split S ways the partial tiles go to an fp32 workspace [S][M][N] and a second kernel
 //     adds them in a fixed order (deterministic), scales and rounds; with S = 1 the tile is
 //     rounded and stored directly.
@@ -29,10 +30,17 @@ constexpr int kThreads = 256;
 constexpr int kTileN = 64;
 
 // kMB x kNB 16x16 blocks per wave, kWM x kWN waves (kWM * kWN == 4).
+// Geometry per input type: 16x16 blocks for all of them (fp8 on the 16x16x128 shape).
+template <class T> struct StreamGeo { typedef Geo<T> type; };
+template <> struct StreamGeo<E4M3> { typedef GeoE4M3Rows type; };
+
 template <class T, class OutT, int kMB, int kNB, int kWM, int kWN, int kDepth>
 __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* partial, int splits) {
-  typedef Geo<T> G;
-  static_assert(G::kBlk == 16 && kWM * kWN == 4, "16x16x32 MFMA, four waves");
+  typedef typename StreamGeo<T>::type G;
+  typedef typename G::Frag Frag;
+  static_assert(G::kBlk == 16 && kWM * kWN == 4, "16x16 MFMA blocks, four waves");
+  constexpr int kSliceChunks = G::kGroups * G::kCpl;   // 16-byte chunks of a row one MFMA consumes
+  constexpr int kSlices = 8 / kSliceChunks;            // MFMAs per k-step and block pair
   constexpr int kTm = 16 * kMB * kWM, kTn = 16 * kNB * kWN;
   static_assert(kTn == kTileN, "grid assumes 64-row W tiles");
   constexpr int kStageBytes = (kTm + kTn) * kRowBytes;
@@ -94,8 +102,15 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
   const uint32_t swz = swizzle(rblk);
   const uint32_t x_lane = (wm * kMB * 16 + rblk) * kRowBytes;
   const uint32_t w_lane = (kTm + wn * kNB * 16 + rblk) * kRowBytes;
-  auto frag = [&](const uint8_t* rows, int blk, int s) __attribute__((always_inline)) -> i32x4 {
-    return *(const i32x4*)(rows + blk * 16 * kRowBytes + (((uint32_t)(s * 4) + grp) ^ swz) * 16);
+  auto frag = [&](const uint8_t* rows, int blk, int s) __attribute__((always_inline)) -> Frag {
+    const uint8_t* p = rows + blk * 16 * kRowBytes;
+    if constexpr (G::kCpl == 1) {
+      return *(const i32x4*)(p + (((uint32_t)(s * kSliceChunks) + grp) ^ swz) * 16);
+    } else {
+      const i32x4 lo = *(const i32x4*)(p + (((uint32_t)(s * kSliceChunks) + grp * 2) ^ swz) * 16);
+      const i32x4 hi = *(const i32x4*)(p + (((uint32_t)(s * kSliceChunks) + grp * 2 + 1) ^ swz) * 16);
+      return (i32x8){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
   };
 
   f32x4 acc[kMB][kNB];
@@ -116,8 +131,8 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
     issue_step(refill, kt + kDepth - 1);
     const uint8_t* st_base = ring + stage * kStageBytes;
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      i32x4 fx[kMB], fw[kNB];
+    for (int s = 0; s < kSlices; ++s) {
+      Frag fx[kMB], fw[kNB];
 #pragma unroll
       for (int j = 0; j < kNB; ++j) fw[j] = frag(st_base + w_lane, j, s);
 #pragma unroll
@@ -233,6 +248,7 @@ int launch_stream(const GemmArgs& g, int in_dtype, int out_dtype, int splits, vo
   switch (in_dtype) {
     case 0: return out_bf16 ? launch_m<BF16, BF16>(g, splits, ws, stream) : launch_m<BF16, F16>(g, splits, ws, stream);
     case 1: return out_bf16 ? launch_m<F16, BF16>(g, splits, ws, stream) : launch_m<F16, F16>(g, splits, ws, stream);
+    case 2: return out_bf16 ? launch_m<E4M3, BF16>(g, splits, ws, stream) : launch_m<E4M3, F16>(g, splits, ws, stream);
   }
   return -1;
 }

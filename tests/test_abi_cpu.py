@@ -45,7 +45,7 @@ def test_version_and_strerror(abi):
     ((256, 256, 24, 32, 32, 256, ac.E4M3, ac.BF16, ac.BASIC), ac.ERR_SHAPE),  # 24 fp8 bytes % 16
     ((64, 256, 128, 128, 128, 256, ac.BF16, ac.BF16, ac.SKINNY), ac.OK),
     ((257, 256, 128, 128, 128, 256, ac.BF16, ac.BF16, ac.SKINNY), ac.ERR_SHAPE),     # M > 256
-    ((64, 256, 128, 128, 128, 256, ac.E4M3, ac.BF16, ac.SKINNY), ac.ERR_SHAPE),      # fp8
+    ((64, 256, 128, 128, 128, 256, ac.E4M3, ac.BF16, ac.SKINNY), ac.OK),             # fp8 streams too
     ((0, 0, 0, 0, 0, 0, ac.BF16, ac.BF16, ac.AUTO), ac.OK),
     # 32-bit offsets inside a tile: 256 rows of A or B below 2 GiB, 256 rows of fp32 partials too
     ((256, 256, 64, 1 << 22, 64, 256, ac.BF16, ac.BF16, ac.BASIC), ac.ERR_SHAPE),
@@ -120,7 +120,8 @@ def test_workspace_bytes(abi):
     need = f(16, 4096, 14336, ac.BF16, ac.AUTO)
     assert need > 0 and need % (16 * 4096 * 4) == 0 and need // (16 * 4096 * 4) <= 16
     assert f(16, 4096, 14336, ac.BF16, ac.PINGPONG) == 0
-    assert f(16, 4096, 14336, ac.E4M3, ac.AUTO) == f(16, 4096, 14336, ac.E4M3, ac.BASIC) > 0   # fp8: tiled kernel + K splits
+    assert f(16, 4096, 14336, ac.E4M3, ac.AUTO) == f(16, 4096, 14336, ac.E4M3, ac.SKINNY) > 0  # fp8 streams too
+    assert f(16, 4096, 14336, ac.E4M3, ac.BASIC) > 0                                           # tiled kernel + K splits
     assert f(-1, 4096, 14336, ac.BF16, ac.AUTO) == 0 and f(16, 4096, 14336, 9, ac.AUTO) == 0
     # tail split: 384 tiles of 256 -> the 128 of the second round are cut in two along K
     assert f(4096, 6144, 4096, ac.BF16, ac.BASIC) == f(4096, 6144, 4096, ac.BF16, ac.AUTO) == 2 * 128 * 256 * 256 * 4
@@ -138,7 +139,8 @@ def test_select_variant(abi):
     assert abi.mi355_gemm_select_variant(16, 14336, 4096, ac.BF16) == ac.SKINNY
     assert abi.mi355_gemm_select_variant(64, 4096, 14336, ac.F16) == ac.SKINNY
     assert abi.mi355_gemm_select_variant(256, 4096, 14336, ac.F16) == ac.BASIC   # 128x128 tiles + K splits
-    assert abi.mi355_gemm_select_variant(16, 14336, 4096, ac.E4M3) == ac.BASIC
+    assert abi.mi355_gemm_select_variant(16, 14336, 4096, ac.E4M3) == ac.SKINNY
+    assert abi.mi355_gemm_select_variant(256, 14336, 4096, ac.E4M3) == ac.BASIC
     assert abi.mi355_gemm_select_variant(100, 30, 77, ac.BF16) == ac.SIMPLE
     assert abi.mi355_gemm_select_variant(8192, 8192, 8192, 9) == ac.ERR_DTYPE
 

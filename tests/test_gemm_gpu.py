@@ -356,13 +356,18 @@ def test_config4_skinny_projections(abi, M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 512, 128), (16, 128, 8), (48, 260, 1096), (256, 64, 4104), (10, 260, 256), (17, 64, 1024), (33, 512, 4096),
                                    (64, 1024, 2048), (100, 640, 1024), (129, 72, 512), (256, 768, 2048)])
-@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
 def test_skinny_kernel_every_tile_height_and_split(abi, dt, M, N, K):
     """Each TM configuration (16/32/64/128/256), with and without K splits, ragged M and N."""
-    A, B = rand((M, K), M + 1, dt), rand((N, K), N + 2, dt)
-    C = run_abi(abi, A, B, ac.SKINNY)
-    check(C, A, B)
-    assert oracle.rel_frobenius(C, oracle.c_gemm_tn_f32(A, B)) <= TOL[dt]
+    if dt == torch.float8_e4m3fn:
+        K = max(16, K // 16 * 16)   # fp8 rows are moved in 16-byte chunks
+        A = rand((M, K), M + 1, torch.float32).clamp_(-100, 100).to(dt)
+        B = rand((N, K), N + 2, torch.float32).clamp_(-100, 100).to(dt)
+    else:
+        A, B = rand((M, K), M + 1, dt), rand((N, K), N + 2, dt)
+    C = run_abi(abi, A, B, ac.SKINNY, 0.25)
+    check(C, A, B, 0.25)
+    assert oracle.rel_frobenius(C, oracle.c_gemm_tn_f32(A, B, 0.25)) <= TOL[dt]
 
 
 def test_skinny_split_k_is_deterministic_and_needs_its_workspace(abi):
