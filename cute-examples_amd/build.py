@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "gemm_kernels")
 LIB = os.path.join(OUT, "libmi355gemm.so")
 
-HIP_SOURCES = ["gemm_api.hip", "gemm_tn_simple.hip", "gemm_tn_ring.hip", "gemm_tn_pingpong.hip", "gemm_tn_stream.hip", "quantize_e4m3.hip", "mx_scales.hip"]
+HIP_SOURCES = ["gemm_api.hip", "gemm_tn_simple.hip", "gemm_tn_ring.hip", "ring_plan.hip", "gemm_tn_pingpong.hip", "gemm_tn_stream.hip", "quantize_e4m3.hip", "mx_scales.hip"]
 
 CHECKED_SOURCE = "gemm_tn_ring.hip"   # its device assembly is verified after compilation
 

@@ -105,6 +105,36 @@ int mi355_gemm_select_variant(int64_t M, int64_t N, int64_t K, int in_dtype) {
   return resolve(M, N, K, K, K, N, in_dtype, MI355_VARIANT_AUTO);
 }
 
+int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant, int* tile_rows, int* tile_cols,
+                    int* k_splits, int* tail_tiles, int* tail_splits) {
+  if (!valid_in(in_dtype)) return MI355_ERR_DTYPE;
+  if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_SIMPLE) return MI355_ERR_VARIANT;
+  if (M < 0 || N < 0 || K < 0) return MI355_ERR_SHAPE;
+  const int v = resolve(M, N, K, K, K, N, in_dtype, variant);
+  if (v < 0) return v;
+  int rows = 0, cols = 0, splits = 1, tt = 0, ts = 1;
+  const int es = elem_bytes(in_dtype);
+  if (v == MI355_VARIANT_SKINNY) {
+    rows = M <= 16 ? 16 : M <= 32 ? 32 : M <= 64 ? 64 : M <= 128 ? 128 : 256;
+    cols = 64;
+    splits = mi355::stream_splits(M, N, K, es);
+  } else if (v == MI355_VARIANT_PINGPONG) {
+    rows = cols = 256;
+  } else if (v == MI355_VARIANT_BASIC) {
+    const int tile = mi355::ring_tile_edge(M, N, K, es);
+    rows = mi355::ring_tile_rows(tile);
+    cols = mi355::ring_tile_cols(tile);
+    splits = mi355::ring_splits(M, N, K, es);
+    if (splits == 1) mi355::ring_tail(M, N, K, es, &tt, &ts);
+  }
+  if (tile_rows) *tile_rows = rows;
+  if (tile_cols) *tile_cols = cols;
+  if (k_splits) *k_splits = splits;
+  if (tail_tiles) *tail_tiles = tt;
+  if (tail_splits) *tail_splits = ts;
+  return v;
+}
+
 size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int in_dtype, int variant) {
   if (!valid_in(in_dtype) || M <= 0 || N <= 0 || K <= 0) return 0;
   if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_SIMPLE) return 0;
@@ -284,8 +314,8 @@ int mi355_gemm_tn_scaled(const void* A, const void* B, void* C, int64_t M, int64
         }
       }
     }
-    g.tiles_m = (M + tile - 1) / tile;
-    g.tiles_n = (N + tile - 1) / tile;
+    g.tiles_m = (M + mi355::ring_tile_rows(tile) - 1) / mi355::ring_tile_rows(tile);
+    g.tiles_n = (N + mi355::ring_tile_cols(tile) - 1) / mi355::ring_tile_cols(tile);
     rc = v == MI355_VARIANT_PINGPONG ? mi355::launch_tile256_pingpong(g, in_dtype, out_dtype, s)
                                      : mi355::launch_tile_ring(g, in_dtype, out_dtype, tile, s);
   } else {

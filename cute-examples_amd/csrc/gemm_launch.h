@@ -46,8 +46,11 @@ __device__ __forceinline__ float output_scale(const GemmArgs& g) {
 // Each returns 0 after a successful enqueue, non-zero if the runtime rejected the launch.
 // in_dtype / out_dtype use the numbering of enum mi355_dtype.
 int launch_tile256_pingpong(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
-// Single-wave-group ring kernel; tile is 256 or 128 (ring_tile_edge and ring_splits are pure host
-// heuristics).
+// Single-wave-group ring kernel.  `tile` is 256 or 128 (square tiles) or kRingTile256x128 (256 rows
+// of A by 128 rows of B); ring_tile_edge, ring_splits and ring_tail are pure host heuristics.
+constexpr int kRingTile256x128 = 384;
+inline int ring_tile_rows(int tile) { return tile == 128 ? 128 : 256; }
+inline int ring_tile_cols(int tile) { return tile == 256 ? 256 : 128; }
 int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes);
 int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes);
 // C = rne(scale * sum_s partial[s]) for partial laid out [splits][M][N] in fp32.

@@ -162,7 +162,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_pingpong(GemmArgs
 
   const float scale = output_scale(g);
   auto epilogue = [&](int64_t m0, int64_t n0) __attribute__((always_inline)) {
-    store_output_tile<G, OutT, kNbA, kNbB, false>(acc, g, m0, n0, kTile, wm * 128, wn * 64, lane, scale);
+    store_output_tile<G, OutT, kNbA, kNbB, false>(acc, g, m0, n0, kTile, kTile, wm * 128, wn * 64, lane, scale);
   };
 
   const uint32_t tiles_m = (uint32_t)g.tiles_m, tiles_n = (uint32_t)g.tiles_n;  // below 2^31 tiles (launcher)

@@ -82,19 +82,25 @@ constexpr uint32_t kMxUnitBytes = 512;
 // kTileT: rows of A and of B per workgroup, 256 or 128.  The 128 variant (64x64 per wave, 80 KiB
 // ring, two workgroups per CU) is for problems with too few 256x256 tiles to occupy the CUs; it
 // moves twice the bytes per flop, so it is copy-bound at about two thirds of the MFMA rate.
-template <class T, class OutT, bool kRaggedK, int kTileT, int kWavesN = 2>
+// kTileNT: rows of B per workgroup when they differ from kTileT: the 256x128 tile (128x64 per wave)
+// has three times as many tiles as 256x256 on shapes that leave most CUs without a 256x256 tile,
+// and moves 1.5 times the bytes per flop instead of the 128x128 tile's two times.
+template <class T, class OutT, bool kRaggedK, int kTileT, int kWavesN = 2, int kTileNT = kTileT>
 __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void gemm_tn_tile_ring(GemmArgs g) {
-  constexpr int kTile = kTileT;
-  constexpr int kSlotBytes = kTile * kRowBytes;   // one operand, one k-step
+  constexpr int kTile = kTileT;                   // rows of A per workgroup
+  constexpr int kTileN = kTileNT;                 // rows of B per workgroup
+  static_assert(kTileN <= kTile, "a slot is sized for the rows of A");
+  constexpr int kSlotBytes = kTile * kRowBytes;   // one operand, one k-step (B may use less of it)
   constexpr int kWaveTileM = kTile / 2;           // rows (of A) per wave
-  constexpr int kWaveTileN = kTile / kWavesN;     // columns (rows of B) per wave
+  constexpr int kWaveTileN = kTileN / kWavesN;    // columns (rows of B) per wave
   constexpr int kWaves = 2 * kWavesN;
   // One direct-to-LDS instruction moves 16 B per lane: 8 rows of 128 B.  (4 B per lane, 2 rows,
   // costs an MFMA stream nothing per instruction in isolation, but four times as many copies
   // through the texture-address unit made the kernel 11 % slower.)
   constexpr int kCopyRows = 8;
   constexpr int kCopyBytes = kCopyRows * kRowBytes;
-  constexpr int kCph = kTile / kWaves / kCopyRows;  // copies per operand per k-step per wave
+  constexpr int kCph = kTile / kWaves / kCopyRows;    // copies of A per k-step per wave
+  constexpr int kCphB = kTileN / kWaves / kCopyRows;  // copies of B
   constexpr int kPar = 2;                           // copies j and j+kPar share their per-lane swizzle
   __shared__ __attribute__((aligned(1024))) uint8_t ring[kSlots * kSlotBytes];
   typedef typename RingGeo<T>::type G;
@@ -164,11 +170,11 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     return make_raw_buffer((const uint8_t*)g.A + m0 * (int64_t)lda_b, (uint32_t)((rows - 1) * lda_b + k_bytes));
   };
   auto panel_b = [&](int64_t n0) __attribute__((always_inline)) {
-    const int64_t rows = g.N - n0 < kTile ? g.N - n0 : kTile;
+    const int64_t rows = g.N - n0 < kTileN ? g.N - n0 : kTileN;
     return make_raw_buffer((const uint8_t*)g.B + n0 * (int64_t)ldb_b, (uint32_t)((rows - 1) * ldb_b + k_bytes));
   };
 
-  // Copy geometry.  Wave w fills rows [w*kTile/4, (w+1)*kTile/4) of a slot, kCopyRows rows per
+  // Copy geometry.  Wave w fills a quarter of an operand's rows in a slot, kCopyRows rows per
   // instruction, the LDS side linear in the lane number.  Lane l therefore fills bytes
   // sub..sub+n of LDS chunk lchunk of row lrow of the copy's rows, and fetches them from global
   // chunk lchunk ^ swizzle(row).  swizzle(row) repeats every kPar copies, so kPar per-lane
@@ -180,7 +186,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   for (int par = 0; par < kPar; ++par) {
     const uint32_t chunk = lchunk ^ swizzle(par * kCopyRows + lrow);
     voff_a[par] = (wave * (kCph * kCopyRows) + lrow) * lda_b + chunk * 16;
-    voff_b[par] = (wave * (kCph * kCopyRows) + lrow) * ldb_b + chunk * 16;
+    voff_b[par] = (wave * (kCphB * kCopyRows) + lrow) * ldb_b + chunk * 16;
     if constexpr (kRaggedK) {
       const bool tail_or_oob = tail_bytes != 0 && chunk * 16 >= tail_bytes;
       tail_a[par] = tail_or_oob ? kOutOfRange : voff_a[par];
@@ -190,7 +196,8 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   const uint32_t a_step = __builtin_amdgcn_readfirstlane(kCopyRows * lda_b);
   const uint32_t b_step = __builtin_amdgcn_readfirstlane(kCopyRows * ldb_b);
   const uint32_t ring0 = __builtin_amdgcn_readfirstlane(lds_address(ring));
-  const uint32_t dma_wave = ring0 + wave * (kCph * kCopyBytes);  // this wave's share of a slot
+  const uint32_t dma_wave_a = ring0 + wave * (kCph * kCopyBytes);  // this wave's share of a slot
+  const uint32_t dma_wave_b = ring0 + wave * (kCphB * kCopyBytes);
 
   // Copy j of an operand's k-step into slot `slot`; soff is the k-step's byte offset inside a row.
   // The row part of the address stays in the vector offset, the only part the hardware
@@ -199,7 +206,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   // k-step, into a slot nobody reads, so the loop body stays branch-free.
   const uint32_t soff_tail = (k_steps - 1) * kRowBytes;  // the k-step that may be ragged
   auto copy_rows = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, auto slotc, uint32_t soff, const uint32_t* voff,
-                       const uint32_t* tail, uint32_t step) __attribute__((always_inline)) {
+                       const uint32_t* tail, uint32_t step, uint32_t dma_wave) __attribute__((always_inline)) {
     constexpr int j = decltype(jc)::value;
     constexpr uint32_t slot = decltype(slotc)::value;
     uint32_t v = voff[j % kPar];
@@ -207,10 +214,10 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     dma_16B_to_lds_at<slot * kSlotBytes + j * kCopyBytes>(dma_wave, v + j * step, rsrc, soff);
   };
   auto copy_a = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, auto slotc, uint32_t soff) __attribute__((always_inline)) {
-    copy_rows(rsrc, jc, slotc, soff, voff_a, tail_a, a_step);
+    copy_rows(rsrc, jc, slotc, soff, voff_a, tail_a, a_step, dma_wave_a);
   };
   auto copy_b = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, auto slotc, uint32_t soff) __attribute__((always_inline)) {
-    copy_rows(rsrc, jc, slotc, soff, voff_b, tail_b, b_step);
+    copy_rows(rsrc, jc, slotc, soff, voff_b, tail_b, b_step, dma_wave_b);
   };
   // Byte offset of k-step kt of the item that starts at global k-step step0, clamped to its last.
   auto soff_of = [&](uint32_t step0, uint32_t kt) __attribute__((always_inline)) -> uint32_t {
@@ -239,9 +246,9 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   auto open_tile = [&](__amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb, uint32_t step0) __attribute__((always_inline)) {
     const uint32_t s0 = soff_of(step0, 0), s1 = soff_of(step0, 1), s2 = soff_of(step0, 2);
     static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, std::integral_constant<uint32_t, 0>{}, s0); });
-    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, std::integral_constant<uint32_t, 1>{}, s0); });
+    static_for<kCphB>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, std::integral_constant<uint32_t, 1>{}, s0); });
     static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, std::integral_constant<uint32_t, 2>{}, s1); });
-    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, std::integral_constant<uint32_t, 3>{}, s1); });
+    static_for<kCphB>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, std::integral_constant<uint32_t, 3>{}, s1); });
     static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, std::integral_constant<uint32_t, 4>{}, s2); });
   };
 
@@ -306,17 +313,17 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   const float scale = output_scale(g);
   constexpr bool kAsmMfma = kTile == 256;  // see mfma_u
   auto epilogue = [&](int64_t m0, int64_t n0) __attribute__((always_inline)) {
-    store_output_tile<G, OutT, kNbM, kNbN, kAsmMfma>(acc, g, m0, n0, kTile, wm * kWaveTileM, wn * kWaveTileN, lane, scale);
+    store_output_tile<G, OutT, kNbM, kNbN, kAsmMfma>(acc, g, m0, n0, kTile, kTileN, wm * kWaveTileM, wn * kWaveTileN, lane, scale);
   };
   auto store_partial = [&](int64_t m0, int64_t n0, uint32_t split, uint32_t tile_no) __attribute__((always_inline)) {
     if (tail_tiles) {
       // a whole tile of the compact tail workspace (rows past M hold zeros: their operands read as 0)
-      float* base = g.partial + ((int64_t)split * tail_tiles + (tile_no - whole_tiles)) * (kTile * kTile);
-      store_partial_tile<G, kNbM, kNbN, kAsmMfma>(acc, base, kTile, kTile, kTile, wm * kWaveTileM, wn * kWaveTileN, lane);
+      float* base = g.partial + ((int64_t)split * tail_tiles + (tile_no - whole_tiles)) * (kTile * kTileN);
+      store_partial_tile<G, kNbM, kNbN, kAsmMfma>(acc, base, kTileN, kTile, kTileN, wm * kWaveTileM, wn * kWaveTileN, lane);
     } else {
       // plane `split` of M x N floats, clipped at the matrix edge
       const int64_t rows = g.M - m0 < kTile ? g.M - m0 : kTile;
-      const uint32_t cols = (uint32_t)(g.N - n0 < kTile ? g.N - n0 : kTile);
+      const uint32_t cols = (uint32_t)(g.N - n0 < kTileN ? g.N - n0 : kTileN);
       float* base = g.partial + ((int64_t)split * g.M + m0) * g.N + n0;
       store_partial_tile<G, kNbM, kNbN, kAsmMfma>(acc, base, (uint32_t)g.N, rows, cols, wm * kWaveTileM, wn * kWaveTileN, lane);
     }
@@ -327,7 +334,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   bool partial_item = decode_item(item, &tile_no, &split);
   tile_coord_t<uint32_t>(tile_no, tiles_m, tiles_n, &tile_m, &tile_n);
   uint32_t step0 = __builtin_amdgcn_readfirstlane(split * steps);  // first k-step of the current item
-  __amdgpu_buffer_rsrc_t rsrc_a = panel_a((int64_t)tile_m * kTile), rsrc_b = panel_b((int64_t)tile_n * kTile);
+  __amdgpu_buffer_rsrc_t rsrc_a = panel_a((int64_t)tile_m * kTile), rsrc_b = panel_b((int64_t)tile_n * kTileN);
   if constexpr (kMx) mx_open_tile(tile_m, tile_n, step0);  // before the copies: see the waits
   open_tile(rsrc_a, rsrc_b, step0);
 
@@ -340,7 +347,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
         for (int r = 0; r < kAccLen; ++r) acc[i][j][r] = 0.f;
 
     // A0 and B0 have landed; A1, B1, A2 may be in flight (the counter saturates at 63).
-    wait_vmcnt<(3 * kCph < 63 ? 3 * kCph : 63)>();
+    wait_vmcnt<(2 * kCph + kCphB < 63 ? 2 * kCph + kCphB : 63)>();
     __builtin_amdgcn_s_barrier();
     if constexpr (kRowSliced) {
 #pragma unroll
@@ -388,7 +395,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
       constexpr int kBarrierWant = kLastOwnRead + 1 + kMfmaPerSlice / 8;
       constexpr int kBarrierAt = kBarrierWant < kMfmaPerSlice ? kBarrierWant : kMfmaPerSlice - 1;
       constexpr int kFirstCopy = kBarrierAt + 1;
-      constexpr int kCopies = 2 * kCph;                                  // B(t+2) then A(t+3)
+      constexpr int kCopies = kCphB + kCph;                              // B(t+2) then A(t+3)
       constexpr int kCopySpan = 2 * kMfmaPerSlice - kFirstCopy;          // positions left in the k-step
       static_assert(kCopySpan > 0, "no room for the copies");
       // copy c is issued at position kFirstCopy + c * kCopySpan / kCopies (evenly spread)
@@ -430,10 +437,10 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
           static_for<kMaxCopiesPerGap>([&](auto ic) __attribute__((always_inline)) {
             constexpr int c = c0 + decltype(ic)::value;
             if constexpr (c < kCopies && copy_position(c, kFirstCopy, kCopySpan, kCopies) == p) {
-              if constexpr (c < kCph)
+              if constexpr (c < kCphB)
                 copy_b(rsrc_b, std::integral_constant<int, c>{}, std::integral_constant<uint32_t, slot_a>{}, soff_b);
               else
-                copy_a(rsrc_a, std::integral_constant<int, c - kCph>{}, std::integral_constant<uint32_t, slot_b>{}, soff_a);
+                copy_a(rsrc_a, std::integral_constant<int, c - kCphB>{}, std::integral_constant<uint32_t, slot_b>{}, soff_a);
             }
           });
         }
@@ -456,7 +463,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     wait_lgkmcnt0();
     __builtin_amdgcn_s_barrier();
 
-    const int64_t done_m0 = (int64_t)tile_m * kTile, done_n0 = (int64_t)tile_n * kTile;
+    const int64_t done_m0 = (int64_t)tile_m * kTile, done_n0 = (int64_t)tile_n * kTileN;
     const uint32_t done_split = split, done_tile = tile_no;
     const bool done_partial = partial_item;
     item += gridDim.x;
@@ -466,7 +473,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
       tile_coord_t<uint32_t>(tile_no, tiles_m, tiles_n, &tile_m, &tile_n);
       step0 = __builtin_amdgcn_readfirstlane(split * steps);
       rsrc_a = panel_a((int64_t)tile_m * kTile);
-      rsrc_b = panel_b((int64_t)tile_n * kTile);
+      rsrc_b = panel_b((int64_t)tile_n * kTileN);
       if constexpr (kMx) mx_open_tile(tile_m, tile_n, step0);
       open_tile(rsrc_a, rsrc_b, step0);  // in flight while the finished tile is stored
     }
@@ -478,27 +485,27 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
 
 // C tiles of a tail split: rne(scale * (partial[0] + ... + partial[S-1])) in that order, for the
 // last g.tail_tiles tiles in tile-map order; one thread per 4 consecutive columns.
-template <class OutT, int kTileT>
+template <class OutT, int kTileT, int kTileNT>
 __global__ __launch_bounds__(256) void tail_reduce(GemmArgs g) {
-  constexpr uint32_t kQuadsPerTile = kTileT * kTileT / 4;
+  constexpr uint32_t kQuadsPerTile = kTileT * kTileNT / 4;
   const uint32_t q = blockIdx.x * 256u + threadIdx.x;
   const uint32_t t = q / kQuadsPerTile, in_tile = q % kQuadsPerTile;
   if (t >= (uint32_t)g.tail_tiles) return;
-  const uint32_t r = in_tile / (kTileT / 4), c = (in_tile % (kTileT / 4)) * 4;
+  const uint32_t r = in_tile / (kTileNT / 4), c = (in_tile % (kTileNT / 4)) * 4;
   uint32_t tile_m, tile_n;
   tile_coord_t<uint32_t>((uint32_t)(g.tiles_m * g.tiles_n) - (uint32_t)g.tail_tiles + t, (uint32_t)g.tiles_m,
                          (uint32_t)g.tiles_n, &tile_m, &tile_n);
-  const int64_t m = (int64_t)tile_m * kTileT + r, n = (int64_t)tile_n * kTileT + c;
+  const int64_t m = (int64_t)tile_m * kTileT + r, n = (int64_t)tile_n * kTileNT + c;
   if (m >= g.M || n >= g.N) return;  // N % 4 == 0: a quad is in or out as a whole
-  const float* p = g.partial + (int64_t)t * (kTileT * kTileT) + r * kTileT + c;
-  const int64_t split_stride = (int64_t)g.tail_tiles * (kTileT * kTileT);
+  const float* p = g.partial + (int64_t)t * (kTileT * kTileNT) + r * kTileNT + c;
+  const int64_t split_stride = (int64_t)g.tail_tiles * (kTileT * kTileNT);
   f32x4 sum = *(const f32x4*)p;
   for (int s = 1; s < g.tail_splits; ++s) sum += *(const f32x4*)(p + s * split_stride);
   const float scale = output_scale(g);
   *(u32x2*)((uint16_t*)g.C + m * g.ldc + n) = Pack4<OutT>::run(sum[0] * scale, sum[1] * scale, sum[2] * scale, sum[3] * scale);
 }
 
-template <class T, class OutT, int kTileT>
+template <class T, class OutT, int kTileT, int kTileNT = kTileT>
 int launch_tile(const GemmArgs& g, hipStream_t stream) {
   const int64_t items = g.tail_tiles ? g.tiles_m * g.tiles_n + (int64_t)g.tail_tiles * (g.tail_splits - 1)
                                      : g.tiles_m * g.tiles_n * g.splits;
@@ -507,17 +514,17 @@ int launch_tile(const GemmArgs& g, hipStream_t stream) {
   const int64_t blocks = items < slots ? items : slots;
   constexpr int kWavesN = 2;
   if ((g.K * T::kBytes) % kRowBytes == 0) {
-    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, false, kTileT, kWavesN>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
+    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, false, kTileT, kWavesN, kTileNT>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
   } else {
     if constexpr (std::is_same<T, MxE4M3>::value) return -1;  // block scales need whole k-steps (host check)
-    else hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, true, kTileT, kWavesN>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
+    else hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, true, kTileT, kWavesN, kTileNT>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
   }
   if (hipGetLastError() != hipSuccess) return -1;
   if (g.splits > 1)
     return launch_splitk_reduce(g.partial, g, std::is_same<OutT, BF16>::value ? 0 : 1, stream);
   if (g.tail_tiles) {
-    const int64_t quads = (int64_t)g.tail_tiles * (kTileT * kTileT / 4);
-    hipLaunchKernelGGL((tail_reduce<OutT, kTileT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, g);
+    const int64_t quads = (int64_t)g.tail_tiles * (kTileT * kTileNT / 4);
+    hipLaunchKernelGGL((tail_reduce<OutT, kTileT, kTileNT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, g);
     if (hipGetLastError() != hipSuccess) return -1;
   }
   return 0;
@@ -525,87 +532,11 @@ int launch_tile(const GemmArgs& g, hipStream_t stream) {
 
 template <class T, class OutT>
 int launch(const GemmArgs& g, int tile, hipStream_t stream) {
+  if (tile == kRingTile256x128) return launch_tile<T, OutT, 256, 128>(g, stream);
   return tile == 128 ? launch_tile<T, OutT, 128>(g, stream) : launch_tile<T, OutT, 256>(g, stream);
 }
 
 }  // namespace
-
-namespace {
-
-constexpr int64_t kSlots256 = 256;  // resident workgroups of 256x256 tiles on an MI355X (one per CU);
-                                    // heuristics only, so no device query here
-
-// Tail split of `tiles` 256x256 tiles with `steps` k-steps each.  When the tiles fill one or two
-// rounds of workgroups plus a last round that is at most half full, the tiles of that round are cut
-// along K so that they occupy (almost) all workgroup slots and the round takes 1/S of a tile's
-// time; every item keeps at least 16 k-steps and the k-steps divide evenly, as in ring_splits.
-// Measured at bf16: +5..+10 % for one or two full rounds (4096x6144x4096, 6144^3); with three
-// full rounds (4096x14336x4096) the partly filled round, which runs at a higher clock, costs no
-// more than the partial tiles' extra traffic and second launch (-1 %), and on 128x128 tiles the
-// split loses (-8 % at 4352^2x4096), so those are never cut.
-void tail_plan(int64_t tiles, int64_t steps, int* tail_tiles, int* tail_splits) {
-  *tail_tiles = 0;
-  *tail_splits = 1;
-  const int64_t rest = tiles % kSlots256;
-  if (tiles < kSlots256 || tiles > 3 * kSlots256 || rest == 0) return;
-  int best = 1;
-  for (int s = 2; s <= 16; ++s) {
-    if (rest * s > kSlots256) break;
-    if (steps % s != 0 || steps / s < 16) continue;
-    best = s;
-  }
-  if (best == 1) return;
-  *tail_tiles = (int)rest;
-  *tail_splits = best;
-}
-
-int64_t k_steps_of(int64_t K, int elem_bytes) { return (K * elem_bytes + kRowBytes - 1) / kRowBytes; }
-
-}  // namespace
-
-// Tile edge the single-group kernel should use: 256 unless that leaves most CUs idle and the
-// 128x128 variant (about 0.36 of a 256-tile's time per tile, up to two per CU) finishes sooner.
-// A last round of 256-tiles that gets a tail split counts as 1/S of a round plus 0.2 for the
-// partial tiles' traffic and the second launch (measured 0.12..0.25).
-int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes) {
-  const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
-  const int64_t t128 = ((M + 127) / 128) * ((N + 127) / 128);
-  int tail_tiles, tail_splits;
-  tail_plan(t256, k_steps_of(K, elem_bytes), &tail_tiles, &tail_splits);
-  const double time256 = tail_tiles ? (double)(t256 / kSlots256) + 1.0 / tail_splits + 0.2
-                                    : (double)((t256 + kSlots256 - 1) / kSlots256);
-  const double time128 = (double)((t128 + kSlots256 - 1) / kSlots256) * 0.36;
-  return time128 < time256 ? 128 : 256;
-}
-
-// K splits for the single-group kernel: only when the tiles alone leave more than half of the CUs
-// idle (the partial tiles cost S*M*N*8 bytes of extra traffic and a second launch), the k-steps
-// divide evenly and every item keeps at least 16 k-steps.
-int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
-  const int tile = ring_tile_edge(M, N, K, elem_bytes);
-  const int64_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile);
-  // One item per CU of an MI355X, also for the 128x128 tiles (two of which fit a CU): filling
-  // both places with K splits measured 7-13 % slower on M = 128..256 against N = 14336.
-  const int64_t slots = 256;  // one item per CU of an MI355X
-  const int64_t steps = k_steps_of(K, elem_bytes);
-  int best = 1;
-  for (int s = 2; s <= 16; ++s) {
-    if (tiles * s > slots) break;
-    if (steps % s != 0 || steps / s < 16) continue;
-    best = s;
-  }
-  return best;
-}
-
-// The tail split (tail_plan) of this problem, if it runs on 256x256 tiles without a uniform K
-// split: returns the workspace bytes of its partial tiles.
-size_t ring_tail(int64_t M, int64_t N, int64_t K, int elem_bytes, int* tail_tiles, int* tail_splits) {
-  *tail_tiles = 0;
-  *tail_splits = 1;
-  if (M <= 0 || N <= 0 || K <= 0 || ring_tile_edge(M, N, K, elem_bytes) != 256) return 0;
-  tail_plan(((M + 255) / 256) * ((N + 255) / 256), k_steps_of(K, elem_bytes), tail_tiles, tail_splits);
-  return (size_t)*tail_tiles * (size_t)*tail_splits * 256 * 256 * sizeof(float);
-}
 
 int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, hipStream_t stream) {
   const bool out_bf16 = out_dtype == 0;

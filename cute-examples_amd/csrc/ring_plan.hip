@@ -1,0 +1,126 @@
+// Host-side planning for the single-group tile kernel (gemm_tn_ring.hip): which tile, whether to
+// split K uniformly, whether to cut the tiles of the last round.  Pure functions of the problem
+// size, so that the workspace query and the launch agree.  Counterpart in the reference: the
+// compile-time tile choice of DefaultConfig (kernels/gemm_kernels/sm90a/gemm.cuh:420-451) and the
+// Scheduler's round structure (gemm.cuh:168-212).
+#include "gemm_launch.h"
+#include "ring_common.h"
+
+namespace mi355 {
+
+namespace {
+
+constexpr int64_t kSlots = 256;  // one work item per CU of an MI355X; heuristics only, so no device query
+
+int64_t k_steps_of(int64_t K, int elem_bytes) { return (K * elem_bytes + kRowBytes - 1) / kRowBytes; }
+
+int64_t tiles_of(int64_t M, int64_t N, int tile) {
+  const int64_t r = ring_tile_rows(tile), c = ring_tile_cols(tile);
+  return ((M + r - 1) / r) * ((N + c - 1) / c);
+}
+
+// Uniform K split of `tiles` tiles: only when the tiles alone leave more than half of the CUs idle
+// (the partial tiles cost S*M*N*8 bytes of extra traffic and a second launch), the k-steps divide
+// evenly and every item keeps at least 16 k-steps.  One item per CU also for the 128x128 tiles
+// (two of which fit a CU): filling both places with K splits measured 7-13 % slower on
+// M = 128..256 against N = 14336.
+int uniform_splits(int64_t tiles, int64_t steps) {
+  int best = 1;
+  for (int s = 2; s <= 16; ++s) {
+    if (tiles * s > kSlots) break;
+    if (steps % s != 0 || steps / s < 16) continue;
+    best = s;
+  }
+  return best;
+}
+
+// Tail split of `tiles` 256x256 tiles with `steps` k-steps each.  When the tiles fill one or two
+// rounds of workgroups plus a last round that is at most half full, the tiles of that round are cut
+// along K so that they occupy (almost) all workgroup slots and the round takes 1/S of a tile's
+// time; same conditions on the k-steps as a uniform split.
+// Measured at bf16: +5..+10 % for one or two full rounds (4096x6144x4096, 6144^3); with three
+// full rounds (4096x14336x4096) the partly filled round, which runs at a higher clock, costs no
+// more than the partial tiles' extra traffic and second launch (-1 %), and on 128x128 tiles the
+// split loses (-8 % at 4352^2x4096), so only 256x256 tiles are cut.
+void tail_plan(int64_t tiles, int64_t steps, int* tail_tiles, int* tail_splits) {
+  *tail_tiles = 0;
+  *tail_splits = 1;
+  const int64_t rest = tiles % kSlots;
+  if (tiles < kSlots || tiles > 3 * kSlots || rest == 0) return;
+  int best = 1;
+  for (int s = 2; s <= 16; ++s) {
+    if (rest * s > kSlots) break;
+    if (steps % s != 0 || steps / s < 16) continue;
+    best = s;
+  }
+  if (best == 1) return;
+  *tail_tiles = (int)rest;
+  *tail_splits = best;
+}
+
+// Estimated duration, in microseconds, of the problem on tile shape `tile`, fitted to timings of
+// twenty mid-sized bf16 and fp8 problems per tile shape (mean regret of the choice 3 %):
+//   rounds x (k-steps per item x time of a k-step + start-up and store of a tile) + reduce
+// A k-step is 128 bytes of K per row for every input type and takes the same time for all of them.
+//   256x256  1.45 us when (nearly) all CUs are busy, 1.2 us otherwise (higher clock); a last round
+//            that gets a tail split counts 1/S of a round plus 0.2
+//   256x128  0.85 us: half the MFMA work of a 256x256 tile, three quarters of its copies
+//   128x128  0.5 us (a quarter of the work, half of the copies), 0.75 us when either dimension has
+//            fewer than 16 tiles (measured; such problems re-read one operand from far away)
+//   reduce   the partial planes are read back at about 5 TB/s, plus a launch
+double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
+  const int64_t rows = ring_tile_rows(tile), cols = ring_tile_cols(tile);
+  const int64_t tm = (M + rows - 1) / rows, tn = (N + cols - 1) / cols, tiles = tm * tn;
+  const int64_t steps = k_steps_of(K, elem_bytes);
+  const int s = uniform_splits(tiles, steps);
+  const int64_t items = tiles * s;
+  double rounds = (double)((items + kSlots - 1) / kSlots);
+  double step_us, fixed_us;
+  if (tile == 256) {
+    step_us = items >= 224 ? 1.45 : 1.2;
+    fixed_us = 6.0;
+    int tail_tiles, tail_splits;
+    tail_plan(tiles, steps, &tail_tiles, &tail_splits);
+    if (tail_tiles) rounds = (double)(tiles / kSlots) + 1.0 / tail_splits + 0.2;
+  } else if (tile == kRingTile256x128) {
+    step_us = 0.85;
+    fixed_us = 6.0;
+  } else {
+    step_us = (tm < tn ? tm : tn) >= 16 ? 0.5 : 0.75;
+    fixed_us = 4.0;
+  }
+  const double reduce_us = s > 1 ? (double)s * (double)M * (double)N * 4.0 / 5.0e6 + 2.0 : 0.0;
+  return rounds * ((double)steps / s * step_us + fixed_us) + reduce_us;
+}
+
+}  // namespace
+
+// Tile the single-group kernel should use (256, 128 or kRingTile256x128): the shortest estimate,
+// except that 128x128 is kept when nothing beats it by 10 % (the estimates of the small tile are
+// the least reliable, and it was the only alternative to 256x256 before) and 256x256 is preferred
+// over 256x128 within 5 % (it moves fewer bytes).
+int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes) {
+  const double e256 = estimate_us(256, M, N, K, elem_bytes);
+  const double e128 = estimate_us(128, M, N, K, elem_bytes);
+  const double e2 = estimate_us(kRingTile256x128, M, N, K, elem_bytes);
+  const double best_large = e256 <= 1.05 * e2 ? e256 : e2;
+  if (e128 <= 1.1 * best_large) return 128;
+  return e256 <= 1.05 * e2 ? 256 : kRingTile256x128;
+}
+
+// K splits for the single-group kernel on the tile ring_tile_edge picks.
+int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
+  return uniform_splits(tiles_of(M, N, ring_tile_edge(M, N, K, elem_bytes)), k_steps_of(K, elem_bytes));
+}
+
+// The tail split (tail_plan) of this problem, if it runs on 256x256 tiles without a uniform K
+// split: returns the workspace bytes of its partial tiles.
+size_t ring_tail(int64_t M, int64_t N, int64_t K, int elem_bytes, int* tail_tiles, int* tail_splits) {
+  *tail_tiles = 0;
+  *tail_splits = 1;
+  if (M <= 0 || N <= 0 || K <= 0 || ring_tile_edge(M, N, K, elem_bytes) != 256) return 0;
+  tail_plan(tiles_of(M, N, 256), k_steps_of(K, elem_bytes), tail_tiles, tail_splits);
+  return (size_t)*tail_tiles * (size_t)*tail_splits * 256 * 256 * sizeof(float);
+}
+
+}  // namespace mi355

@@ -44,12 +44,12 @@ __device__ __forceinline__ void pin_acc_block(Acc& a) {
   if constexpr (kPinned) asm volatile("" : "+a"(a));
 }
 
-// The wave's part of the output tile at (m0, n0), tile_edge rows and columns at most.
+// The wave's part of the output tile at (m0, n0), tile_rows x tile_cols at most.
 // wave_row / wave_col: first row / column of the wave inside the tile.
 template <class G, class OutT, int kNbM, int kNbN, bool kAsmRead>
 __device__ __forceinline__ void store_output_tile(typename G::Acc (&acc)[kNbM][kNbN], const GemmArgs& g,
-                                                  int64_t m0, int64_t n0, int tile_edge, uint32_t wave_row,
-                                                  uint32_t wave_col, uint32_t lane, float scale) {
+                                                  int64_t m0, int64_t n0, int tile_rows, int tile_cols,
+                                                  uint32_t wave_row, uint32_t wave_col, uint32_t lane, float scale) {
   typedef typename G::Acc Acc;
   constexpr int kBlk = G::kBlk;
   // Non-temporal, write-through stores (nt + sc1) keep C out of L2: it is written once and would
@@ -58,8 +58,8 @@ __device__ __forceinline__ void store_output_tile(typename G::Acc (&acc)[kNbM][k
   // not (32 bytes: measured 3 % slower with sc1, 25 % with nt + sc1).
   constexpr int kAux = kBlk == 16 ? 18 : 0;
   const uint32_t rblk = lane & (kBlk - 1), grp = lane / kBlk;
-  const int64_t rows = g.M - m0 < tile_edge ? g.M - m0 : tile_edge;
-  const uint32_t cols = (uint32_t)(g.N - n0 < tile_edge ? g.N - n0 : tile_edge);
+  const int64_t rows = g.M - m0 < tile_rows ? g.M - m0 : tile_rows;
+  const uint32_t cols = (uint32_t)(g.N - n0 < tile_cols ? g.N - n0 : tile_cols);
   const uint32_t ldc_b = (uint32_t)g.ldc * 2;
   const __amdgpu_buffer_rsrc_t rc =
       make_raw_buffer((const uint16_t*)g.C + m0 * g.ldc + n0, (uint32_t)(((rows - 1) * g.ldc + cols) * 2));
@@ -106,7 +106,7 @@ __device__ __forceinline__ void store_output_tile(typename G::Acc (&acc)[kNbM][k
       }
     });
   };
-  if (cols == (uint32_t)tile_edge) {
+  if (cols == (uint32_t)tile_cols) {
     convert([&](auto ic, auto colc, u32x2 x, u32x2 y) __attribute__((always_inline)) {
       constexpr int i = decltype(ic)::value, col = decltype(colc)::value;
       store_16B_guarded<kAux>((u32x4){x[0], x[1], y[0], y[1]}, rc, v0 + col * 2, i * block_step);

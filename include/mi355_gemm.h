@@ -177,6 +177,16 @@ int mi355_quantize_mxfp8(const void *x, int x_dtype, int64_t rows, int64_t K, in
 size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K,
                                   int in_dtype, int variant);
 
+/* What mi355_gemm_tn would launch for this problem: the resolved variant (return value, or a
+ * negative mi355_status), and for the tiled variants the tile (rows of A x rows of B per
+ * workgroup), the uniform K split and the tail split (tiles of the last round cut along K;
+ * 0 tiles / 1 split when there is none).  For the skinny variant tile_rows x 64 and its K split.
+ * Any output pointer may be NULL.  Pure host function.  Counterpart in the reference: the
+ * compile-time DefaultConfig (kernels/gemm_kernels/sm90a/gemm.cuh:420-451). */
+int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant,
+                    int *tile_rows, int *tile_cols, int *k_splits,
+                    int *tail_tiles, int *tail_splits);
+
 /* The variant MI355_VARIANT_AUTO resolves to for this problem (an enum mi355_variant value),
  * or a negative mi355_status.  Replaces the compile-time choice of kernel header at
  * kernels/gemm_kernels/sm90a/gemm_test.cu:7 / kernels/setup.py:12-15. */

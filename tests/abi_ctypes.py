@@ -46,6 +46,9 @@ def load():
     L.mi355_quantize_mxfp8.restype = ci
     L.mi355_gemm_workspace_bytes.argtypes = [i64, i64, i64, ci, ci]
     L.mi355_gemm_workspace_bytes.restype = sz
+    ip = ctypes.POINTER(ctypes.c_int)
+    L.mi355_gemm_plan.argtypes = [i64, i64, i64, ci, ci, ip, ip, ip, ip, ip]
+    L.mi355_gemm_plan.restype = ci
     L.mi355_gemm_select_variant.argtypes = [i64, i64, i64, ci]
     L.mi355_gemm_select_variant.restype = ci
     L.mi355_gemm_check.argtypes = [i64, i64, i64, i64, i64, i64, ci, ci, ci]
@@ -102,3 +105,10 @@ def gemm_tn_mxfp8(L, A_q, B_q, sa, sb, C, shuffled=False, stream=None):
     return L.mi355_gemm_tn_mxfp8(A_q.data_ptr(), B_q.data_ptr(), C.data_ptr(), M, N, K, A_q.stride(0),
                                  B_q.stride(0), C.stride(0), sa.data_ptr(), sa.stride(0), sb.data_ptr(),
                                  sb.stride(0), 0, out_dt, ws.data_ptr(), ws_bytes, s)
+
+
+def plan(L, M, N, K, in_dt, variant=AUTO):
+    """(variant, tile_rows, tile_cols, k_splits, tail_tiles, tail_splits) from mi355_gemm_plan."""
+    v = [ctypes.c_int() for _ in range(5)]
+    rc = L.mi355_gemm_plan(M, N, K, in_dt, variant, *[ctypes.byref(x) for x in v])
+    return (rc,) + tuple(x.value for x in v)

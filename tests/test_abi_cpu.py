@@ -115,7 +115,8 @@ def test_workspace_bytes(abi):
     assert f(8192, 8192, 8192, ac.BF16, ac.AUTO) == 0
     assert f(8192, 8192, 8192, ac.BF16, ac.BASIC) == 0
     assert f(8192, 8192, 8192, ac.BF16, ac.PINGPONG) == 0
-    assert f(256, 4096, 14336, ac.BF16, ac.BASIC) == 4 * 256 * 4096 * 4        # 64 tiles of 128x128 -> 4 K splits
+    assert f(256, 4096, 14336, ac.BF16, ac.BASIC) == 8 * 256 * 4096 * 4        # 32 tiles of 256x128 -> 8 K splits
+    assert ac.plan(abi, 256, 4096, 14336, ac.BF16, ac.BASIC) == (ac.BASIC, 256, 128, 8, 0, 1)
     assert f(16, 512, 128, ac.BF16, ac.SKINNY) == 0              # too few k-steps to split
     need = f(16, 4096, 14336, ac.BF16, ac.AUTO)
     assert need > 0 and need % (16 * 4096 * 4) == 0 and need // (16 * 4096 * 4) <= 16
@@ -132,6 +133,28 @@ def test_workspace_bytes(abi):
     assert f(6144, 6144, 6144, ac.BF16, ac.BASIC) == 4 * 64 * 256 * 256 * 4    # two full rounds + 64 tiles cut in four
     assert f(4096, 14336, 4096, ac.BF16, ac.BASIC) == 0         # three full rounds: not worth it
     assert f(4096, 6144, 4096, ac.BF16, ac.PINGPONG) == 0
+
+
+def test_plan(abi):
+    """mi355_gemm_plan reports what a call would launch; the workspace query must agree with it."""
+    assert ac.plan(abi, 8192, 8192, 8192, ac.BF16) == (ac.BASIC, 256, 256, 1, 0, 1)
+    assert ac.plan(abi, 8192, 8192, 8192, ac.E4M3, ac.PINGPONG) == (ac.PINGPONG, 256, 256, 1, 0, 1)
+    assert ac.plan(abi, 4096, 6144, 4096, ac.BF16) == (ac.BASIC, 256, 256, 1, 128, 2)       # tail split
+    assert ac.plan(abi, 512, 14336, 4096, ac.BF16) == (ac.BASIC, 256, 128, 1, 0, 1)         # 224 rectangular tiles
+    assert ac.plan(abi, 2048, 2048, 2048, ac.F16) == (ac.BASIC, 128, 128, 1, 0, 1)          # 256 small tiles
+    assert ac.plan(abi, 512, 6144, 4096, ac.BF16) == (ac.BASIC, 256, 256, 4, 0, 1)          # 48 tiles cut in four
+    v, rows, cols, splits, _, _ = ac.plan(abi, 16, 14336, 4096, ac.BF16)
+    assert (v, rows, cols) == (ac.SKINNY, 16, 64) and splits >= 2
+    assert ac.plan(abi, 100, 30, 77, ac.BF16)[0] == ac.SIMPLE
+    assert ac.plan(abi, 256, 256, 68, ac.BF16, ac.BASIC)[0] == ac.ERR_SHAPE
+    assert ac.plan(abi, 256, 256, 64, 7)[0] == ac.ERR_DTYPE
+    assert abi.mi355_gemm_plan(256, 256, 64, ac.BF16, ac.AUTO, None, None, None, None, None) == ac.BASIC
+    for dt, es in ((ac.BF16, 2), (ac.E4M3, 1)):
+        for (M, N, K) in [(512, 6144, 4096), (1024, 6144, 4096), (256, 4096, 14336), (768, 768, 8192), (4352, 4352, 4096),
+                          (300, 1000, 2048), (6144, 6144, 6144), (64, 4096, 14336)]:
+            v, rows, cols, splits, tail_tiles, tail_splits = ac.plan(abi, M, N, K, dt)
+            want = splits * M * N * 4 if splits > 1 else tail_tiles * tail_splits * rows * cols * 4
+            assert abi.mi355_gemm_workspace_bytes(M, N, K, dt, ac.AUTO) == want, (dt, M, N, K)
 
 
 def test_select_variant(abi):

@@ -252,6 +252,49 @@ def test_tail_split(abi, dt, M, N, K):
     assert 0.5 < same < 1.0 or dt == torch.float8_e4m3fn, same
 
 
+@pytest.mark.parametrize("dt,M,N,K", [
+    (torch.bfloat16, 512, 14336, 4096),        # 2 x 112 tiles
+    (torch.bfloat16, 500, 14000, 4104),        # ragged rows, columns and last k-step
+    (torch.float16, 256, 4096, 14336),         # 32 tiles, K split 8 ways
+    (torch.float8_e4m3fn, 1024, 6144, 4096),
+    (torch.float8_e4m3fn, 1000, 6100, 4112),   # ragged; 4112 fp8 bytes = 32 k-steps + 16 bytes
+    (torch.float8_e4m3fn, 256, 4096, 14336),   # K split 7 ways
+    (torch.bfloat16, 768, 768, 8192),          # 3 x 6 tiles, K split 8 ways
+])
+def test_rectangular_tile(abi, dt, M, N, K):
+    """Problems the planner gives the 256x128 tile: against the oracle and, element by element,
+    against the one-thread-per-output kernel; twice for determinism."""
+    v, rows, cols, splits, _, _ = ac.plan(abi, M, N, K, ac.torch_code(dt), ac.BASIC)
+    assert (v, rows, cols) == (ac.BASIC, 256, 128), (rows, cols, splits)
+    A = rand((M, K), M, torch.float32).clamp_(-50, 50).to(dt)
+    B = rand((N, K), N, torch.float32).clamp_(-50, 50).to(dt)
+    scale = 2.0 ** -4
+    C = run_abi(abi, A, B, ac.BASIC, scale, ldc=N + 8)
+    check(C, A, B, scale)
+    S = torch.empty((M, N), dtype=out_dtype_of(dt), device="cuda")
+    assert ac.gemm_tn(abi, A.cuda(), B.cuda(), S, scale, ac.SIMPLE) == 0
+    torch.cuda.synchronize()
+    d = (C.float() - S.cpu().float()).abs()
+    bad = d > 2e-2 * S.cpu().float().abs() + 2e-2 * (K ** 0.5) * scale
+    assert int(bad.sum()) == 0, (int(bad.sum()), float(d.max()))
+    C2 = run_abi(abi, A, B, ac.AUTO, scale)
+    assert torch.equal(C.view(torch.int16), C2.view(torch.int16))
+
+
+def test_rectangular_tile_permutation_is_exact(abi):
+    """B = permutation matrix on a problem that runs on 256x128 tiles: pins the narrower B slot's
+    copy and fragment addressing bit for bit."""
+    M, N, K = 512, 14336, 1024
+    assert ac.plan(abi, M, N, K, ac.BF16, ac.BASIC)[1:3] == (256, 128)
+    A = rand((M, K), 1, torch.float32).clamp_(-200, 200).to(torch.bfloat16)
+    idx = torch.randint(0, K, (N,), generator=torch.Generator().manual_seed(2))
+    P = torch.zeros(N, K)
+    P[torch.arange(N), idx] = 1.0
+    got = run_abi(abi, A, P.to(torch.bfloat16), ac.BASIC)
+    want = (A.float()[:, idx] + 0.0).to(torch.bfloat16)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
 def test_k_zero_and_empty(abi):
     A, B = torch.zeros(8, 0, dtype=torch.bfloat16), torch.zeros(4, 0, dtype=torch.bfloat16)
     C = run_abi(abi, A, B)
