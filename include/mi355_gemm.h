@@ -35,7 +35,7 @@ enum mi355_dtype {
  * MI355_ERR_SHAPE when the shape does not meet that family's constraints). */
 enum mi355_variant {
   MI355_VARIANT_AUTO = 0,
-  MI355_VARIANT_BASIC = 1,    /* 256x256 or 128x128 tile, one wave group, 5-slot LDS ring     */
+  MI355_VARIANT_BASIC = 1,    /* 256x256, 256x128 or 128x128 tile, one wave group, LDS ring   */
   MI355_VARIANT_PINGPONG = 2, /* same tile, two wave groups alternating MFMA and load phases   */
   MI355_VARIANT_SKINNY = 3,   /* small-M weight-streaming kernel with split-K                  */
   MI355_VARIANT_SIMPLE = 4    /* one thread per output element; any shape; slow; self-check    */
