@@ -299,16 +299,18 @@ int mi355_gemm_tn_scaled(const void* A, const void* B, void* C, int64_t M, int64
   } else if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG) {
     const int tile = v == MI355_VARIANT_PINGPONG ? 256 : mi355::ring_tile_edge(M, N, K, elem_bytes(in_dtype));
     if (v == MI355_VARIANT_BASIC) {
+      // Both kinds of K split are optional for this kernel: without a (large enough, aligned)
+      // workspace the same tiles run unsplit, slower but with the same result contract.
+      const auto usable = [&](size_t need) {
+        return need && workspace && workspace_bytes >= need && (uintptr_t)workspace % 16 == 0;
+      };
       const int splits = mi355::ring_splits(M, N, K, elem_bytes(in_dtype));
-      const size_t need = splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0;
-      if (need && (!workspace || workspace_bytes < need || (uintptr_t)workspace % 16 != 0)) return MI355_ERR_WORKSPACE;
-      g.splits = splits;
       g.partial = (float*)workspace;
-      if (splits == 1) {
-        // Optional: without a workspace the tiles of the last round simply run unsplit.
+      if (splits > 1) {
+        if (usable((size_t)splits * (size_t)M * (size_t)N * sizeof(float))) g.splits = splits;
+      } else {
         int tail_tiles, tail_splits;
-        const size_t tail_bytes = mi355::ring_tail(M, N, K, elem_bytes(in_dtype), &tail_tiles, &tail_splits);
-        if (tail_bytes && workspace && workspace_bytes >= tail_bytes && (uintptr_t)workspace % 16 == 0) {
+        if (usable(mi355::ring_tail(M, N, K, elem_bytes(in_dtype), &tail_tiles, &tail_splits))) {
           g.tail_tiles = tail_tiles;
           g.tail_splits = tail_splits;
         }

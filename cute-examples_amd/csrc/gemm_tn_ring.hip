@@ -1,6 +1,6 @@
-// "basic" variant: 256x256 (or 128x128) output tile, ONE wave group of 4 waves (one per SIMD), each
-// wave owning a quarter of it (128x128 held in 256 fp32 accumulator registers per lane for the
-// 256 tile, which the description below uses).
+// "basic" variant: 256x256 (or 256x128, or 128x128) output tile, ONE wave group of 4 waves (one per
+// SIMD), each wave owning a quarter of it (128x128 held in 256 fp32 accumulator registers per lane
+// for the 256x256 tile, which the description below uses).  ring_plan.hip picks the tile.
 //
 // Data path per k-step (128 bytes of K per row: 64 bf16/fp16 or 128 fp8 elements):
 //

@@ -65,9 +65,9 @@ enum mi355_status {
  *             (1.0f for bf16/fp16; scale_a*scale_b for per-tensor-scaled fp8)
  *   variant   enum mi355_variant
  *   workspace device scratch of at least mi355_gemm_workspace_bytes(...) bytes, or NULL when
- *             that function returns 0; contents need not be initialised.  A K split needs it
- *             (MI355_ERR_WORKSPACE otherwise); the tail split of the tiled kernel (the tiles of
- *             a partly filled last round of workgroups cut along K) is skipped without it
+ *             that function returns 0; contents need not be initialised.  The skinny variant
+ *             needs it for its K split (MI355_ERR_WORKSPACE otherwise); the tiled variant runs
+ *             without its K split or tail split, i.e. slower, when it is NULL or too small
  *   stream    hipStream_t on which the kernels are enqueued (NULL = the null stream)
  *
  * Replaces test::gemm_tn_test (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92): same operand

@@ -295,6 +295,25 @@ def test_rectangular_tile_permutation_is_exact(abi):
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
+def test_tiled_kernel_runs_unsplit_without_a_workspace(abi):
+    """The K split of the tiled variant is optional: with no workspace (or one that is too small)
+    the call succeeds and gives the unsplit result."""
+    M, N, K = 512, 6144, 4096
+    v, rows, cols, splits, _, _ = ac.plan(abi, M, N, K, ac.BF16, ac.BASIC)
+    assert splits > 1
+    A, B = rand((M, K), 5, torch.bfloat16), rand((N, K), 6, torch.bfloat16)
+    Ad, Bd = A.cuda(), B.cuda()
+    s = torch.cuda.current_stream().cuda_stream
+    small = torch.empty(1024, dtype=torch.uint8, device="cuda")
+    for ws, nbytes in ((None, 0), (small.data_ptr(), 1024)):
+        C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        rc = abi.mi355_gemm_tn(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, K, N, ac.BF16, ac.BF16, 1.0,
+                               ac.BASIC, ws, nbytes, s)
+        assert rc == 0
+        torch.cuda.synchronize()
+        check(C.cpu(), A, B)
+
+
 def test_k_zero_and_empty(abi):
     A, B = torch.zeros(8, 0, dtype=torch.bfloat16), torch.zeros(4, 0, dtype=torch.bfloat16)
     C = run_abi(abi, A, B)
