@@ -180,6 +180,49 @@ def test_random_shape_sweep(abi, dt):
             assert err <= TOL[dt], (M, N, K, variant, err)
 
 
+def _random_mid_shapes(count, seed):
+    """Seeded shapes from a few hundred to a few thousand rows: between them they make the planner
+    use every tile shape, with and without a K split, and the tail split."""
+    import random
+    rng = random.Random(seed)
+    shapes = []
+    for _ in range(count):
+        M = rng.choice([rng.randint(200, 700), rng.randint(701, 2300), rng.randint(2301, 4700)])
+        N = 4 * rng.choice([rng.randint(100, 400), rng.randint(401, 1600), rng.randint(1601, 3700)])
+        K = 16 * rng.choice([rng.randint(64, 160), rng.randint(161, 400), rng.randint(401, 900)])
+        shapes.append((M, N, K))
+    return shapes
+
+
+@pytest.mark.parametrize("dt", list(DTYPES.values()))
+def test_random_mid_shape_sweep(abi, dt):
+    """16 seeded mid-sized shapes per input type through AUTO: every element against the
+    one-thread-per-output kernel, 64 sampled rows against the oracle, NaN guards around C."""
+    plans = set()
+    for (M, N, K) in _random_mid_shapes(16, 4):
+        plan = ac.plan(abi, M, N, K, ac.torch_code(dt))
+        plans.add((plan[1], plan[2], plan[3] > 1, plan[4] > 0))
+        if dt == torch.float8_e4m3fn:
+            g = torch.Generator().manual_seed(M + K)
+            A = torch.randint(0, 120, (M, K), dtype=torch.uint8, generator=g).view(dt)
+            B = torch.randint(0, 120, (N, K), dtype=torch.uint8, generator=g).view(dt)
+            scale = 2.0 ** -6
+        else:
+            A, B, scale = rand((M, K), M + K, dt), rand((N, K), N + K, dt), 1.0
+        C = run_abi(abi, A, B, ac.AUTO, scale=scale, ldc=N + 8 if (M + N) % 3 == 0 else None)
+        S = torch.empty((M, N), dtype=out_dtype_of(dt), device="cuda")
+        assert ac.gemm_tn(abi, A.cuda(), B.cuda(), S, scale, ac.SIMPLE) == 0
+        torch.cuda.synchronize()
+        Sf = S.cpu().float()
+        d = (C.float() - Sf).abs()
+        bad = d > 2e-2 * Sf.abs() + 2e-2 * (K ** 0.5) * scale * (40.0 if dt == torch.float8_e4m3fn else 1.0)
+        assert oracle.no_nan_left(C) and int(bad.sum()) == 0, (M, N, K, plan, int(bad.sum()), float(d.max()))
+        rows = torch.randperm(M, generator=torch.Generator().manual_seed(M))[:64]
+        assert oracle.rel_frobenius(C[rows], oracle.gemm_tn_fp32(A[rows], B, scale)) <= TOL[dt], (M, N, K, plan)
+    if dt != torch.float8_e4m3fn:
+        assert len(plans) >= 6, plans   # 256x256 / 256x128 / 128x128, split and unsplit, a tail split
+
+
 @pytest.mark.parametrize("M,N,K", [(5, 7, 3), (33, 17, 50), (100, 30, 77), (64, 64, 4)])
 @pytest.mark.parametrize("dt", list(DTYPES.values()))
 def test_shapes_only_the_simple_kernel_takes(abi, dt, M, N, K):
