@@ -16,7 +16,7 @@
 // load phase refills the registers the preceding MFMA phase has just finished with, and the other
 // group's MFMA phase (32 MFMAs, ~512 cycles) hides the LDS latency.  MFMA phases run at raised
 // wave priority.  LDS ring, swizzle, copy geometry and tile walk are those of the single-group
-// kernel (ring_common.h, gemm_tn_ring.hip): five 32 KiB slots, operand-steps queued as
+// kernel (ring_common.h, gemm_tn_ring.h): five 32 KiB slots, operand-steps queued as
 // A0 B0 A1 B1 A2 ..., the two slots of k-step t refilled with B(t+2), A(t+3) once both groups
 // have read them (end of phase 4t+2).
 //

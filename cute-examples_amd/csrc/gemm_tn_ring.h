@@ -42,6 +42,10 @@
 // Counterpart in the reference: the cooperative kernel, kernels/gemm_kernels/sm90a/gemm.cuh:246-418
 // (TMA producer warpgroup, mbarrier full/empty ring of 3 stages, two consumer warpgroups); here
 // every wave is loader and math at once because direct-to-LDS loads need no registers.
+//
+// This header holds the kernel and its launch templates; gemm_tn_ring_{bf16,f16,e4m3,mx}.hip
+// instantiate them per input type, one translation unit each so that they compile in parallel.
+#pragma once
 #include "gemm_launch.h"
 #include "ring_common.h"
 #include "tile_map.h"
@@ -537,21 +541,5 @@ int launch(const GemmArgs& g, int tile, hipStream_t stream) {
 }
 
 }  // namespace
-
-int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, hipStream_t stream) {
-  const bool out_bf16 = out_dtype == 0;
-  switch (in_dtype) {
-    case 0: return out_bf16 ? launch<BF16, BF16>(g, tile, stream) : launch<BF16, F16>(g, tile, stream);
-    case 1: return out_bf16 ? launch<F16, BF16>(g, tile, stream) : launch<F16, F16>(g, tile, stream);
-    case 2: return out_bf16 ? launch<E4M3, BF16>(g, tile, stream) : launch<E4M3, F16>(g, tile, stream);
-  }
-  return -1;
-}
-
-// e4m3 operands with block scales in the shuffled layout (g.mx_a, g.mx_b); 256x256 tiles, no K split.
-int launch_tile_ring_mx(const GemmArgs& g, int out_dtype, hipStream_t stream) {
-  if (g.splits != 1 || !g.mx_a || !g.mx_b) return -1;
-  return out_dtype == 0 ? launch_tile<MxE4M3, BF16, 256>(g, stream) : launch_tile<MxE4M3, F16, 256>(g, stream);
-}
 
 }  // namespace mi355

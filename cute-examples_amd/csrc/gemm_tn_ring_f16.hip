@@ -1,0 +1,10 @@
+// Single-group tile kernel (gemm_tn_ring.h), fp16 operands.
+#include "gemm_tn_ring.h"
+
+namespace mi355 {
+
+int launch_tile_ring_f16(const GemmArgs& g, int out_dtype, int tile, hipStream_t stream) {
+  return out_dtype == 0 ? launch<F16, BF16>(g, tile, stream) : launch<F16, F16>(g, tile, stream);
+}
+
+}  // namespace mi355

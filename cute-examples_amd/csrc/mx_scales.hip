@@ -11,7 +11,7 @@
 // The reference has no fp8 path; this is the block-scaled variant of the quantiser in
 // quantize_e4m3.hip, and the format the scaled MFMA of gfx950 consumes.
 //
-// The GEMM kernel reads scales in a "shuffled" layout (gemm_tn_ring.hip: kMxUnitBytes), produced
+// The GEMM kernel reads scales in a "shuffled" layout (gemm_tn_ring.h: kMxUnitBytes), produced
 // here from the natural row-major one: one 512-byte unit per (group of 128 rows, k-step of 128
 // elements), units ordered [row group][k-step], 8 bytes per lane: byte i of lane l is the scale of
 // row 16*i + l%16 of the group for block 4*kstep + l/16.  Rows are padded to whole 256-row tiles

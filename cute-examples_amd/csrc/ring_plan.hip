@@ -1,4 +1,4 @@
-// Host-side planning for the single-group tile kernel (gemm_tn_ring.hip): which tile, whether to
+// Host-side planning for the single-group tile kernel (gemm_tn_ring.h): which tile, whether to
 // split K uniformly, whether to cut the tiles of the last round.  Pure functions of the problem
 // size, so that the workspace query and the launch agree.  Counterpart in the reference: the
 // compile-time tile choice of DefaultConfig (kernels/gemm_kernels/sm90a/gemm.cuh:420-451) and the
@@ -121,6 +121,15 @@ size_t ring_tail(int64_t M, int64_t N, int64_t K, int elem_bytes, int* tail_tile
   if (M <= 0 || N <= 0 || K <= 0 || ring_tile_edge(M, N, K, elem_bytes) != 256) return 0;
   tail_plan(tiles_of(M, N, 256), k_steps_of(K, elem_bytes), tail_tiles, tail_splits);
   return (size_t)*tail_tiles * (size_t)*tail_splits * 256 * 256 * sizeof(float);
+}
+
+int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, hipStream_t stream) {
+  switch (in_dtype) {
+    case 0: return launch_tile_ring_bf16(g, out_dtype, tile, stream);
+    case 1: return launch_tile_ring_f16(g, out_dtype, tile, stream);
+    case 2: return launch_tile_ring_e4m3(g, out_dtype, tile, stream);
+  }
+  return -1;
 }
 
 }  // namespace mi355
