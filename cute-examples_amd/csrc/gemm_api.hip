@@ -238,8 +238,7 @@ int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, in
     if (!workspace || workspace_bytes < bytes_a + bytes_b || (uintptr_t)workspace % 16 != 0) return MI355_ERR_WORKSPACE;
     uint8_t* wa = (uint8_t*)workspace;
     uint8_t* wb = wa + bytes_a;  // bytes_a is a multiple of 1024
-    if (mi355::launch_mx_shuffle(scale_a, M, K, ld_scale_a, wa, s) != 0) return MI355_ERR_LAUNCH;
-    if (mi355::launch_mx_shuffle(scale_b, N, K, ld_scale_b, wb, s) != 0) return MI355_ERR_LAUNCH;
+    if (mi355::launch_mx_shuffle2(scale_a, M, ld_scale_a, wa, scale_b, N, ld_scale_b, wb, K, s) != 0) return MI355_ERR_LAUNCH;
     g.mx_a = wa;
     g.mx_b = wb;
   }

@@ -69,6 +69,8 @@ int launch_tile_ring_e4m3(const GemmArgs& g, int out_dtype, int tile, hipStream_
 // (x (rows, K) -> e4m3 elements + natural-layout E8M0 scales).
 size_t mx_shuffled_bytes(int64_t rows, int64_t K);
 int launch_mx_shuffle(const uint8_t* scales, int64_t rows, int64_t K, int64_t ld, uint8_t* out, hipStream_t stream);
+int launch_mx_shuffle2(const uint8_t* scales_a, int64_t rows_a, int64_t ld_a, uint8_t* out_a, const uint8_t* scales_b,
+                       int64_t rows_b, int64_t ld_b, uint8_t* out_b, int64_t K, hipStream_t stream);
 int launch_quantize_mxfp8(const void* x, int in_dtype, int64_t rows, int64_t K, int64_t ldx, void* q,
                           uint8_t* scales, hipStream_t stream);
 // Skinny (small-M) weight-streaming kernel.  stream_splits is a pure host function.

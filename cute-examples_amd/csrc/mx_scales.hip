@@ -25,11 +25,25 @@ namespace {
 
 constexpr int kMxBlock = 32;
 
-__global__ __launch_bounds__(256) void mx_shuffle_kernel(const uint8_t* __restrict__ scales, int64_t rows,
-                                                         int64_t ld, uint32_t k_steps, uint64_t slots,
-                                                         uint8_t* __restrict__ out) {
-  const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;  // one lane slot of 8 bytes
-  if (id >= slots) return;
+// One operand's scale bytes and where its shuffled copy goes.
+struct MxOperand {
+  const uint8_t* scales;
+  int64_t rows, ld;
+  uint64_t slots;  // 8-byte lane slots of the shuffled layout
+  uint8_t* out;
+};
+
+// Shuffles one operand, or two in one launch (second.slots == 0 if there is only one): thread ids
+// below first.slots work on the first operand, the rest on the second.
+__global__ __launch_bounds__(256) void mx_shuffle_kernel(MxOperand first, MxOperand second, uint32_t k_steps) {
+  uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;  // one lane slot of 8 bytes
+  const bool is_second = id >= first.slots;
+  if (is_second) id -= first.slots;
+  const MxOperand& op = is_second ? second : first;
+  if (id >= op.slots) return;
+  const uint8_t* __restrict__ scales = op.scales;
+  uint8_t* __restrict__ out = op.out;
+  const int64_t rows = op.rows, ld = op.ld;
   const uint32_t lane = (uint32_t)(id & 63u);
   const uint64_t unit = id >> 6;
   const uint64_t group = unit / k_steps;
@@ -97,12 +111,19 @@ size_t mx_shuffled_bytes(int64_t rows, int64_t K) {
 }
 
 int launch_mx_shuffle(const uint8_t* scales, int64_t rows, int64_t K, int64_t ld, uint8_t* out, hipStream_t stream) {
-  const uint64_t slots = mx_shuffled_bytes(rows, K) / 8;
-  if (slots == 0) return 0;
-  const uint64_t blocks = (slots + 255) / 256;
+  return launch_mx_shuffle2(scales, rows, ld, out, nullptr, 0, 0, nullptr, K, stream);
+}
+
+// Both operands of a GEMM in one launch (rows_b == 0: only the first).
+int launch_mx_shuffle2(const uint8_t* scales_a, int64_t rows_a, int64_t ld_a, uint8_t* out_a,
+                       const uint8_t* scales_b, int64_t rows_b, int64_t ld_b, uint8_t* out_b, int64_t K,
+                       hipStream_t stream) {
+  const MxOperand a = {scales_a, rows_a, ld_a, mx_shuffled_bytes(rows_a, K) / 8, out_a};
+  const MxOperand b = {scales_b, rows_b, ld_b, mx_shuffled_bytes(rows_b, K) / 8, out_b};
+  if (a.slots + b.slots == 0) return 0;
+  const uint64_t blocks = (a.slots + b.slots + 255) / 256;
   if (blocks >= ((uint64_t)1 << 31)) return -1;
-  hipLaunchKernelGGL(mx_shuffle_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, scales, rows, ld,
-                     (uint32_t)(K / 128), slots, out);
+  hipLaunchKernelGGL(mx_shuffle_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, a, b, (uint32_t)(K / 128));
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
