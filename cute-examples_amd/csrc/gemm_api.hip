@@ -198,8 +198,10 @@ int mi355_gemm_mx_check(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ld
 }
 
 size_t mi355_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int scales_shuffled) {
-  if (scales_shuffled || M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
-  return mi355::mx_shuffled_bytes(M, K) + mi355::mx_shuffled_bytes(N, K);
+  if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
+  int splits, tail_tiles, tail_splits;
+  const size_t partial = mi355::ring_plan_256(M, N, K, 1, &splits, &tail_tiles, &tail_splits);
+  return partial + (scales_shuffled ? 0 : mi355::mx_shuffled_bytes(M, K) + mi355::mx_shuffled_bytes(N, K));
 }
 
 int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
@@ -228,6 +230,7 @@ int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, in
   }
   if (!A_q || !B_q || !scale_a || !scale_b) return MI355_ERR_NULL;
   if ((uintptr_t)A_q % 16 != 0 || (uintptr_t)B_q % 16 != 0 || (uintptr_t)C % 8 != 0) return MI355_ERR_ALIGN;
+  size_t used = 0;  // bytes of the workspace taken by the shuffled scales
   if (scales_shuffled) {
     if ((uintptr_t)scale_a % 8 != 0 || (uintptr_t)scale_b % 8 != 0) return MI355_ERR_ALIGN;
     g.mx_a = scale_a;
@@ -241,6 +244,17 @@ int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, in
     if (mi355::launch_mx_shuffle2(scale_a, M, ld_scale_a, wa, scale_b, N, ld_scale_b, wb, K, s) != 0) return MI355_ERR_LAUNCH;
     g.mx_a = wa;
     g.mx_b = wb;
+    used = bytes_a + bytes_b;
+  }
+  // K split or tail split when the rest of the workspace holds the partial results (optional, as
+  // for the other tiled kernels: without it the tiles run unsplit).
+  int splits, tail_tiles, tail_splits;
+  const size_t partial = mi355::ring_plan_256(M, N, K, 1, &splits, &tail_tiles, &tail_splits);
+  if (partial && workspace && (uintptr_t)workspace % 16 == 0 && workspace_bytes >= used + partial) {
+    g.partial = (float*)((uint8_t*)workspace + used);  // used is a multiple of 1024
+    g.splits = splits;
+    g.tail_tiles = tail_tiles;
+    g.tail_splits = tail_splits;
   }
   g.tiles_m = (M + 255) / 256;
   g.tiles_n = (N + 255) / 256;

@@ -125,11 +125,13 @@ int mi355_quantize_e4m3(const void *x, int x_dtype, int64_t n, void *x_q,
  *                      workspace first (one small kernel per operand).  With scales_shuffled == 1
  *                      they are the output of mi355_mx_shuffle_scales (ld_scale_* ignored) and no
  *                      workspace is needed: do this once for weights.
- *   workspace          at least mi355_gemm_mx_workspace_bytes(M, N, K, scales_shuffled) bytes,
- *                      16-byte aligned.
+ *   workspace          mi355_gemm_mx_workspace_bytes(M, N, K, scales_shuffled) bytes, 16-byte
+ *                      aligned: the shuffled scales (required when scales_shuffled == 0) followed
+ *                      by the partial results of a K split or tail split (optional: with less
+ *                      room the tiles run unsplit).
  * Constraints: K % 128 == 0; A, B 16-byte aligned with row strides that are multiples of 16;
  * N % 4 == 0, ldc % 4 == 0, C 8-byte aligned; the size limits of the tiled variants.  Always runs
- * the 256x256-tile kernel (MI355_VARIANT_BASIC) without a K split.
+ * the 256x256-tile kernel (MI355_VARIANT_BASIC).
  * Counterpart in the reference: none (it has no fp8 path); same launcher contract as
  * mi355_gemm_tn (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92), block format per the OCP
  * Microscaling Formats (MX) specification v1.0.
@@ -142,7 +144,7 @@ int mi355_gemm_tn_mxfp8(const void *A_q, const void *B_q, void *C,
                         int scales_shuffled, int out_dtype,
                         void *workspace, size_t workspace_bytes, void *stream);
 
-/* Workspace mi355_gemm_tn_mxfp8 needs (0 when the scales are already shuffled). */
+/* Workspace mi355_gemm_tn_mxfp8 wants: shuffled scales (unless already shuffled) + split partials. */
 size_t mi355_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int scales_shuffled);
 
 /* Argument check of mi355_gemm_tn_mxfp8 without pointers; runs without a GPU. */

@@ -97,9 +97,11 @@ def gemm_tn_mxfp8(L, A_q, B_q, sa, sb, C, shuffled=False, stream=None):
         rc = rc or L.mi355_mx_shuffle_scales(sb.data_ptr(), N, K, sb.stride(0), pb.data_ptr(), s)
         if rc:
             return rc
+        ws_bytes = L.mi355_gemm_mx_workspace_bytes(M, N, K, 1)     # partial results of a K split, if any
+        ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=A_q.device)
         return L.mi355_gemm_tn_mxfp8(A_q.data_ptr(), B_q.data_ptr(), C.data_ptr(), M, N, K, A_q.stride(0),
                                      B_q.stride(0), C.stride(0), pa.data_ptr(), 0, pb.data_ptr(), 0, 1, out_dt,
-                                     None, 0, s)
+                                     ws.data_ptr(), ws_bytes, s)
     ws_bytes = L.mi355_gemm_mx_workspace_bytes(M, N, K, 0)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=A_q.device)
     return L.mi355_gemm_tn_mxfp8(A_q.data_ptr(), B_q.data_ptr(), C.data_ptr(), M, N, K, A_q.stride(0),

@@ -70,6 +70,35 @@ def test_ragged_tiles(abi, shape):
     check(C, A, sa, B, sb)
 
 
+@pytest.mark.parametrize("shuffled", [False, True])
+@pytest.mark.parametrize("shape", [(512, 6144, 4096), (256, 4096, 14336), (4096, 6144, 4096), (300, 1000, 8192)])
+def test_k_split_and_tail_split(abi, shape, shuffled):
+    """Few tiles: K split 2, 7 and 4 ways; 384 tiles: the last round cut in two.  Same result as
+    without the workspace for the partial results (unsplit), up to the summation order."""
+    M, N, K = shape
+    assert abi.mi355_gemm_mx_workspace_bytes(M, N, K, 1) > 0
+    A, sa = random_mx(M, K, 11, 120, 132)
+    B, sb = random_mx(N, K, 12, 120, 132)
+    C = run_mx(abi, A, sa, B, sb, shuffled=shuffled)
+    err, ref = check(C, A, sa, B, sb)
+    assert err < 5e-3
+    C2 = run_mx(abi, A, sa, B, sb, shuffled=shuffled)
+    assert torch.equal(C.view(torch.int16), C2.view(torch.int16))       # deterministic
+    if shuffled:
+        return
+    # natural-layout scales with a workspace that only holds the shuffled scales: runs unsplit
+    Ad, Bd, sad, sbd = A.cuda(), B.cuda(), sa.cuda(), sb.cuda()
+    only_scales = abi.mi355_mx_shuffled_bytes(M, K) + abi.mi355_mx_shuffled_bytes(N, K)
+    ws = torch.empty(only_scales, dtype=torch.uint8, device="cuda")
+    C3 = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rc = abi.mi355_gemm_tn_mxfp8(Ad.data_ptr(), Bd.data_ptr(), C3.data_ptr(), M, N, K, K, K, N, sad.data_ptr(), K // 32,
+                                 sbd.data_ptr(), K // 32, 0, ac.BF16, ws.data_ptr(), only_scales,
+                                 torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert oracle.rel_frobenius(C3.cpu(), ref) < 5e-3
+
+
 def test_each_scale_byte_reaches_its_block_only(abi):
     """All elements 1, all scales 1 except ONE (row, block) of A doubled: exactly row m changes, by
     exactly +32 per column, for every position of the block in the k-step, the scale group and the
