@@ -499,6 +499,60 @@ def test_skinny_split_k_is_deterministic_and_needs_its_workspace(abi):
                       torch.empty(300, 64, dtype=torch.bfloat16, device="cuda"), 1.0, ac.SKINNY) == ac.ERR_SHAPE
 
 
+@pytest.mark.parametrize("variant", [ac.AUTO, ac.PINGPONG, ac.SIMPLE])
+def test_c_larger_than_4_gib(abi, variant):
+    """65836 x 32772 bf16 outputs (4.3 GB): row offsets into C pass 2^31 elements and 2^32 bytes.
+    Sampled rows against the oracle; the reference narrows sizes and strides to int
+    (gemm_test.cu:29-31, :44-46) and could not run this."""
+    M, N, K = 65536 + 300, 32768 + 4, 64
+    g = torch.Generator(device="cuda").manual_seed(3)
+    A = torch.randn(M, K, generator=g, device="cuda").bfloat16()
+    B = torch.randn(N, K, generator=g, device="cuda").bfloat16()
+    C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert C.numel() * 2 > 2 ** 32
+    assert ac.gemm_tn(abi, A, B, C, 1.0, variant) == 0
+    torch.cuda.synchronize()
+    rows = torch.tensor([0, 1, 255, 256, 32767, 32768, 65535, 65536, 65537, 65791, 65792, M - 2, M - 1])
+    got = C[rows.cuda()].cpu()
+    assert oracle.no_nan_left(got)
+    assert oracle.rel_frobenius(got, oracle.gemm_tn_fp32(A[rows.cuda()].cpu(), B.cpu())) <= 1e-2
+    # every element was written: no NaN left anywhere (checked on the device, in slabs)
+    for r0 in range(0, M, 8192):
+        assert not torch.isnan(C[r0:r0 + 8192]).any(), r0
+
+
+@pytest.mark.parametrize("variant", [ac.AUTO, ac.PINGPONG])
+def test_a_larger_than_4_gib(abi, variant):
+    """A is 70000 x 32768 bf16 (4.6 GB): the byte offset of the last row panels passes 2^32."""
+    M, N, K = 70000, 256, 32768
+    g = torch.Generator(device="cuda").manual_seed(4)
+    A = torch.empty(M, K, dtype=torch.bfloat16, device="cuda")
+    for r0 in range(0, M, 10000):
+        A[r0:r0 + 10000] = torch.randn(min(10000, M - r0), K, generator=g, device="cuda").bfloat16()
+    B = torch.randn(N, K, generator=g, device="cuda").bfloat16()
+    assert A.numel() * 2 > 2 ** 32
+    C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert ac.gemm_tn(abi, A, B, C, 1.0, variant) == 0
+    torch.cuda.synchronize()
+    assert not torch.isnan(C).any()
+    rows = torch.tensor([0, 255, 256, 65535, 65536, 65537, 69887, 69888, M - 1])
+    ref = oracle.gemm_tn_fp32(A[rows.cuda()].cpu(), B.cpu())
+    assert oracle.rel_frobenius(C[rows.cuda()].cpu(), ref) <= 1e-2
+    # and with the big matrix on the B side (columns of C)
+    Ct = torch.full((N, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+    assert ac.gemm_tn(abi, B, A, Ct, 1.0, variant) == 0
+    torch.cuda.synchronize()
+    assert not torch.isnan(Ct).any()
+    assert oracle.rel_frobenius(Ct[:, rows.cuda()].cpu(), ref.t()) <= 1e-2
+    if variant == ac.AUTO:   # 16 rows against the 4.6 GB of weights: the streaming kernel
+        assert abi.mi355_gemm_select_variant(16, M, K, ac.BF16) == ac.SKINNY
+        Cs = torch.full((16, M), float("nan"), dtype=torch.bfloat16, device="cuda")
+        assert ac.gemm_tn(abi, B[:16].contiguous(), A, Cs, 1.0, ac.AUTO) == 0
+        torch.cuda.synchronize()
+        assert not torch.isnan(Cs).any()
+        assert oracle.rel_frobenius(Cs[:, rows.cuda()].cpu(), ref[:, :16].t()) <= 1e-2
+
+
 # ---------------------------------------------------------------- Python module
 
 def test_python_module_is_the_reference_call(abi):
