@@ -197,3 +197,31 @@ def test_tile_map_keeps_an_xcd_compact(abi):
             rows.add(a.value)
             cols.add(b.value)
         assert len(rows) + len(cols) <= 12, (xcd, rows, cols)
+
+
+def test_header_is_plain_c_and_links_from_c(tmp_path):
+    """The public header compiles as C99 and as C++, and a C program linked against the library
+    can call the entry points that need no GPU."""
+    import os
+    src = tmp_path / "use_abi.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include "mi355_gemm.h"
+int main(void) {
+  int rows, cols, splits, tail_tiles, tail_splits;
+  int v = mi355_gemm_plan(4096, 6144, 4096, MI355_BF16, MI355_VARIANT_AUTO, &rows, &cols, &splits, &tail_tiles, &tail_splits);
+  if (mi355_gemm_version() < 1) return 1;
+  if (mi355_gemm_check(256, 256, 64, 64, 64, 256, MI355_BF16, MI355_BF16, MI355_VARIANT_AUTO) != MI355_OK) return 2;
+  if (mi355_gemm_tn(NULL, NULL, NULL, 256, 256, 64, 64, 64, 256, MI355_BF16, MI355_BF16, 1.0f, MI355_VARIANT_AUTO, NULL, 0, NULL) != MI355_ERR_NULL) return 3;
+  printf("%d %d %d %d %d %d %s\n", v, rows, cols, splits, tail_tiles, tail_splits, mi355_gemm_strerror(MI355_ERR_SHAPE));
+  return 0;
+}
+''')
+    inc = os.path.dirname(ac.HEADER)
+    libdir = os.path.dirname(ac.LIB)
+    exe = tmp_path / "use_abi"
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", inc, str(src), "-o", str(exe),
+                    "-L", libdir, "-l:libmi355gemm.so", "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    out = subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split(None, 6)
+    assert [int(x) for x in out[:6]] == [ac.BASIC, 256, 256, 1, 128, 2] and "constraint" in out[6]
+    subprocess.run(["g++", "-std=c++11", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", "-I", inc, ac.HEADER], check=True)
