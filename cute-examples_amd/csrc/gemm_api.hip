@@ -197,11 +197,22 @@ int mi355_gemm_mx_check(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ld
   return MI355_OK;
 }
 
+namespace {
+// Partial results of the block-scaled GEMM's K split or tail split (the planner's, as for plain fp8).
+size_t mx_partial_bytes(int64_t M, int64_t N, int64_t K, int* splits, int* tail_tiles, int* tail_splits) {
+  int s = mi355::ring_splits(M, N, K, 1), tt = 0, ts = 1;
+  size_t bytes = s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : mi355::ring_tail(M, N, K, 1, &tt, &ts);
+  if (splits) *splits = s;
+  if (tail_tiles) *tail_tiles = tt;
+  if (tail_splits) *tail_splits = ts;
+  return bytes;
+}
+}  // namespace
+
 size_t mi355_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int scales_shuffled) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
-  int splits, tail_tiles, tail_splits;
-  const size_t partial = mi355::ring_plan_256(M, N, K, 1, &splits, &tail_tiles, &tail_splits);
-  return partial + (scales_shuffled ? 0 : mi355::mx_shuffled_bytes(M, K) + mi355::mx_shuffled_bytes(N, K));
+  return mx_partial_bytes(M, N, K, nullptr, nullptr, nullptr) +
+         (scales_shuffled ? 0 : mi355::mx_shuffled_bytes(M, K) + mi355::mx_shuffled_bytes(N, K));
 }
 
 int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
@@ -249,16 +260,17 @@ int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, in
   // K split or tail split when the rest of the workspace holds the partial results (optional, as
   // for the other tiled kernels: without it the tiles run unsplit).
   int splits, tail_tiles, tail_splits;
-  const size_t partial = mi355::ring_plan_256(M, N, K, 1, &splits, &tail_tiles, &tail_splits);
+  const size_t partial = mx_partial_bytes(M, N, K, &splits, &tail_tiles, &tail_splits);
   if (partial && workspace && (uintptr_t)workspace % 16 == 0 && workspace_bytes >= used + partial) {
     g.partial = (float*)((uint8_t*)workspace + used);  // used is a multiple of 1024
     g.splits = splits;
     g.tail_tiles = tail_tiles;
     g.tail_splits = tail_splits;
   }
-  g.tiles_m = (M + 255) / 256;
-  g.tiles_n = (N + 255) / 256;
-  return mi355::launch_tile_ring_mx(g, out_dtype, s) == 0 ? MI355_OK : MI355_ERR_LAUNCH;
+  const int tile = mi355::ring_tile_edge(M, N, K, 1);
+  g.tiles_m = (M + mi355::ring_tile_rows(tile) - 1) / mi355::ring_tile_rows(tile);
+  g.tiles_n = (N + mi355::ring_tile_cols(tile) - 1) / mi355::ring_tile_cols(tile);
+  return mi355::launch_tile_ring_mx(g, out_dtype, tile, s) == 0 ? MI355_OK : MI355_ERR_LAUNCH;
 }
 
 int mi355_gemm_tn(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,

@@ -59,8 +59,7 @@ int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, h
 // Tail split the single-group kernel would use for this problem (pure host heuristic): returns the
 // workspace bytes it needs (0 = no tail split) and sets *tail_tiles, *tail_splits.
 size_t ring_tail(int64_t M, int64_t N, int64_t K, int elem_bytes, int* tail_tiles, int* tail_splits);
-size_t ring_plan_256(int64_t M, int64_t N, int64_t K, int elem_bytes, int* splits, int* tail_tiles, int* tail_splits);
-int launch_tile_ring_mx(const GemmArgs& g, int out_dtype, hipStream_t stream);
+int launch_tile_ring_mx(const GemmArgs& g, int out_dtype, int tile, hipStream_t stream);
 // Per-input-type halves of launch_tile_ring (one translation unit each).
 int launch_tile_ring_bf16(const GemmArgs& g, int out_dtype, int tile, hipStream_t stream);
 int launch_tile_ring_f16(const GemmArgs& g, int out_dtype, int tile, hipStream_t stream);

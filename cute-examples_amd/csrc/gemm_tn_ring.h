@@ -118,8 +118,9 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   // spans all of them, the two halves of the wave's rows of A.
   constexpr bool kRowSliced = G::kRowSliced;
   constexpr bool kMx = G::kMx;
-  static_assert(!kMx || (kRowSliced && !kRaggedK && kWaveTileM == 128 && kWaveTileN == 128),
-                "block scales: whole k-steps, one 128-row scale group per wave and operand");
+  static_assert(!kMx || (kRowSliced && !kRaggedK && (kWaveTileM == 128 || kWaveTileM == 64) &&
+                         (kWaveTileN == 128 || kWaveTileN == 64)),
+                "block scales: whole k-steps, a whole or half 128-row scale group per wave and operand");
   constexpr int kHalfM = kNbM / 2;                       // row blocks of A per slice when kRowSliced
   constexpr int kMfmaPerSlice = kRowSliced ? kHalfM * kNbN : kNbM * kNbN;
   constexpr int kReadsPerSlice = kNbM + kNbN;            // fragment loads per slice (K-sliced case)
@@ -231,17 +232,22 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   // Block scales (kMx only).  Set ph holds the scales of the k-step worked off in ring phase ph:
   // [0] rows 0..63 and [1] rows 64..127 of the wave's rows of A (sca) and of B (scb), one byte per
   // 16-row block.  A set is loaded two k-steps ahead by load_8B_async; see the waits at its users.
+  // A wave with only 64 rows of an operand starts its 8 bytes at the half of the 128-row unit that
+  // holds them and uses [0] only ([1] then holds bytes of the next lane, or zeros past the end).
   u32x2 sca[kSlots], scb[kSlots];
-  const __amdgpu_buffer_rsrc_t rsrc_sa = make_raw_buffer(g.mx_a, kMx ? tiles_m * 2u * k_steps * kMxUnitBytes : 0u);
-  const __amdgpu_buffer_rsrc_t rsrc_sb = make_raw_buffer(g.mx_b, kMx ? tiles_n * 2u * k_steps * kMxUnitBytes : 0u);
+  const uint32_t mx_bytes_a = kMx ? (uint32_t)((g.M + 255) / 256) * 2u * k_steps * kMxUnitBytes : 0u;
+  const uint32_t mx_bytes_b = kMx ? (uint32_t)((g.N + 255) / 256) * 2u * k_steps * kMxUnitBytes : 0u;
+  const __amdgpu_buffer_rsrc_t rsrc_sa = make_raw_buffer(g.mx_a, mx_bytes_a);
+  const __amdgpu_buffer_rsrc_t rsrc_sb = make_raw_buffer(g.mx_b, mx_bytes_b);
   uint32_t voff_sa = 0, voff_sb = 0;  // lane's bytes of the current item's first unit
   // Scale offset of k-step kt of the current item, clamped to its last like soff_of.
   auto mx_soff_of = [&](uint32_t kt) __attribute__((always_inline)) -> uint32_t {
     return __builtin_amdgcn_readfirstlane((kt < steps ? kt : steps - 1) * kMxUnitBytes);
   };
   auto mx_open_tile = [&](uint32_t tm, uint32_t tn, uint32_t step0) __attribute__((always_inline)) {
-    voff_sa = ((tm * 2 + wm) * k_steps + step0) * kMxUnitBytes + lane * 8;
-    voff_sb = ((tn * 2 + wn) * k_steps + step0) * kMxUnitBytes + lane * 8;
+    const uint32_t row_a = tm * kTile + wm * kWaveTileM, row_b = tn * kTileN + wn * kWaveTileN;  // the wave's first rows
+    voff_sa = ((row_a / 128) * k_steps + step0) * kMxUnitBytes + lane * 8 + (row_a % 128) / 64 * 4;
+    voff_sb = ((row_b / 128) * k_steps + step0) * kMxUnitBytes + lane * 8 + (row_b % 128) / 64 * 4;
     load_8B_async(sca[0], rsrc_sa, voff_sa, mx_soff_of(0));
     load_8B_async(scb[0], rsrc_sb, voff_sb, mx_soff_of(0));
     load_8B_async(sca[1], rsrc_sa, voff_sa, mx_soff_of(1));
@@ -304,7 +310,6 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     constexpr int ph = decltype(phc)::value, s = decltype(sc)::value, u = decltype(uc)::value;
     constexpr int j = u / kHalfM, r = u % kHalfM, i = s * kHalfM + r;
     if constexpr (kMx) {
-      static_assert(kTile == 256, "block scales run on the 256-wide tile only");
       G::template mfma_scaled_inplace<j % 4, i % 4>(fb[0][j], fa[s][r], acc[i][j], scb[ph][j / 4], sca[ph][i / 4]);
     } else {
       (void)ph;
@@ -315,7 +320,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
 
   // Stores of the tile at (m0, n0): converted output, or fp32 partials for a split-K item.
   const float scale = output_scale(g);
-  constexpr bool kAsmMfma = kTile == 256;  // see mfma_u
+  constexpr bool kAsmMfma = kTile == 256 || kMx;  // see mfma_u; the scaled MFMA is always inline assembly
   auto epilogue = [&](int64_t m0, int64_t n0) __attribute__((always_inline)) {
     store_output_tile<G, OutT, kNbM, kNbN, kAsmMfma>(acc, g, m0, n0, kTile, kTileN, wm * kWaveTileM, wn * kWaveTileN, lane, scale);
   };

@@ -123,20 +123,6 @@ size_t ring_tail(int64_t M, int64_t N, int64_t K, int elem_bytes, int* tail_tile
   return (size_t)*tail_tiles * (size_t)*tail_splits * 256 * 256 * sizeof(float);
 }
 
-// K split and tail split of a problem that runs on 256x256 tiles whatever its size (the
-// block-scaled kernel): returns the workspace bytes of the partial results.
-size_t ring_plan_256(int64_t M, int64_t N, int64_t K, int elem_bytes, int* splits, int* tail_tiles, int* tail_splits) {
-  *splits = 1;
-  *tail_tiles = 0;
-  *tail_splits = 1;
-  if (M <= 0 || N <= 0 || K <= 0) return 0;
-  const int64_t tiles = tiles_of(M, N, 256), steps = k_steps_of(K, elem_bytes);
-  *splits = uniform_splits(tiles, steps);
-  if (*splits > 1) return (size_t)*splits * (size_t)M * (size_t)N * sizeof(float);
-  tail_plan(tiles, steps, tail_tiles, tail_splits);
-  return (size_t)*tail_tiles * (size_t)*tail_splits * 256 * 256 * sizeof(float);
-}
-
 int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, hipStream_t stream) {
   switch (in_dtype) {
     case 0: return launch_tile_ring_bf16(g, out_dtype, tile, stream);

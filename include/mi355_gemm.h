@@ -131,7 +131,8 @@ int mi355_quantize_e4m3(const void *x, int x_dtype, int64_t n, void *x_q,
  *                      room the tiles run unsplit).
  * Constraints: K % 128 == 0; A, B 16-byte aligned with row strides that are multiples of 16;
  * N % 4 == 0, ldc % 4 == 0, C 8-byte aligned; the size limits of the tiled variants.  Always runs
- * the 256x256-tile kernel (MI355_VARIANT_BASIC).
+ * the tiled kernel (MI355_VARIANT_BASIC) with the tile and splits mi355_gemm_plan reports for
+ * MI355_E4M3 operands of this shape.
  * Counterpart in the reference: none (it has no fp8 path); same launcher contract as
  * mi355_gemm_tn (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92), block format per the OCP
  * Microscaling Formats (MX) specification v1.0.

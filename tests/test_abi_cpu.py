@@ -95,10 +95,13 @@ def test_mx_sizes_and_rejections_before_any_device_access(abi):
     assert abi.mi355_mx_shuffled_bytes(256, 96) == 0                 # K % 128
     assert abi.mi355_gemm_mx_workspace_bytes(300, 100, 256, 0) == (512 + 256) * 8
     assert abi.mi355_gemm_mx_workspace_bytes(300, 100, 256, 1) == 0
-    # K split of 48 tiles in two (32 k-steps), and the tail split of 384 tiles: partial results behind the scales
-    assert abi.mi355_gemm_mx_workspace_bytes(512, 6144, 4096, 1) == 2 * 512 * 6144 * 4
-    assert abi.mi355_gemm_mx_workspace_bytes(512, 6144, 4096, 0) == 2 * 512 * 6144 * 4 + (512 + 6144) * 128
+    # partial results of the planner's K split (32 tiles of 256x128 cut in seven) or tail split
+    # (384 tiles of 256x256) behind the shuffled scales; the plan is the one for plain e4m3
+    assert ac.plan(abi, 256, 4096, 14336, ac.E4M3)[1:4] == (256, 128, 7)
+    assert abi.mi355_gemm_mx_workspace_bytes(256, 4096, 14336, 1) == 7 * 256 * 4096 * 4
+    assert abi.mi355_gemm_mx_workspace_bytes(256, 4096, 14336, 0) == 7 * 256 * 4096 * 4 + (256 + 4096) * 448
     assert abi.mi355_gemm_mx_workspace_bytes(4096, 6144, 4096, 1) == 2 * 128 * 256 * 256 * 4
+    assert abi.mi355_gemm_mx_workspace_bytes(512, 6144, 4096, 1) == 0      # 192 tiles of 128x128, unsplit
     f = abi.mi355_gemm_tn_mxfp8
     assert f(None, None, None, 256, 256, 128, 128, 128, 256, None, 4, None, 4, 0, ac.BF16, None, 0, None) == ac.ERR_NULL
     assert f(None, None, None, 256, 256, 100, 128, 128, 256, None, 4, None, 4, 0, ac.BF16, None, 0, None) == ac.ERR_SHAPE

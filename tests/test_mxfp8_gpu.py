@@ -71,10 +71,11 @@ def test_ragged_tiles(abi, shape):
 
 
 @pytest.mark.parametrize("shuffled", [False, True])
-@pytest.mark.parametrize("shape", [(512, 6144, 4096), (256, 4096, 14336), (4096, 6144, 4096), (300, 1000, 8192)])
+@pytest.mark.parametrize("shape", [(768, 768, 8192), (256, 4096, 14336), (4096, 6144, 4096), (300, 1000, 8192)])
 def test_k_split_and_tail_split(abi, shape, shuffled):
-    """Few tiles: K split 2, 7 and 4 ways; 384 tiles: the last round cut in two.  Same result as
-    without the workspace for the partial results (unsplit), up to the summation order."""
+    """Few tiles: K split 4 ways on 128x128 tiles, 7 ways on 256x128 tiles; 384 tiles of 256x256: the
+    last round cut in two.  Same result as without the workspace for the partial results (unsplit),
+    up to the summation order."""
     M, N, K = shape
     assert abi.mi355_gemm_mx_workspace_bytes(M, N, K, 1) > 0
     A, sa = random_mx(M, K, 11, 120, 132)
@@ -97,6 +98,51 @@ def test_k_split_and_tail_split(abi, shape, shuffled):
     assert rc == 0
     torch.cuda.synchronize()
     assert oracle.rel_frobenius(C3.cpu(), ref) < 5e-3
+
+
+@pytest.mark.parametrize("shape,tile", [((2048, 2048, 2048), (128, 128)), ((512, 6144, 4096), (128, 128)),
+                                        ((1024, 6144, 4096), (256, 128)), ((1000, 6100, 4224), (256, 128)),
+                                        ((2048, 6144, 4096), (256, 256)), ((100, 260, 256), (128, 128))])
+def test_every_tile_shape(abi, shape, tile):
+    """The block-scaled kernel runs on the tile the planner picks for plain e4m3; a wave with 64 rows
+    of an operand reads half a 128-row scale unit."""
+    M, N, K = shape
+    assert ac.plan(abi, M, N, K, ac.E4M3)[1:3] == tile
+    A, sa = random_mx(M, K, 21)
+    B, sb = random_mx(N, K, 22)
+    C = run_mx(abi, A, sa, B, sb, ldc=N + 4)
+    err, _ = check(C, A, sa, B, sb)
+    assert err < 5e-3
+
+
+@pytest.mark.parametrize("M,N", [(128, 128), (256, 128), (256, 256)])
+def test_each_scale_byte_reaches_its_block_only_on_every_tile(abi, M, N):
+    """One doubled scale byte changes exactly its row (or column) by exactly +32, for rows in every
+    16-row block of every wave, whichever tile shape the planner gives the problem."""
+    K = 256
+    big_m, big_n = {(128, 128): (2048, 2048), (256, 128): (1024, 6144), (256, 256): (2048, 6144)}[(M, N)]
+    K = {(128, 128): 2048, (256, 128): 4096, (256, 256): 4096}[(M, N)]
+    assert ac.plan(abi, big_m, big_n, K, ac.E4M3)[1:3] == (M, N)
+    ones_a = torch.ones(big_m, K).to(torch.float8_e4m3fn)
+    ones_b = torch.ones(big_n, K).to(torch.float8_e4m3fn)
+    base_a = torch.full((big_m, K // 32), 127, dtype=torch.uint8)
+    base_b = torch.full((big_n, K // 32), 127, dtype=torch.uint8)
+    rows = [0, 17, 63, 64, 127, 128, 191, 255, 256 + 70, big_m - 1]
+    sa = base_a.clone()
+    for i, r in enumerate(rows):
+        sa[r, (5 * i + 3) % (K // 32)] = 128
+    C = run_mx(abi, ones_a, sa, ones_b, base_b).float()
+    want = torch.full((big_m, big_n), float(K))
+    want[rows, :] += 32.0
+    assert torch.equal(C, want)
+    cols = [0, 15, 16, 63, 64, 100, 127, 128, 255, 300, big_n - 1]
+    sb = base_b.clone()
+    for i, c in enumerate(cols):
+        sb[c, (7 * i + 1) % (K // 32)] = 128
+    C = run_mx(abi, ones_a, base_a, ones_b, sb).float()
+    want = torch.full((big_m, big_n), float(K))
+    want[:, cols] += 32.0
+    assert torch.equal(C, want)
 
 
 def test_each_scale_byte_reaches_its_block_only(abi):
