@@ -173,14 +173,15 @@ int mi355_mx_shuffle_scales(const uint8_t* scales, int64_t rows, int64_t K, int6
 }
 
 int mi355_quantize_mxfp8(const void* x, int x_dtype, int64_t rows, int64_t K, int64_t ldx, void* x_q,
-                         uint8_t* scales, void* stream) {
+                         uint8_t* scales, int scales_shuffled, void* stream) {
   if (x_dtype != MI355_BF16 && x_dtype != MI355_F16 && x_dtype != MI355_F32) return MI355_ERR_DTYPE;
   if (rows < 0 || K < 0 || K % 32 != 0 || ldx < K) return MI355_ERR_SHAPE;
+  if (scales_shuffled && K % 128 != 0) return MI355_ERR_SHAPE;
   if (rows == 0 || K == 0) return MI355_OK;
   if (!x || !x_q || !scales) return MI355_ERR_NULL;
   const int64_t es = x_dtype == MI355_F32 ? 4 : 2;
   if ((uintptr_t)x % 16 != 0 || (ldx * es) % 16 != 0 || (uintptr_t)x_q % 16 != 0) return MI355_ERR_ALIGN;
-  return mi355::launch_quantize_mxfp8(x, x_dtype, rows, K, ldx, x_q, scales, (hipStream_t)stream) == 0
+  return mi355::launch_quantize_mxfp8(x, x_dtype, rows, K, ldx, x_q, scales, scales_shuffled != 0, (hipStream_t)stream) == 0
              ? MI355_OK : MI355_ERR_LAUNCH;
 }
 

@@ -72,7 +72,7 @@ int launch_mx_shuffle(const uint8_t* scales, int64_t rows, int64_t K, int64_t ld
 int launch_mx_shuffle2(const uint8_t* scales_a, int64_t rows_a, int64_t ld_a, uint8_t* out_a, const uint8_t* scales_b,
                        int64_t rows_b, int64_t ld_b, uint8_t* out_b, int64_t K, hipStream_t stream);
 int launch_quantize_mxfp8(const void* x, int in_dtype, int64_t rows, int64_t K, int64_t ldx, void* q,
-                          uint8_t* scales, hipStream_t stream);
+                          uint8_t* scales, bool shuffled, hipStream_t stream);
 // Skinny (small-M) weight-streaming kernel.  stream_splits is a pure host function.
 int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes);
 int launch_stream(const GemmArgs& g, int in_dtype, int out_dtype, int splits, void* workspace, hipStream_t stream);

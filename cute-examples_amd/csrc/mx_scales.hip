@@ -59,14 +59,27 @@ __global__ __launch_bounds__(256) void mx_shuffle_kernel(MxOperand first, MxOper
   *(u32x2*)(out + id * 8) = (u32x2){w[0], w[1]};
 }
 
-// One thread per block of 32 elements.
-template <class In>
+// Where the scale of (row, block) lives in the shuffled layout.
+__device__ __forceinline__ int64_t shuffled_index(int64_t row, int64_t blk, int64_t blocks_per_row) {
+  const int64_t unit = (row / 128) * (blocks_per_row / 4) + blk / 4;
+  const int64_t lane = row % 16 + 16 * (blk % 4);
+  return unit * 512 + lane * 8 + (row % 128) / 16;
+}
+
+// One thread per block of 32 elements.  kShuffled: the scales are written straight into the layout
+// the GEMM reads (rows padded to a multiple of 256 with the scale 1), which saves the shuffle launch.
+template <class In, bool kShuffled>
 __global__ __launch_bounds__(256) void mx_quantize_kernel(const void* __restrict__ x, int64_t rows, int64_t blocks_per_row,
                                                           int64_t ldx, uint8_t* __restrict__ q,
                                                           uint8_t* __restrict__ scales) {
   const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (id >= rows * blocks_per_row) return;
+  const int64_t padded_rows = kShuffled ? (rows + 255) / 256 * 256 : rows;
+  if (id >= padded_rows * blocks_per_row) return;
   const int64_t row = id / blocks_per_row, blk = id % blocks_per_row;
+  if (kShuffled && row >= rows) {
+    scales[shuffled_index(row, blk, blocks_per_row)] = 127;
+    return;
+  }
   const int64_t at = row * ldx + blk * kMxBlock;
   float v[kMxBlock];
 #pragma unroll
@@ -89,17 +102,22 @@ __global__ __launch_bounds__(256) void mx_quantize_kernel(const void* __restrict
   u32x4* dst = (u32x4*)(q + row * blocks_per_row * kMxBlock + blk * kMxBlock);
   dst[0] = (u32x4){w[0], w[1], w[2], w[3]};
   dst[1] = (u32x4){w[4], w[5], w[6], w[7]};
-  scales[id] = (uint8_t)byte;
+  scales[kShuffled ? shuffled_index(row, blk, blocks_per_row) : id] = (uint8_t)byte;
 }
 
 template <class In>
-int run_quantize(const void* x, int64_t rows, int64_t K, int64_t ldx, void* q, uint8_t* scales, hipStream_t stream) {
-  const int64_t n = rows * (K / kMxBlock);
+int run_quantize(const void* x, int64_t rows, int64_t K, int64_t ldx, void* q, uint8_t* scales, bool shuffled,
+                 hipStream_t stream) {
+  const int64_t n = (shuffled ? (rows + 255) / 256 * 256 : rows) * (K / kMxBlock);
   if (n == 0) return 0;
   const int64_t blocks = (n + 255) / 256;
   if (blocks >= ((int64_t)1 << 31)) return -1;
-  hipLaunchKernelGGL((mx_quantize_kernel<In>), dim3((unsigned)blocks), dim3(256), 0, stream, x, rows, K / kMxBlock, ldx,
-                     (uint8_t*)q, scales);
+  if (shuffled)
+    hipLaunchKernelGGL((mx_quantize_kernel<In, true>), dim3((unsigned)blocks), dim3(256), 0, stream, x, rows,
+                       K / kMxBlock, ldx, (uint8_t*)q, scales);
+  else
+    hipLaunchKernelGGL((mx_quantize_kernel<In, false>), dim3((unsigned)blocks), dim3(256), 0, stream, x, rows,
+                       K / kMxBlock, ldx, (uint8_t*)q, scales);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 
@@ -129,11 +147,11 @@ int launch_mx_shuffle2(const uint8_t* scales_a, int64_t rows_a, int64_t ld_a, ui
 
 // in_dtype: 0 bf16, 1 fp16, 3 fp32.
 int launch_quantize_mxfp8(const void* x, int in_dtype, int64_t rows, int64_t K, int64_t ldx, void* q,
-                          uint8_t* scales, hipStream_t stream) {
+                          uint8_t* scales, bool shuffled, hipStream_t stream) {
   switch (in_dtype) {
-    case 0: return run_quantize<BF16>(x, rows, K, ldx, q, scales, stream);
-    case 1: return run_quantize<F16>(x, rows, K, ldx, q, scales, stream);
-    case 3: return run_quantize<float>(x, rows, K, ldx, q, scales, stream);
+    case 0: return run_quantize<BF16>(x, rows, K, ldx, q, scales, shuffled, stream);
+    case 1: return run_quantize<F16>(x, rows, K, ldx, q, scales, shuffled, stream);
+    case 3: return run_quantize<float>(x, rows, K, ldx, q, scales, shuffled, stream);
   }
   return -1;
 }

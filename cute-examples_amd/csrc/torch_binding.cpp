@@ -250,7 +250,8 @@ torch::Tensor shuffle_mx_scales(const torch::Tensor scales) {
 
 // (x_q, scales): x (rows, K) -> float8_e4m3fn (rows, K) and uint8 E8M0 scale bytes (rows, K/32),
 // one per 32 consecutive elements of a row, x ~= x_q * 2^(scales - 127).
-std::pair<torch::Tensor, torch::Tensor> quantize_mxfp8(const torch::Tensor x) {
+// With shuffled the scales come back flat, in the layout gemm_tn_mxfp8(..., scales_shuffled=True) takes.
+std::pair<torch::Tensor, torch::Tensor> quantize_mxfp8(const torch::Tensor x, bool shuffled) {
   TORCH_CHECK(x.dim() == 2 && x.is_contiguous(), "x must be a contiguous 2D tensor");
   int dt;
   switch (x.scalar_type()) {
@@ -265,9 +266,11 @@ std::pair<torch::Tensor, torch::Tensor> quantize_mxfp8(const torch::Tensor x) {
   c10::DeviceGuard guard(x.device());
   hipStream_t stream = c10::hip::getCurrentHIPStream(x.device().index()).stream();
   torch::Tensor q = torch::empty({rows, K}, x.options().dtype(at::kFloat8_e4m3fn));
-  torch::Tensor sc = torch::empty({rows, K / 32}, x.options().dtype(at::kByte));
+  TORCH_CHECK(!shuffled || K % 128 == 0, "shuffled scales need the last dimension to be a multiple of 128");
+  torch::Tensor sc = shuffled ? torch::empty({(int64_t)mi355_mx_shuffled_bytes(rows, K)}, x.options().dtype(at::kByte))
+                              : torch::empty({rows, K / 32}, x.options().dtype(at::kByte));
   int st = mi355_quantize_mxfp8(x.const_data_ptr(), dt, rows, K, K, q.mutable_data_ptr(), sc.data_ptr<uint8_t>(),
-                                (void*)stream);
+                                shuffled ? 1 : 0, (void*)stream);
   TORCH_CHECK(st == MI355_OK, "gemm_kernels: ", mi355_gemm_strerror(st));
   return {q, sc};
 }
@@ -302,7 +305,9 @@ PYBIND11_MODULE(_C, m) {
   m.def("shuffle_mx_scales", &test::shuffle_mx_scales,
         "re-lay MX scale bytes (rows, K/32) into the layout the kernel reads", py::arg("scales"));
   m.def("quantize_mxfp8", &test::quantize_mxfp8,
-        "MX quantisation on the device: returns (x_q float8_e4m3fn, scales uint8 (rows, K/32))", py::arg("x"));
+        "MX quantisation on the device: returns (x_q float8_e4m3fn, scales uint8 (rows, K/32), or flat in the "
+        "GEMM's layout with shuffled=True)",
+        py::arg("x"), py::arg("shuffled") = false);
   m.def("select_variant", &test::select_variant, py::arg("M"), py::arg("N"), py::arg("K"),
         py::arg("dtype"));
   m.def("version", []() { return mi355_gemm_version(); });

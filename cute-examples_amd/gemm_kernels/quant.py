@@ -37,11 +37,14 @@ def quantize_e4m3_torch(x):
     return x_q, scale
 
 
-def quantize_mxfp8(x):
-    """Returns (x_q, scales): x (rows, K) -> float8_e4m3fn (rows, K), uint8 scale bytes (rows, K/32)."""
+def quantize_mxfp8(x, shuffled=False):
+    """Returns (x_q, scales): x (rows, K) -> float8_e4m3fn (rows, K), uint8 scale bytes (rows, K/32);
+    with shuffled=True (HIP tensors only) the scales come back in the layout the GEMM reads."""
     if x.is_cuda and x.dtype in (torch.float32, torch.bfloat16, torch.float16):
         from ._C import quantize_mxfp8 as _native
-        return _native(x.detach().contiguous())
+        return _native(x.detach().contiguous(), shuffled)
+    if shuffled:
+        raise ValueError("shuffled scales are produced on a HIP device only")
     return quantize_mxfp8_torch(x)
 
 

@@ -164,14 +164,15 @@ size_t mi355_mx_shuffled_bytes(int64_t rows, int64_t K);
 
 /*
  * MX quantiser: x (rows, K) of x_dtype (BF16, F16 or F32), row stride ldx elements, K % 32 == 0
- * -> x_q (rows, K) contiguous e4m3 and scales (rows, K/32) contiguous E8M0 bytes in the natural
- * layout.  Per block: scale = 2^(floor(log2(amax)) - 8) (1 for a block of zeros), elements
+ * -> x_q (rows, K) contiguous e4m3 and the E8M0 scale bytes: (rows, K/32) contiguous in the natural
+ * layout, or, with scales_shuffled != 0 (K % 128 == 0), mi355_mx_shuffled_bytes(rows, K) bytes in the
+ * layout mi355_gemm_tn_mxfp8 takes with scales_shuffled == 1 (no shuffle launch then).  Per block: scale = 2^(floor(log2(amax)) - 8) (1 for a block of zeros), elements
  * x/scale rounded to nearest even, saturated at +-448.  x 16-byte aligned with ldx*elem_bytes
  * % 16 == 0, x_q 16-byte aligned.  NaN and infinity are not supported.
  * Counterpart in the reference: none; OCP MX specification v1.0, section 6.3.
  */
 int mi355_quantize_mxfp8(const void *x, int x_dtype, int64_t rows, int64_t K, int64_t ldx,
-                         void *x_q, uint8_t *scales, void *stream);
+                         void *x_q, uint8_t *scales, int scales_shuffled, void *stream);
 
 /* Scratch bytes mi355_gemm_tn wants for this problem and variant (0 for most shapes).
  * Counterpart: none in the reference (it has no split-K); sizes the split-K partials that

@@ -42,7 +42,7 @@ def load():
     L.mi355_mx_shuffle_scales.restype = ci
     L.mi355_mx_shuffled_bytes.argtypes = [i64, i64]
     L.mi355_mx_shuffled_bytes.restype = sz
-    L.mi355_quantize_mxfp8.argtypes = [vp, ci, i64, i64, i64, vp, u8p, vp]
+    L.mi355_quantize_mxfp8.argtypes = [vp, ci, i64, i64, i64, vp, u8p, ci, vp]
     L.mi355_quantize_mxfp8.restype = ci
     L.mi355_gemm_workspace_bytes.argtypes = [i64, i64, i64, ci, ci]
     L.mi355_gemm_workspace_bytes.restype = sz

@@ -111,10 +111,11 @@ def test_mx_sizes_and_rejections_before_any_device_access(abi):
     assert f(24, 16, 16, 256, 256, 128, 128, 128, 256, 16, 4, 16, 4, 1, ac.BF16, None, 0, None) == ac.ERR_ALIGN
     assert abi.mi355_mx_shuffle_scales(None, 256, 128, 4, None, None) == ac.ERR_NULL
     assert abi.mi355_mx_shuffle_scales(None, 256, 96, 4, None, None) == ac.ERR_SHAPE
-    assert abi.mi355_quantize_mxfp8(None, ac.BF16, 4, 64, 64, None, None, None) == ac.ERR_NULL
-    assert abi.mi355_quantize_mxfp8(None, ac.E4M3, 4, 64, 64, None, None, None) == ac.ERR_DTYPE
-    assert abi.mi355_quantize_mxfp8(None, ac.BF16, 4, 48, 48, None, None, None) == ac.ERR_SHAPE
-    assert abi.mi355_quantize_mxfp8(16, ac.BF16, 4, 64, 68, 16, 16, None) == ac.ERR_ALIGN
+    assert abi.mi355_quantize_mxfp8(None, ac.BF16, 4, 64, 64, None, None, 0, None) == ac.ERR_NULL
+    assert abi.mi355_quantize_mxfp8(None, ac.E4M3, 4, 64, 64, None, None, 0, None) == ac.ERR_DTYPE
+    assert abi.mi355_quantize_mxfp8(None, ac.BF16, 4, 48, 48, None, None, 0, None) == ac.ERR_SHAPE
+    assert abi.mi355_quantize_mxfp8(None, ac.BF16, 4, 64, 64, None, None, 1, None) == ac.ERR_SHAPE   # shuffled: K % 128
+    assert abi.mi355_quantize_mxfp8(16, ac.BF16, 4, 64, 68, 16, 16, 0, None) == ac.ERR_ALIGN
 
 
 def test_workspace_bytes(abi):

@@ -216,12 +216,35 @@ def test_quantizer_is_bit_exact(abi, dtype):
     xd = x.cuda()
     code = {torch.bfloat16: ac.BF16, torch.float16: ac.F16, torch.float32: ac.F32}[dtype]
     rc = abi.mi355_quantize_mxfp8(xd.data_ptr(), code, x.shape[0], x.shape[1], xd.stride(0), q.data_ptr(), sc.data_ptr(),
-                                  torch.cuda.current_stream().cuda_stream)
+                                  0, torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     torch.cuda.synchronize()
     want_q, want_s = oracle.quantize_mxfp8(x)
     assert torch.equal(sc.cpu(), want_s)
     assert torch.equal(q.cpu(), want_q.view(torch.uint8))
+
+
+@pytest.mark.parametrize("rows", [300, 256, 1])
+def test_quantizer_writes_shuffled_scales_directly(abi, rows):
+    """The quantiser's shuffled output is byte for byte what mi355_mx_shuffle_scales makes of its
+    natural output (padding rows included), and feeds the GEMM without a shuffle launch."""
+    import gemm_kernels
+    g = torch.Generator().manual_seed(rows)
+    x = (torch.randn(rows, 1024, generator=g) * torch.exp2(torch.randint(-8, 8, (rows, 1), generator=g).float())).bfloat16().cuda()
+    q1, s_nat = gemm_kernels.quantize_mxfp8(x)
+    q2, s_shuf = gemm_kernels.quantize_mxfp8(x, shuffled=True)
+    torch.cuda.synchronize()
+    assert torch.equal(q1.view(torch.uint8), q2.view(torch.uint8))
+    assert torch.equal(s_shuf, gemm_kernels.shuffle_mx_scales(s_nat))
+    w = torch.randn(512, 1024, generator=g).bfloat16().cuda()
+    wq, sw = gemm_kernels.quantize_mxfp8(w, shuffled=True)
+    C1 = torch.empty(rows, 512, dtype=torch.bfloat16, device="cuda")
+    C2 = torch.empty_like(C1)
+    gemm_kernels.gemm_tn_mxfp8(q2, wq, s_shuf, sw, C1, scales_shuffled=True)
+    wq_n, sw_n = gemm_kernels.quantize_mxfp8(w)
+    gemm_kernels.gemm_tn_mxfp8(q1, wq_n, s_nat, sw_n, C2)
+    torch.cuda.synchronize()
+    assert torch.equal(C1.view(torch.int16), C2.view(torch.int16))
 
 
 def test_end_to_end_from_bf16(abi):
