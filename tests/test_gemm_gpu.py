@@ -357,6 +357,33 @@ def test_tiled_kernel_runs_unsplit_without_a_workspace(abi):
         check(C.cpu(), A, B)
 
 
+@pytest.mark.parametrize("variant", [ac.AUTO, ac.BASIC, ac.PINGPONG, ac.SKINNY, ac.SIMPLE])
+@pytest.mark.parametrize("dt", list(DTYPES.values()))
+def test_operands_with_padded_rows(abi, dt, variant):
+    """lda > K and ldb > K (rows of a wider matrix), which the reference's contiguity check
+    (gemm_test.cu:18) excludes: the padding holds NaN and must never be read into a result."""
+    M, N, K = (48, 520, 1024) if variant == ac.SKINNY else (300, 520, 1024)
+    pad_a, pad_b = 64, 160
+    es = 1 if dt == torch.float8_e4m3fn else 2
+    g = torch.Generator().manual_seed(9)
+    def padded(rows, pad):
+        if dt == torch.float8_e4m3fn:
+            full = torch.full((rows, K + pad), 0x7f, dtype=torch.uint8)          # e4m3 NaN
+            full[:, :K] = torch.randint(0, 120, (rows, K), dtype=torch.uint8, generator=g)
+            return full.view(dt).cuda()
+        full = torch.full((rows, K + pad), float("nan"), dtype=dt)
+        full[:, :K] = torch.randn(rows, K, generator=g).to(dt)
+        return full.cuda()
+    Af, Bf = padded(M, pad_a), padded(N, pad_b)
+    A, B = Af[:, :K], Bf[:, :K]                       # views with row strides K + pad
+    assert A.stride(0) == K + pad_a and (A.stride(0) * es) % 16 == 0
+    scale = 2.0 ** -6 if dt == torch.float8_e4m3fn else 1.0
+    C = torch.full((M, N), float("nan"), dtype=out_dtype_of(dt), device="cuda")
+    assert ac.gemm_tn(abi, A, B, C, scale, variant) == 0
+    torch.cuda.synchronize()
+    check(C.cpu(), A.cpu().contiguous(), B.cpu().contiguous(), scale)
+
+
 def test_k_zero_and_empty(abi):
     A, B = torch.zeros(8, 0, dtype=torch.bfloat16), torch.zeros(4, 0, dtype=torch.bfloat16)
     C = run_abi(abi, A, B)
