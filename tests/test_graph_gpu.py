@@ -76,3 +76,63 @@ def test_quantise_and_fp8_gemms_replay():
         ref = X.float() @ W.float().t()
         assert float((got1.float() - ref).norm() / ref.norm()) < 6e-2
         assert float((got2.float() - ref).norm() / ref.norm()) < 6e-2
+
+
+def test_host_threads_on_their_own_streams():
+    """Four host threads, each on its own stream, issue different problems at the same time (tile
+    kernel with a tail split, streaming kernel with a K split, fp8, block-scaled fp8): the library
+    keeps no state between calls, so every result equals the one computed alone."""
+    import threading
+    torch.manual_seed(0)
+    jobs = []
+    for kind, (M, N, K) in (("bf16", (4096, 6144, 1024)), ("bf16", (16, 4096, 4096)), ("fp8", (512, 1024, 2048)),
+                            ("mx", (768, 768, 2048))):
+        X = torch.randn(M, K, device="cuda").bfloat16()
+        W = torch.randn(N, K, device="cuda").bfloat16()
+        jobs.append((kind, X, W))
+
+    def run(kind, X, W, C):
+        if kind == "bf16":
+            gemm_kernels.gemm_tn_test(X, W, C)
+        elif kind == "fp8":
+            (xq, sx), (wq, sw) = gemm_kernels.quantize_e4m3(X), gemm_kernels.quantize_e4m3(W)
+            gemm_kernels.gemm_tn_fp8(xq, wq, sx, sw, C)
+        else:
+            (xq, sx), (wq, sw) = gemm_kernels.quantize_mxfp8(X, True), gemm_kernels.quantize_mxfp8(W, True)
+            gemm_kernels.gemm_tn_mxfp8(xq, wq, sx, sw, C, True)
+
+    alone = []
+    for kind, X, W in jobs:
+        C = torch.empty(X.shape[0], W.shape[0], dtype=torch.bfloat16, device="cuda")
+        run(kind, X, W, C)
+        alone.append(C)
+    torch.cuda.synchronize()
+
+    results = [None] * len(jobs)
+    errors = []
+
+    def worker(i):
+        try:
+            kind, X, W = jobs[i]
+            stream = torch.cuda.Stream()
+            stream.wait_stream(torch.cuda.default_stream())
+            outs = []
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    C = torch.full((X.shape[0], W.shape[0]), float("nan"), dtype=torch.bfloat16, device="cuda")
+                    run(kind, X, W, C)
+                    outs.append(C)
+            stream.synchronize()
+            results[i] = outs
+        except Exception as e:  # surfaced below: an exception in a thread would otherwise be lost
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(jobs))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i, outs in enumerate(results):
+        for C in outs:
+            assert torch.equal(C.view(torch.int16), alone[i].view(torch.int16)), i
