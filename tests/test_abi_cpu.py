@@ -229,3 +229,40 @@ int main(void) {
     out = subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split(None, 6)
     assert [int(x) for x in out[:6]] == [ac.BASIC, 256, 256, 1, 128, 2] and "constraint" in out[6]
     subprocess.run(["g++", "-std=c++11", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", "-I", inc, ac.HEADER], check=True)
+
+
+def test_plan_invariants_over_random_shapes(abi):
+    """3000 seeded random problems per input type: whatever the planner picks must be launchable as
+    the kernels assume (splits divide the k-steps and leave at least 16, split items fit the CUs,
+    a tail split only on 256x256 tiles and only for the tiles of the last round) and the workspace
+    query must match it."""
+    import random
+    rng = random.Random(7)
+    seen = set()
+    for dt, es in ((ac.BF16, 2), (ac.F16, 2), (ac.E4M3, 1)):
+        for _ in range(3000):
+            M = rng.choice([rng.randint(1, 300), rng.randint(1, 5000), rng.randint(1, 20000)])
+            N = 4 * rng.choice([rng.randint(1, 100), rng.randint(1, 2000), rng.randint(1, 8000)])
+            K = (16 // es) * rng.choice([rng.randint(1, 64), rng.randint(1, 1024), rng.randint(1, 4096)])
+            v, rows, cols, splits, tail_tiles, tail_splits = ac.plan(abi, M, N, K, dt)
+            steps = -(-K * es // 128)
+            assert v in (ac.BASIC, ac.SKINNY), (M, N, K, v)
+            assert (v == ac.SKINNY) == (M <= 64)
+            tiles = -(-M // rows) * -(-N // cols)
+            assert splits >= 1 and tail_splits >= 1 and tail_tiles >= 0
+            if splits > 1:
+                assert steps % splits == 0 and tail_tiles == 0, (M, N, K, splits)
+                assert steps // splits >= (16 if v == ac.BASIC else 8), (M, N, K, splits)
+            want = splits * M * N * 4 if splits > 1 else 0
+            if v == ac.BASIC:
+                assert (rows, cols) in ((256, 256), (256, 128), (128, 128))
+                if splits > 1:
+                    assert tiles * splits <= 256
+                if tail_tiles:
+                    assert (rows, cols) == (256, 256) and splits == 1 and tail_splits > 1
+                    assert 256 <= tiles <= 3 * 256 and tail_tiles == tiles % 256
+                    assert tail_tiles * tail_splits <= 256 and steps % tail_splits == 0 and steps // tail_splits >= 16
+                    want = tail_tiles * tail_splits * 256 * 256 * 4
+                seen.add((rows, cols, splits > 1, tail_tiles > 0))
+            assert abi.mi355_gemm_workspace_bytes(M, N, K, dt, ac.AUTO) == want, (M, N, K)
+    assert len(seen) >= 7, seen
