@@ -52,3 +52,61 @@ def test_rejects_a_file_without_the_kernel(tmp_path):
     f.write_text("\ts_endpgm\n")
     with pytest.raises(RuntimeError, match="no block-scaled kernel"):
         check_async_loads.check(str(f))
+
+
+def test_lds_swizzle_is_a_bijection_and_conflict_free():
+    """CPU model of the LDS layout of the tile kernels (the counterpart of the reference's swizzled
+    shared-memory layouts, kernels/gemm_kernels/sm90a/gemm.cuh:420-451).  A row is 128 bytes = 8
+    chunks of 16; chunk c of row r is stored at chunk c ^ swizzle(r).  Checked: the map is a
+    bijection on a 256-row slot; what the direct-to-LDS copies write (lane l of a copy lands at
+    16*l and fetches global chunk (l%8) ^ swizzle(row)) is exactly that layout; and every
+    ds_read_b128 the kernels issue is conflict-free under the model that such a read is served 16
+    lanes at a time from 64 four-byte banks (the hardware counter SQ_LDS_BANK_CONFLICT reads 0 on
+    the real kernels)."""
+    import re
+    src = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "cute-examples_amd", "csrc",
+                            "ring_common.h")).read()
+    m = re.search(r"uint32_t swizzle\(uint32_t row\) \{ return \(row >> (\d+)\) & (\d+)u; \}", src)
+    assert m, "the swizzle in ring_common.h changed: update this model"
+    shift, mask = int(m.group(1)), int(m.group(2))
+    swz = lambda r: (r >> shift) & mask
+
+    def address(row, chunk):              # byte address of logical chunk `chunk` of row `row` inside a slot
+        return row * 128 + ((chunk ^ swz(row)) * 16)
+
+    rows = 256
+    assert len({address(r, c) for r in range(rows) for c in range(8)}) == rows * 8
+    assert all(0 <= address(r, c) < rows * 128 for r in range(rows) for c in range(8))
+
+    # copies: one instruction covers 8 rows; lane l -> row l/8, LDS bytes [16 l, 16 l + 16) of those rows
+    for first_row in range(0, rows, 8):
+        for lane in range(64):
+            row = first_row + lane // 8
+            fetched_chunk = (lane % 8) ^ swz(row)
+            assert address(row, fetched_chunk) == first_row * 128 + 16 * lane
+
+    def conflict_free(lane_addresses):
+        for q in range(0, 64, 16):        # 16 lanes x 16 bytes = all 64 banks once
+            banks = set()
+            for a in lane_addresses[q:q + 16]:
+                for b in range(4):
+                    banks.add((a // 4 + b) % 64)
+            if len(banks) != 64:
+                return False
+        return True
+
+    # fragment reads: lane l reads row (block base + l%16); group l/16 picks the logical chunk
+    patterns = {
+        "16-bit, slice s": lambda s, g, e: s * 4 + g,
+        "fp8, two chunks per lane": lambda s, g, e: 2 * g + e,
+        "block-scaled fp8": lambda s, g, e: g + 4 * e,
+    }
+    for name, chunk_of in patterns.items():
+        for base in range(0, rows, 16):
+            for s in range(2):
+                for e in range(2):
+                    addrs = [address(base + l % 16, chunk_of(s, l // 16, e)) for l in range(64)]
+                    assert conflict_free(addrs), (name, base, s, e)
+    # and the layout without the swizzle would conflict, so the check has teeth
+    plain = [(l % 16) * 128 + (l // 16) * 16 for l in range(64)]
+    assert not conflict_free(plain)
