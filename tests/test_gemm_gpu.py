@@ -83,6 +83,43 @@ def test_permutation_matrix_moves_columns_exactly(abi, dt, variant):
     assert torch.equal(got_t.view(torch.int16), want.t().contiguous().view(torch.int16))
 
 
+@pytest.mark.parametrize("variant", [ac.BASIC, ac.PINGPONG, ac.SKINNY, ac.SIMPLE])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_epilogue_rounds_ties_to_even(abi, dt, variant):
+    """Every output is x + h or x + h + tiny with h exactly half an ulp of x in the output type: the
+    fp32 accumulator holds the sum exactly, so the result pins the down-conversion (the
+    reference's NumericArrayConverter, gemm.cuh:375-377) to round-to-nearest-even, ties included,
+    for both signs, odd and even last bits and across exponent boundaries."""
+    mant = 7 if dt == torch.bfloat16 else 10
+    M = 256
+    g = torch.Generator().manual_seed(31)
+    # x: random values of the type with exponents -4..8; h = half an ulp of x (a power of two)
+    x = (torch.rand(M, generator=g) + 1.0) * torch.exp2(torch.randint(-4, 9, (M,), generator=g).float())
+    x = (x * torch.where(torch.rand(M, generator=g) < 0.5, -1.0, 1.0)).to(dt)
+    x[0], x[1], x[2], x[3] = 1.0, -1.0, 2.0 - 2.0 ** -mant, -(4.0 - 2.0 ** (1 - mant))     # even, even, all-ones mantissas
+    exp = torch.floor(torch.log2(x.float().abs()))
+    h = torch.exp2(exp - mant - 1) * torch.sign(x.float())
+    K = 16
+    A = torch.zeros(M, K)
+    A[:, 0], A[:, 1], A[:, 2] = x.float(), h, h * 2.0 ** -8            # the third term breaks the tie upwards
+    B = torch.zeros(8, K)
+    B[0:4, 0] = 1.0
+    B[0:4, 1] = 1.0                                                    # columns 0-3: exact ties
+    B[4:8, 0] = 1.0
+    B[4:8, 1] = 1.0
+    B[4:8, 2] = 1.0                                                    # columns 4-7: just above the tie
+    A, B = A.to(dt), B.to(dt)
+    assert torch.equal(A.float()[:, 1], h) and torch.equal(A.float()[:, 2], h * 2.0 ** -8)
+    exact = A.double() @ B.double().t()                                # three-term sums, exact in fp32 too
+    assert torch.equal(exact.float().double(), exact)
+    want = exact.float().to(dt)                                        # torch rounds to nearest even
+    got = run_abi(abi, A, B, variant)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    # the ties went to the even neighbour, the others up (away from x)
+    assert torch.equal(want[:, 0].float() == x.float(), (x.view(torch.int16) & 1) == 0)
+    assert torch.all(want[:, 4].float().abs() > x.float().abs())
+
+
 # ---------------------------------------------------------------- oracle parity, seeded random
 
 @pytest.mark.parametrize("variant", [ac.AUTO] + TILED)
