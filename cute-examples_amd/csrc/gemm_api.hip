@@ -60,6 +60,39 @@ int resolve(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t l
   return variant;
 }
 
+// Repacking: MI355_VARIANT_AUTO turns a problem the tiled kernels cannot address (K*elem_bytes or
+// a row stride not a multiple of 16, N or ldc not a multiple of 4, misaligned pointers) into an
+// aligned one in the caller's workspace -- A and B copied to zero-padded 16-byte-aligned rows, C
+// computed into a padded buffer and copied out -- when the workspace is large enough and the
+// problem is big enough to pay for three more passes over the operands.  The generic kernel takes
+// about a millisecond per GFLOP; the repacked problem runs at the tiled kernels' rate.
+struct Repack {
+  bool a, b, c;
+  int64_t Kp, Np;                 // padded K (elements) and N
+  size_t bytes_a, bytes_b, bytes_c;
+};
+
+size_t round_up(size_t x, size_t to) { return (x + to - 1) / to * to; }
+
+bool repack_plan(const void* A, const void* B, const void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
+                 int64_t ldb, int64_t ldc, int in_dtype, Repack* r) {
+  const int64_t es = elem_bytes(in_dtype);
+  if (M <= 0 || N <= 0 || K <= 0) return false;
+  if (2.0 * (double)M * (double)N * (double)K < 134217728.0) return false;   // under ~0.1 ms on the generic kernel
+  const int64_t per16 = 16 / es;
+  r->Kp = (K + per16 - 1) / per16 * per16;
+  r->Np = (N + 3) / 4 * 4;
+  r->a = r->Kp != K || (lda * es) % 16 != 0 || (uintptr_t)A % 16 != 0;
+  r->b = r->Kp != K || (ldb * es) % 16 != 0 || (uintptr_t)B % 16 != 0 || r->Np != N;
+  r->c = r->Np != N || ldc % 4 != 0 || (uintptr_t)C % 8 != 0;
+  if (!r->a && !r->b && !r->c) return false;
+  r->bytes_a = r->a ? round_up((size_t)M * (size_t)r->Kp * (size_t)es, 256) : 0;
+  r->bytes_b = r->b ? round_up((size_t)r->Np * (size_t)r->Kp * (size_t)es, 256) : 0;
+  r->bytes_c = r->c ? round_up((size_t)M * (size_t)r->Np * 2, 256) : 0;
+  // the repacked problem must be one the tiled kernels take
+  return tile256_ok(M, r->Np, r->Kp, r->a ? r->Kp : lda, r->b ? r->Kp : ldb, r->c ? r->Np : ldc, in_dtype);
+}
+
 }  // namespace
 
 extern "C" {
@@ -139,6 +172,12 @@ size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int in_dtype,
   if (!valid_in(in_dtype) || M <= 0 || N <= 0 || K <= 0) return 0;
   if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_SIMPLE) return 0;
   const int v = resolve(M, N, K, K, K, N, in_dtype, variant);
+  if (v == MI355_VARIANT_SIMPLE && variant == MI355_VARIANT_AUTO) {
+    // contiguous, aligned operands assumed: only K and N decide what is repacked
+    Repack r;
+    if (!repack_plan(nullptr, nullptr, nullptr, M, N, K, K, K, N, in_dtype, &r)) return 0;
+    return r.bytes_a + r.bytes_b + r.bytes_c + mi355_gemm_workspace_bytes(M, r.Np, r.Kp, in_dtype, MI355_VARIANT_AUTO);
+  }
   int splits = 1;
   if (v == MI355_VARIANT_SKINNY) splits = mi355::stream_splits(M, N, K, elem_bytes(in_dtype));
   else if (v == MI355_VARIANT_BASIC) splits = mi355::ring_splits(M, N, K, elem_bytes(in_dtype));
@@ -311,6 +350,32 @@ int mi355_gemm_tn_scaled(const void* A, const void* B, void* C, int64_t M, int64
     if (!aligned) {
       if (variant != MI355_VARIANT_AUTO) return MI355_ERR_ALIGN;
       v = MI355_VARIANT_SIMPLE;
+    }
+  }
+  if (v == MI355_VARIANT_SIMPLE && variant == MI355_VARIANT_AUTO && workspace && (uintptr_t)workspace % 256 == 0) {
+    Repack r;
+    // The streaming kernel insists on the workspace of its K split, so the rest must cover it.
+    const auto inner_ok = [&](const Repack& p) {
+      const size_t rest = workspace_bytes - (p.bytes_a + p.bytes_b + p.bytes_c);
+      return mi355_gemm_select_variant(M, p.Np, p.Kp, in_dtype) != MI355_VARIANT_SKINNY ||
+             rest >= mi355_gemm_workspace_bytes(M, p.Np, p.Kp, in_dtype, MI355_VARIANT_AUTO);
+    };
+    if (repack_plan(A, B, C, M, N, K, lda, ldb, ldc, in_dtype, &r) &&
+        workspace_bytes >= r.bytes_a + r.bytes_b + r.bytes_c && inner_ok(r)) {
+      const int64_t es = elem_bytes(in_dtype);
+      uint8_t* wa = (uint8_t*)workspace;
+      uint8_t* wb = wa + r.bytes_a;
+      uint8_t* wc = wb + r.bytes_b;
+      uint8_t* rest = wc + r.bytes_c;
+      const size_t rest_bytes = workspace_bytes - (r.bytes_a + r.bytes_b + r.bytes_c);
+      if (r.a && mi355::launch_repack_rows(A, M, K * es, lda * es, wa, M, r.Kp * es, (int)es, s) != 0) return MI355_ERR_LAUNCH;
+      if (r.b && mi355::launch_repack_rows(B, N, K * es, ldb * es, wb, r.Np, r.Kp * es, (int)es, s) != 0) return MI355_ERR_LAUNCH;
+      st = mi355_gemm_tn_scaled(r.a ? wa : A, r.b ? wb : B, r.c ? (void*)wc : C, M, r.Np, r.Kp, r.a ? r.Kp : lda,
+                                r.b ? r.Kp : ldb, r.c ? r.Np : ldc, in_dtype, out_dtype, scale, scale_a, scale_b,
+                                MI355_VARIANT_AUTO, rest_bytes ? rest : nullptr, rest_bytes, stream);
+      if (st != MI355_OK) return st;
+      if (r.c && mi355::launch_copy_out(wc, M, N, r.Np, C, ldc, s) != 0) return MI355_ERR_LAUNCH;
+      return MI355_OK;
     }
   }
   int rc;

@@ -79,5 +79,13 @@ int launch_stream(const GemmArgs& g, int in_dtype, int out_dtype, int splits, vo
 // Per-tensor e4m3 quantisation (amax -> scale -> cast); scale_amax points to two floats.
 int launch_quantize_e4m3(const void* x, int in_dtype, int64_t n, void* q, float* scale_amax, hipStream_t stream);
 int launch_simple(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
+// Repacking for problems the tiled kernels cannot address (gemm_tn_simple.hip): rows of `row_bytes`
+// bytes with stride src_ld bytes -> 16-byte aligned rows with stride dst_ld bytes, the tail of every
+// row and the rows from `rows` up to dst_rows zero-filled; and a (rows x cols) block of 16-bit
+// elements with row stride src_ld elements -> row stride dst_ld elements at any 2-byte alignment.
+int launch_repack_rows(const void* src, int64_t rows, int64_t row_bytes, int64_t src_ld, void* dst, int64_t dst_rows,
+                       int64_t dst_ld, int elem_bytes, hipStream_t stream);
+int launch_copy_out(const void* src, int64_t rows, int64_t cols, int64_t src_ld, void* dst, int64_t dst_ld,
+                    hipStream_t stream);
 
 }  // namespace mi355

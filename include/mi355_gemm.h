@@ -67,7 +67,10 @@ enum mi355_status {
  *   workspace device scratch of at least mi355_gemm_workspace_bytes(...) bytes, or NULL when
  *             that function returns 0; contents need not be initialised.  The skinny variant
  *             needs it for its K split (MI355_ERR_WORKSPACE otherwise); the tiled variant runs
- *             without its K split or tail split, i.e. slower, when it is NULL or too small
+ *             without its K split or tail split, i.e. slower, when it is NULL or too small.
+ *             MI355_VARIANT_AUTO also uses it (256-byte aligned) to repack a large problem the
+ *             tiled kernels cannot address (K*elem_bytes % 16, N % 4, strides, pointers) into
+ *             an aligned one; without it such a problem runs on the slow generic kernel
  *   stream    hipStream_t on which the kernels are enqueued (NULL = the null stream)
  *
  * Replaces test::gemm_tn_test (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92): same operand

@@ -421,6 +421,75 @@ def test_operands_with_padded_rows(abi, dt, variant):
     check(C.cpu(), A.cpu().contiguous(), B.cpu().contiguous(), scale)
 
 
+@pytest.mark.parametrize("dt,M,N,K", [
+    (torch.bfloat16, 1000, 50257, 768),        # an odd vocabulary size: N % 4 != 0
+    (torch.bfloat16, 1001, 1003, 1001),        # everything odd: K*2 % 16 != 0 too
+    (torch.float16, 515, 2050, 4100),          # N % 4 == 2, K*2 % 16 == 8
+    (torch.float8_e4m3fn, 777, 1001, 1003),    # fp8 rows of 1003 bytes
+    (torch.bfloat16, 48, 50257, 768),          # few rows: the repacked problem streams the weights
+])
+def test_auto_repacks_misaligned_problems(abi, dt, M, N, K):
+    """Problems the tiled kernels cannot address run on them all the same when the caller lends a
+    workspace: operands copied to aligned zero-padded rows, C computed padded and copied out.  The
+    result must be the one the generic kernel gives (same products, fp32 sums), nothing may be
+    written outside C, and without the workspace the call still succeeds (generic kernel)."""
+    code = ac.torch_code(dt)
+    assert abi.mi355_gemm_select_variant(M, N, K, code) == ac.SIMPLE
+    need = abi.mi355_gemm_workspace_bytes(M, N, K, code, ac.AUTO)
+    assert need > 0
+    if dt == torch.float8_e4m3fn:
+        g = torch.Generator().manual_seed(M + K)
+        A = torch.randint(0, 120, (M, K), dtype=torch.uint8, generator=g).view(dt)
+        B = torch.randint(0, 120, (N, K), dtype=torch.uint8, generator=g).view(dt)
+        scale = 2.0 ** -6
+    else:
+        A, B, scale = rand((M, K), M + K, dt), rand((N, K), N + K, dt), 1.0
+    C = run_abi(abi, A, B, ac.AUTO, scale, ldc=N + 3)          # odd row stride of C as well, NaN guards around it
+    Ad, Bd = A.cuda(), B.cuda()
+    S = torch.empty((M, N), dtype=out_dtype_of(dt), device="cuda")
+    assert ac.gemm_tn(abi, Ad, Bd, S, scale, ac.SIMPLE) == 0
+    torch.cuda.synchronize()
+    Sf = S.cpu().float()
+    d = (C.float() - Sf).abs()
+    bad = d > 2e-2 * Sf.abs() + 2e-2 * (K ** 0.5) * scale * (40.0 if dt == torch.float8_e4m3fn else 1.0)
+    assert oracle.no_nan_left(C) and int(bad.sum()) == 0, (int(bad.sum()), float(d.max()))
+    rows = torch.randperm(M, generator=torch.Generator().manual_seed(1))[:32]
+    assert oracle.rel_frobenius(C[rows], oracle.gemm_tn_fp32(A[rows], B, scale)) <= TOL[dt]
+    # no workspace: the generic kernel, same contract
+    C2 = torch.full((M, N), float("nan"), dtype=out_dtype_of(dt), device="cuda")
+    rc = abi.mi355_gemm_tn(Ad.data_ptr(), Bd.data_ptr(), C2.data_ptr(), M, N, K, K, K, N, code, ac.torch_code(C2.dtype),
+                           scale, ac.AUTO, None, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.equal(C2.cpu().view(torch.int16), S.cpu().view(torch.int16))
+
+
+def test_auto_repacks_misaligned_pointers_and_strides(abi):
+    """Aligned shape, but A starts 2 bytes into an allocation and B has a row stride that is not a
+    multiple of 16 bytes: repacked when the workspace allows, generic kernel otherwise."""
+    M, N, K = 1024, 2048, 1024
+    g = torch.Generator().manual_seed(2)
+    a_store = torch.randn(M * K + 8, generator=g).bfloat16().cuda()
+    A = a_store[1:1 + M * K].view(M, K)                        # 2-byte aligned only
+    b_store = torch.randn(N, K + 4, generator=g).bfloat16().cuda()
+    B = b_store[:, :K]                                         # row stride 2056 bytes
+    assert A.data_ptr() % 16 != 0 and (B.stride(0) * 2) % 16 != 0
+    ref = oracle.gemm_tn_fp32(A.cpu().contiguous(), B.cpu().contiguous())
+    s = torch.cuda.current_stream().cuda_stream
+    big = torch.empty(64 << 20, dtype=torch.uint8, device="cuda")
+    for ws, nbytes in ((big.data_ptr(), big.numel()), (None, 0)):
+        C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+        rc = abi.mi355_gemm_tn(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0), N, ac.BF16,
+                               ac.BF16, 1.0, ac.AUTO, ws, nbytes, s)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert oracle.no_nan_left(C) and oracle.rel_frobenius(C.cpu(), ref) <= 1e-2
+    # an explicit tiled variant still refuses
+    rc = abi.mi355_gemm_tn(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0), N, ac.BF16,
+                           ac.BF16, 1.0, ac.BASIC, big.data_ptr(), big.numel(), s)
+    assert rc in (ac.ERR_SHAPE, ac.ERR_ALIGN)
+
+
 def test_k_zero_and_empty(abi):
     A, B = torch.zeros(8, 0, dtype=torch.bfloat16), torch.zeros(4, 0, dtype=torch.bfloat16)
     C = run_abi(abi, A, B)
