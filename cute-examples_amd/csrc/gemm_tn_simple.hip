@@ -44,12 +44,20 @@ __global__ __launch_bounds__(256) void repack_rows(const uint8_t* __restrict__ s
   *(u32x4*)(dst + row * dst_ld + at) = out;
 }
 
+// One thread per four columns: the source rows are 8-byte aligned (src_ld % 4 == 0), the
+// destination has only element alignment.
 __global__ __launch_bounds__(256) void copy_out(const uint16_t* __restrict__ src, int64_t rows, int64_t cols,
                                                 int64_t src_ld, uint16_t* __restrict__ dst, int64_t dst_ld) {
+  const int64_t quads = (cols + 3) / 4;
   const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (id >= rows * cols) return;
-  const int64_t row = id / cols, col = id % cols;
-  dst[row * dst_ld + col] = src[row * src_ld + col];
+  if (id >= rows * quads) return;
+  const int64_t row = id / quads, col = (id % quads) * 4;
+  const u32x2 v = *(const u32x2*)(src + row * src_ld + col);
+  uint16_t* d = dst + row * dst_ld + col;
+  d[0] = (uint16_t)v[0];
+  if (col + 1 < cols) d[1] = (uint16_t)(v[0] >> 16);
+  if (col + 2 < cols) d[2] = (uint16_t)v[1];
+  if (col + 3 < cols) d[3] = (uint16_t)(v[1] >> 16);
 }
 
 template <class T, class OutT>
@@ -78,10 +86,10 @@ int launch_repack_rows(const void* src, int64_t rows, int64_t row_bytes, int64_t
 
 int launch_copy_out(const void* src, int64_t rows, int64_t cols, int64_t src_ld, void* dst, int64_t dst_ld,
                     hipStream_t stream) {
-  const int64_t n = rows * cols;
+  const int64_t n = rows * ((cols + 3) / 4);
   if (n == 0) return 0;
   const int64_t blocks = (n + 255) / 256;
-  if (blocks >= ((int64_t)1 << 31)) return -1;
+  if (blocks >= ((int64_t)1 << 31) || src_ld % 4 != 0 || (uintptr_t)src % 8 != 0) return -1;
   hipLaunchKernelGGL(copy_out, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint16_t*)src, rows, cols, src_ld,
                      (uint16_t*)dst, dst_ld);
   return hipGetLastError() == hipSuccess ? 0 : -1;
