@@ -19,7 +19,10 @@ LIB = os.path.join(OUT, "libmi355gemm.so")
 
 HIP_SOURCES = ["gemm_api.hip", "gemm_tn_simple.hip", "gemm_tn_ring_bf16.hip", "gemm_tn_ring_f16.hip", "gemm_tn_ring_e4m3.hip", "gemm_tn_ring_mx.hip", "ring_plan.hip", "gemm_tn_pingpong.hip", "gemm_tn_stream.hip", "quantize_e4m3.hip", "mx_scales.hip"]
 
-CHECKED_SOURCE = "gemm_tn_ring_mx.hip"   # its device assembly is verified after compilation
+# Sources whose device assembly is verified after compilation (check_async_loads.py): the copies'
+# LDS base in all of them, the asynchronous scale loads in the block-scaled one.
+CHECKED_SOURCES = ["gemm_tn_ring_bf16.hip", "gemm_tn_ring_f16.hip", "gemm_tn_ring_e4m3.hip", "gemm_tn_ring_mx.hip"]
+CHECKED_SOURCE = "gemm_tn_ring_mx.hip"
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -53,16 +56,21 @@ def build_lib():
     with tempfile.TemporaryDirectory() as tmp:
         def compile_one(src):
             obj = os.path.join(tmp, src.replace(".hip", ".o"))
-            extra = ["-save-temps=obj"] if src == CHECKED_SOURCE else []
+            extra = ["-save-temps=obj"] if src in CHECKED_SOURCES else []
             _run([hipcc] + HIPCC_FLAGS + ["-c"] + extra + ["-o", obj, os.path.join(CSRC, src)])
             return obj
 
         with ThreadPoolExecutor(max_workers=min(len(HIP_SOURCES), os.cpu_count() or 1)) as pool:
             objs = list(pool.map(compile_one, HIP_SOURCES))
-        asm = glob.glob(os.path.join(tmp, CHECKED_SOURCE.replace(".hip", "") + "-hip-amdgcn-*gfx950.s"))
-        if len(asm) != 1:
-            raise RuntimeError("expected one device assembly file for %s, found %r" % (CHECKED_SOURCE, asm))
-        print("check_async_loads: %d scale operands ok" % check_async_loads.check(asm[0]), flush=True)
+        copies = 0
+        for src in CHECKED_SOURCES:
+            asm = glob.glob(os.path.join(tmp, src.replace(".hip", "") + "-hip-amdgcn-*gfx950.s"))
+            if len(asm) != 1:
+                raise RuntimeError("expected one device assembly file for %s, found %r" % (src, asm))
+            copies += check_async_loads.check_lds_base(asm[0])
+            if src == CHECKED_SOURCE:
+                print("check_async_loads: %d scale operands ok" % check_async_loads.check(asm[0]), flush=True)
+        print("check_async_loads: %d direct-to-LDS copies ok" % copies, flush=True)
         _run([hipcc] + HIPCC_FLAGS + ["-o", LIB] + objs)
     return LIB
 

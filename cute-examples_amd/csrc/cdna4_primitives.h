@@ -78,6 +78,18 @@ __device__ __forceinline__ void load_8B_async(u32x2& dst, __amdgpu_buffer_rsrc_t
                : "memory");
 }
 
+// The two halves of dma_16B_to_lds_at as separate statements, so that other instructions can sit
+// between the write of M0 and the copy that uses it.
+template <uint32_t kLdsAdd>
+__device__ __forceinline__ void dma_set_lds_base(uint32_t lds_base) {
+  asm volatile("s_add_u32 m0, %0, %1" ::"s"(__builtin_amdgcn_readfirstlane(lds_base)), "n"(kLdsAdd) : "scc");
+}
+__device__ __forceinline__ void dma_16B_to_lds_base_set(uint32_t voffset, __amdgpu_buffer_rsrc_t rsrc, uint32_t soffset) {
+  asm volatile("buffer_load_dwordx4 %0, %1, %2 offen lds" ::"v"(voffset), "s"(rsrc),
+               "s"(__builtin_amdgcn_readfirstlane(soffset))
+               : "memory");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");

@@ -218,6 +218,17 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     if constexpr (kRaggedK) v = soff == soff_tail ? tail[j % kPar] : v;
     dma_16B_to_lds_at<slot * kSlotBytes + j * kCopyBytes>(dma_wave, v + j * step, rsrc, soff);
   };
+  // The same in two steps: the LDS base first, the copy later.
+  auto prep_rows = [&](auto jc, auto slotc, uint32_t dma_wave) __attribute__((always_inline)) {
+    dma_set_lds_base<decltype(slotc)::value * kSlotBytes + decltype(jc)::value * kCopyBytes>(dma_wave);
+  };
+  auto fire_rows = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, uint32_t soff, const uint32_t* voff, const uint32_t* tail,
+                       uint32_t step) __attribute__((always_inline)) {
+    constexpr int j = decltype(jc)::value;
+    uint32_t v = voff[j % kPar];
+    if constexpr (kRaggedK) v = soff == soff_tail ? tail[j % kPar] : v;
+    dma_16B_to_lds_base_set(v + j * step, rsrc, soff);
+  };
   auto copy_a = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, auto slotc, uint32_t soff) __attribute__((always_inline)) {
     copy_rows(rsrc, jc, slotc, soff, voff_a, tail_a, a_step, dma_wave_a);
   };
@@ -441,17 +452,33 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
           wait_vmcnt<kCph + (kMx ? 2 : 0)>();  // the two scale requests of this k-step are younger still
           __builtin_amdgcn_s_barrier();
         }
+        // Copy c is "prepared" (its LDS base written to M0) one MFMA before it is issued when it
+        // is alone at its position; otherwise M0 is written right in front of it.
         if constexpr (p >= kFirstCopy) {
           constexpr int c0 = first_copy_at(p, kFirstCopy, kCopySpan, kCopies);
           static_for<kMaxCopiesPerGap>([&](auto ic) __attribute__((always_inline)) {
             constexpr int c = c0 + decltype(ic)::value;
             if constexpr (c < kCopies && copy_position(c, kFirstCopy, kCopySpan, kCopies) == p) {
-              if constexpr (c < kCphB)
-                copy_b(rsrc_b, std::integral_constant<int, c>{}, std::integral_constant<uint32_t, slot_a>{}, soff_b);
-              else
-                copy_a(rsrc_a, std::integral_constant<int, c - kCphB>{}, std::integral_constant<uint32_t, slot_b>{}, soff_a);
+              constexpr bool prepared = c > 0 && copy_position(c - 1, kFirstCopy, kCopySpan, kCopies) < p - 1 &&
+                                        (c + 1 >= kCopies || copy_position(c + 1, kFirstCopy, kCopySpan, kCopies) > p);
+              if constexpr (c < kCphB) {
+                if constexpr (!prepared) prep_rows(std::integral_constant<int, c>{}, std::integral_constant<uint32_t, slot_a>{}, dma_wave_b);
+                fire_rows(rsrc_b, std::integral_constant<int, c>{}, soff_b, voff_b, tail_b, b_step);
+              } else {
+                if constexpr (!prepared) prep_rows(std::integral_constant<int, c - kCphB>{}, std::integral_constant<uint32_t, slot_b>{}, dma_wave_a);
+                fire_rows(rsrc_a, std::integral_constant<int, c - kCphB>{}, soff_a, voff_a, tail_a, a_step);
+              }
             }
           });
+        }
+        if constexpr (p + 1 >= kFirstCopy && p + 1 < 2 * kMfmaPerSlice) {
+          constexpr int c = first_copy_at(p + 1, kFirstCopy, kCopySpan, kCopies);
+          if constexpr (c > 0 && c < kCopies && copy_position(c, kFirstCopy, kCopySpan, kCopies) == p + 1 &&
+                        copy_position(c - 1, kFirstCopy, kCopySpan, kCopies) < p &&
+                        (c + 1 >= kCopies || copy_position(c + 1, kFirstCopy, kCopySpan, kCopies) > p + 1)) {
+            if constexpr (c < kCphB) prep_rows(std::integral_constant<int, c>{}, std::integral_constant<uint32_t, slot_a>{}, dma_wave_b);
+            else prep_rows(std::integral_constant<int, c - kCphB>{}, std::integral_constant<uint32_t, slot_b>{}, dma_wave_a);
+          }
         }
         if constexpr (kRowSliced)
           mfma_rows(phase, std::integral_constant<int, s>{}, std::integral_constant<int, u>{});

@@ -110,3 +110,30 @@ def test_lds_swizzle_is_a_bijection_and_conflict_free():
     # and the layout without the swizzle would conflict, so the check has teeth
     plain = [(l % 16) * 128 + (l // 16) * 16 for l in range(64)]
     assert not conflict_free(plain)
+
+
+RING_HEAD = "_ZN5mi35512_GLOBAL__N_117gemm_tn_tile_ringINS_4BF16ES2_Lb0ELi256ELi2ELi256EEEvNS_8GemmArgsE: ; @kernel\n"
+SET = "\ts_add_u32 m0, s12, 0x8000\n"
+COPY = "\tbuffer_load_dwordx4 v175, s[40:43], s61 offen lds\n"
+MFMA16 = "\tv_mfma_f32_16x16x32_bf16 a[0:3], v[2:5], v[6:9], a[0:3]\n"
+
+
+def run_lds(tmp_path, body):
+    f = tmp_path / "r.s"
+    f.write_text(RING_HEAD + body + TAIL)
+    return check_async_loads.check_lds_base(str(f))
+
+
+def test_lds_base_check_accepts_a_write_one_mfma_ahead(tmp_path):
+    assert run_lds(tmp_path, SET + MFMA16 + COPY + MFMA16 + SET + COPY) == 2
+
+
+@pytest.mark.parametrize("body,msg", [
+    (SET + "\ts_mov_b32 m0, -1\n" + COPY, "written by something else"),
+    (SET + SET + COPY, "two writes of M0"),
+    (SET + COPY + COPY, "without its own write"),
+    (SET + COPY + SET, "no copy uses"),
+])
+def test_lds_base_check_rejects(tmp_path, body, msg):
+    with pytest.raises(RuntimeError, match=msg):
+        run_lds(tmp_path, body)
