@@ -14,6 +14,19 @@ int elem_bytes(int dtype) { return dtype == MI355_E4M3 ? 1 : 2; }
 bool valid_in(int d) { return d == MI355_BF16 || d == MI355_F16 || d == MI355_E4M3; }  // MI355_F32: quantiser only
 bool valid_out(int d) { return d == MI355_BF16 || d == MI355_F16; }
 
+// Sizes far beyond what 288 GB of HBM can hold are refused up front, so that none of the size
+// arithmetic below (byte counts, tile counts, workspace sizes) can leave 64 bits: every extent and
+// row stride is at most 2^40 and every array has at most 2^50 elements.
+constexpr int64_t kMaxExtent = (int64_t)1 << 40;
+constexpr double kMaxElements = 1125899906842624.0;  // 2^50
+bool array_ok(int64_t rows, int64_t ld) {
+  return rows <= kMaxExtent && ld <= kMaxExtent && (double)rows * (double)ld <= kMaxElements;
+}
+bool extents_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc) {
+  return K <= kMaxExtent && array_ok(M, lda) && array_ok(N, ldb) && array_ok(M, ldc) && array_ok(M, N) &&
+         array_ok(M, K) && array_ok(N, K);
+}
+
 // Constraints of the 256x256-tile kernels beyond the generic ones.
 bool tile256_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int in_dtype) {
   const int64_t es = elem_bytes(in_dtype);
@@ -42,6 +55,7 @@ int check_common(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int6
   if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_SIMPLE) return MI355_ERR_VARIANT;
   if (M < 0 || N < 0 || K < 0) return MI355_ERR_SHAPE;
   if (lda < K || ldb < K || ldc < N) return MI355_ERR_SHAPE;
+  if (!extents_ok(M, N, K, lda, ldb, ldc)) return MI355_ERR_SHAPE;
   return MI355_OK;
 }
 
@@ -119,7 +133,9 @@ const char* mi355_gemm_strerror(int status) {
 int mi355_gemm_tile_coord(int64_t block, int64_t tiles_m, int64_t tiles_n, int64_t* tile_m,
                           int64_t* tile_n) {
   if (!tile_m || !tile_n) return MI355_ERR_NULL;
-  if (tiles_m <= 0 || tiles_n <= 0 || block < 0 || block >= tiles_m * tiles_n) return MI355_ERR_SHAPE;
+  if (tiles_m <= 0 || tiles_n <= 0 || block < 0) return MI355_ERR_SHAPE;
+  if (tiles_m > ((int64_t)1 << 60) / tiles_n) return MI355_ERR_SHAPE;   // the map's arithmetic stays inside 64 bits
+  if (block >= tiles_m * tiles_n) return MI355_ERR_SHAPE;
   mi355::tile_coord(block, tiles_m, tiles_n, tile_m, tile_n);
   return MI355_OK;
 }
@@ -134,7 +150,7 @@ int mi355_gemm_check(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, 
 
 int mi355_gemm_select_variant(int64_t M, int64_t N, int64_t K, int in_dtype) {
   if (!valid_in(in_dtype)) return MI355_ERR_DTYPE;
-  if (M < 0 || N < 0 || K < 0) return MI355_ERR_SHAPE;
+  if (M < 0 || N < 0 || K < 0 || !extents_ok(M, N, K, K, K, N)) return MI355_ERR_SHAPE;
   return resolve(M, N, K, K, K, N, in_dtype, MI355_VARIANT_AUTO);
 }
 
@@ -142,7 +158,7 @@ int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant, 
                     int* k_splits, int* tail_tiles, int* tail_splits) {
   if (!valid_in(in_dtype)) return MI355_ERR_DTYPE;
   if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_SIMPLE) return MI355_ERR_VARIANT;
-  if (M < 0 || N < 0 || K < 0) return MI355_ERR_SHAPE;
+  if (M < 0 || N < 0 || K < 0 || !extents_ok(M, N, K, K, K, N)) return MI355_ERR_SHAPE;
   const int v = resolve(M, N, K, K, K, N, in_dtype, variant);
   if (v < 0) return v;
   int rows = 0, cols = 0, splits = 1, tt = 0, ts = 1;
@@ -171,6 +187,7 @@ int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant, 
 size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int in_dtype, int variant) {
   if (!valid_in(in_dtype) || M <= 0 || N <= 0 || K <= 0) return 0;
   if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_SIMPLE) return 0;
+  if (!extents_ok(M, N, K, K, K, N)) return 0;
   const int v = resolve(M, N, K, K, K, N, in_dtype, variant);
   if (v == MI355_VARIANT_SIMPLE && variant == MI355_VARIANT_AUTO) {
     // contiguous, aligned operands assumed: only K and N decide what is repacked
@@ -191,7 +208,7 @@ size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int in_dtype,
 
 int mi355_quantize_e4m3(const void* x, int x_dtype, int64_t n, void* x_q, float* scale_amax, void* stream) {
   if (x_dtype != MI355_BF16 && x_dtype != MI355_F16 && x_dtype != MI355_F32) return MI355_ERR_DTYPE;
-  if (n < 0) return MI355_ERR_SHAPE;
+  if (n < 0 || (double)n > kMaxElements) return MI355_ERR_SHAPE;
   if (!scale_amax || (n > 0 && (!x || !x_q))) return MI355_ERR_NULL;
   if ((uintptr_t)x % 16 != 0 || (uintptr_t)x_q % 8 != 0 || (uintptr_t)scale_amax % 4 != 0) return MI355_ERR_ALIGN;
   return mi355::launch_quantize_e4m3(x, x_dtype, n, x_q, scale_amax, (hipStream_t)stream) == 0 ? MI355_OK
@@ -199,12 +216,13 @@ int mi355_quantize_e4m3(const void* x, int x_dtype, int64_t n, void* x_q, float*
 }
 
 size_t mi355_mx_shuffled_bytes(int64_t rows, int64_t K) {
-  if (rows <= 0 || K <= 0 || K % 128 != 0) return 0;
+  if (rows <= 0 || K <= 0 || K % 128 != 0 || !array_ok(rows, K)) return 0;
   return mi355::mx_shuffled_bytes(rows, K);
 }
 
 int mi355_mx_shuffle_scales(const uint8_t* scales, int64_t rows, int64_t K, int64_t ld, uint8_t* out, void* stream) {
   if (rows < 0 || K < 0 || K % 128 != 0 || ld < K / 32) return MI355_ERR_SHAPE;
+  if (!array_ok(rows, K) || !array_ok(rows, ld)) return MI355_ERR_SHAPE;
   if (rows == 0 || K == 0) return MI355_OK;
   if (!scales || !out) return MI355_ERR_NULL;
   if ((uintptr_t)out % 8 != 0) return MI355_ERR_ALIGN;
@@ -214,7 +232,7 @@ int mi355_mx_shuffle_scales(const uint8_t* scales, int64_t rows, int64_t K, int6
 int mi355_quantize_mxfp8(const void* x, int x_dtype, int64_t rows, int64_t K, int64_t ldx, void* x_q,
                          uint8_t* scales, int scales_shuffled, void* stream) {
   if (x_dtype != MI355_BF16 && x_dtype != MI355_F16 && x_dtype != MI355_F32) return MI355_ERR_DTYPE;
-  if (rows < 0 || K < 0 || K % 32 != 0 || ldx < K) return MI355_ERR_SHAPE;
+  if (rows < 0 || K < 0 || K % 32 != 0 || ldx < K || !array_ok(rows, ldx)) return MI355_ERR_SHAPE;
   if (scales_shuffled && K % 128 != 0) return MI355_ERR_SHAPE;
   if (rows == 0 || K == 0) return MI355_OK;
   if (!x || !x_q || !scales) return MI355_ERR_NULL;
@@ -228,6 +246,7 @@ int mi355_gemm_mx_check(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ld
   if (!valid_out(out_dtype)) return MI355_ERR_DTYPE;
   if (M < 0 || N < 0 || K < 0) return MI355_ERR_SHAPE;
   if (lda < K || ldb < K || ldc < N) return MI355_ERR_SHAPE;
+  if (!extents_ok(M, N, K, lda, ldb, ldc)) return MI355_ERR_SHAPE;
   if (K % 128 != 0) return MI355_ERR_SHAPE;
   if (M == 0 || N == 0) return MI355_OK;
   if (K > 0 && !tile256_ok(M, N, K, lda, ldb, ldc, MI355_E4M3)) return MI355_ERR_SHAPE;
@@ -250,7 +269,7 @@ size_t mx_partial_bytes(int64_t M, int64_t N, int64_t K, int* splits, int* tail_
 }  // namespace
 
 size_t mi355_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int scales_shuffled) {
-  if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0) return 0;
+  if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0 || !extents_ok(M, N, K, K, K, N)) return 0;
   return mx_partial_bytes(M, N, K, nullptr, nullptr, nullptr) +
          (scales_shuffled ? 0 : mi355::mx_shuffled_bytes(M, K) + mi355::mx_shuffled_bytes(N, K));
 }
@@ -288,6 +307,7 @@ int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, in
     g.mx_b = scale_b;
   } else {
     if (ld_scale_a < K / 32 || ld_scale_b < K / 32) return MI355_ERR_SHAPE;
+    if (!array_ok(M, ld_scale_a) || !array_ok(N, ld_scale_b)) return MI355_ERR_SHAPE;
     const size_t bytes_a = mi355::mx_shuffled_bytes(M, K), bytes_b = mi355::mx_shuffled_bytes(N, K);
     if (!workspace || workspace_bytes < bytes_a + bytes_b || (uintptr_t)workspace % 16 != 0) return MI355_ERR_WORKSPACE;
     uint8_t* wa = (uint8_t*)workspace;

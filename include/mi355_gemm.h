@@ -78,6 +78,9 @@ enum mi355_status {
  * by the tile is not required (the tiled variants need K*elem_bytes % 16 == 0, row strides that
  * are multiples of 16 bytes, N % 4 == 0, ldc % 4 == 0, 256 rows of A and of B below 2 GiB and
  * 256*ldc below 2^29 elements; MI355_VARIANT_AUTO routes anything else to the generic kernel).
+ * Every entry point of this header refuses (MI355_ERR_SHAPE, or 0 from the size queries) an
+ * extent or row stride above 2^40 and an array of more than 2^50 elements, so that its size
+ * arithmetic stays inside 64 bits.
  * Asynchronous: returns after enqueueing.
  */
 int mi355_gemm_tn(const void *A, const void *B, void *C,

@@ -58,6 +58,31 @@ def test_check(abi, args, want):
     assert abi.mi355_gemm_check(*args) == want
 
 
+def test_sizes_beyond_any_memory_are_refused_before_any_arithmetic_on_them(abi):
+    """Extents above 2^40 and arrays above 2^50 elements come back as MI355_ERR_SHAPE (0 from the
+    size queries) from every entry point: products of such sizes would leave 64 bits."""
+    huge = [2**62, 2**63 - 1, 2**48 + 16, 2**41]
+    for h in huge:
+        assert abi.mi355_gemm_check(256, 256, h, h, h, 256, ac.BF16, ac.BF16, ac.AUTO) == ac.ERR_SHAPE
+        assert abi.mi355_gemm_check(h, 256, 64, 64, 64, 256, ac.BF16, ac.BF16, ac.AUTO) == ac.ERR_SHAPE
+        assert abi.mi355_gemm_check(256, 256, 64, 64, 64, h, ac.BF16, ac.BF16, ac.AUTO) == ac.ERR_SHAPE
+        assert abi.mi355_gemm_select_variant(8253, 160, h, ac.F16) == ac.ERR_SHAPE
+        assert abi.mi355_gemm_select_variant(h, h, 64, ac.F16) == ac.ERR_SHAPE
+        assert ac.plan(abi, 256, h, 256, ac.E4M3)[0] == ac.ERR_SHAPE
+        assert abi.mi355_gemm_workspace_bytes(16, h, 4096, ac.BF16, ac.AUTO) == 0
+        assert abi.mi355_gemm_mx_check(256, 256, h, h, h, 256, ac.BF16) == ac.ERR_SHAPE
+        assert abi.mi355_gemm_mx_workspace_bytes(h, 256, 128, 0) == 0
+        assert abi.mi355_mx_shuffled_bytes(h, 128) == 0
+        assert abi.mi355_quantize_e4m3(None, ac.BF16, max(h, 2**50 + 1), None, None, None) == ac.ERR_SHAPE
+        assert abi.mi355_quantize_mxfp8(None, ac.BF16, 4, 128, h, None, None, 0, None) == ac.ERR_SHAPE
+        a, b = ctypes.c_int64(), ctypes.c_int64()
+        assert abi.mi355_gemm_tile_coord(5, h, h, ctypes.byref(a), ctypes.byref(b)) == ac.ERR_SHAPE
+    # 2^25 x 2^25 x 2^25 is within the bound (2^50 elements per array): the queries answer
+    assert abi.mi355_gemm_select_variant(2**25, 2**25, 2**25, ac.BF16) == ac.SIMPLE      # rows too long for the tiled kernels
+    assert abi.mi355_gemm_select_variant(2**26, 2**25, 64, ac.BF16) == ac.ERR_SHAPE     # C would have 2^51 elements
+    assert abi.mi355_gemm_tile_coord(5, 2**29, 2**29, ctypes.byref(a), ctypes.byref(b)) == ac.OK
+
+
 def test_gemm_tn_rejects_before_any_device_access(abi):
     """Bad arguments and NULL pointers come back as codes without a GPU present."""
     f = abi.mi355_gemm_tn
