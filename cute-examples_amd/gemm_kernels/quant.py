@@ -31,7 +31,8 @@ def quantize_e4m3_torch(x):
     """The same contract in torch ops, on whatever device x lives on."""
     xf = x.detach().float()
     amax = xf.abs().amax()
-    scale = torch.where(amax > 0, amax / E4M3_MAX, torch.ones_like(amax))
+    # A tensor divisor: with a Python scalar torch multiplies by the reciprocal on a device, one ulp off.
+    scale = torch.where(amax > 0, amax / torch.full_like(amax, E4M3_MAX), torch.ones_like(amax))
     # Clamp before the cast: torch's e4m3fn cast maps values that round above 448 to NaN.
     x_q = (xf / scale).clamp_(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
     return x_q, scale
@@ -55,6 +56,10 @@ def quantize_mxfp8_torch(x):
     amax = xf.abs().amax(-1)
     _, ex = torch.frexp(amax)                       # amax = m * 2^ex, m in [0.5, 1): floor(log2) = ex - 1
     byte = torch.where(amax > 0, (ex - 1 - 8 + 127).clamp(0, 254), torch.full_like(ex, 127))
-    scaled = torch.ldexp(xf, (127 - byte)[..., None])
+    # 1/scale = 2^(127-byte), built from its bits (exponent field 254-byte; 2^-127 is subnormal) so that
+    # the product is exact on every device: torch.ldexp goes through pow, which is not on a GPU.
+    field = (254 - byte).to(torch.int32)
+    inv_scale = torch.where(field > 0, field << 23, torch.full_like(field, 0x00400000)).view(torch.float32)
+    scaled = xf * inv_scale[..., None]
     x_q = scaled.clamp_(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn).reshape(rows, K)
     return x_q, byte.to(torch.uint8)

@@ -314,3 +314,25 @@ def test_rejects_bad_arguments(abi):
     rc = abi.mi355_gemm_tn_mxfp8(Ad.data_ptr(), Ad.data_ptr(), C.data_ptr(), 256, 256, 128, 128, 128, 256, None, 4,
                                  sad.data_ptr(), 4, 0, ac.BF16, None, 0, s)
     assert rc == ac.ERR_NULL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("std", [1.0, 1e-4, 30.0])
+def test_torch_op_quantisers_agree_with_the_kernels_on_the_device(dtype, std):
+    """gemm_kernels.quant's torch-op versions state the same contract "on whatever device"; on the GPU
+    that needs exact arithmetic (torch.ldexp and division by a Python scalar are not exact there)."""
+    import gemm_kernels
+    from gemm_kernels.quant import quantize_e4m3_torch, quantize_mxfp8_torch
+    x = (torch.randn(257, 512, device="cuda", generator=torch.Generator(device="cuda").manual_seed(5)) * std).to(dtype)
+
+    def same_codes(a, b):   # the sign of a zero aside
+        a, b = a.view(torch.uint8), b.view(torch.uint8)
+        nz = (b & 0x7f) != 0
+        return torch.equal(a[nz], b[nz]) and not (a[~nz] & 0x7f).any()
+
+    q, s = gemm_kernels.quantize_mxfp8(x)
+    qt, st = quantize_mxfp8_torch(x)
+    assert torch.equal(s, st) and same_codes(q, qt)
+    q, s = gemm_kernels.quantize_e4m3(x)
+    qt, st = quantize_e4m3_torch(x)
+    assert float(s) == float(st) and same_codes(q, qt)
