@@ -11,6 +11,7 @@ namespace mi355 {
 namespace {
 
 constexpr int64_t kSlots = 256;  // one work item per CU of an MI355X; heuristics only, so no device query
+constexpr int64_t kSmallProblemTiles = 2 * kSlots;  // 128x128 tiles that are resident all at once
 
 int64_t k_steps_of(int64_t K, int elem_bytes) { return (K * elem_bytes + kRowBytes - 1) / kRowBytes; }
 
@@ -59,14 +60,16 @@ void tail_plan(int64_t tiles, int64_t steps, int* tail_tiles, int* tail_splits) 
 }
 
 // Estimated duration, in microseconds, of the problem on tile shape `tile`, fitted to timings of
-// twenty mid-sized bf16 and fp8 problems per tile shape (mean regret of the choice 3 %):
+// 124 bf16 and fp8 problems of 1-400 GFLOP per tile shape:
 //   rounds x (k-steps per item x time of a k-step + start-up and store of a tile) + reduce
 // A k-step is 128 bytes of K per row for every input type and takes the same time for all of them.
-//   256x256  1.45 us when (nearly) all CUs are busy, 1.2 us otherwise (higher clock); a last round
-//            that gets a tail split counts 1/S of a round plus 0.2
+//   256x256  1.45 us when (nearly) all CUs are busy, 1.2 us otherwise (higher clock), also in a last
+//            round that is not nearly full; a last round that gets a tail split counts 1/S of a
+//            round plus 0.2
 //   256x128  0.85 us: half the MFMA work of a 256x256 tile, three quarters of its copies
-//   128x128  0.5 us (a quarter of the work, half of the copies), 0.75 us when either dimension has
-//            fewer than 16 tiles (measured; such problems re-read one operand from far away)
+//   128x128  0.45 us + 1/800 us per k-step of the item (a quarter of the work, half of the copies; 0.49 us
+//            measured at 32 k-steps, 0.61 at 128: long items run at a lower clock), 0.75 us when either
+//            dimension has fewer than 16 tiles (measured; such problems re-read one operand from far away)
 //   reduce   the partial planes are read back at about 5 TB/s, plus a launch
 double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
   const int64_t rows = ring_tile_rows(tile), cols = ring_tile_cols(tile);
@@ -81,12 +84,19 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
     fixed_us = 6.0;
     int tail_tiles, tail_splits;
     tail_plan(tiles, steps, &tail_tiles, &tail_splits);
-    if (tail_tiles) rounds = (double)(tiles / kSlots) + 1.0 / tail_splits + 0.2;
+    if (tail_tiles) {
+      rounds = (double)(tiles / kSlots) + 1.0 / tail_splits + 0.2;
+    } else if (s == 1 && items > kSlots) {
+      // full rounds, then a last round that runs at the higher clock unless it is (nearly) full too
+      const int64_t rest = items % kSlots;
+      const double last = rest == 0 ? 0.0 : (double)steps * (rest >= 224 ? 1.45 : 1.2) + fixed_us;
+      return (double)(items / kSlots) * ((double)steps * 1.45 + fixed_us) + last;
+    }
   } else if (tile == kRingTile256x128) {
     step_us = 0.85;
     fixed_us = 6.0;
   } else {
-    step_us = (tm < tn ? tm : tn) >= 16 ? 0.5 : 0.75;
+    step_us = (tm < tn ? tm : tn) >= 16 ? 0.45 + 0.00125 * (double)(steps / s) : 0.75;
     fixed_us = 4.0;
   }
   const double reduce_us = s > 1 ? (double)s * (double)M * (double)N * 4.0 / 5.0e6 + 2.0 : 0.0;
@@ -96,15 +106,18 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
 }  // namespace
 
 // Tile the single-group kernel should use (256, 128 or kRingTile256x128): the shortest estimate,
-// except that 128x128 is kept when nothing beats it by 10 % (the estimates of the small tile are
-// the least reliable, and it was the only alternative to 256x256 before) and 256x256 is preferred
-// over 256x128 within 5 % (it moves fewer bytes).
+// except that 256x256 is preferred over 256x128 within 5 % (it moves fewer bytes) and that a small
+// problem (at most two 128x128 tiles per CU) stays on 128x128 tiles unless a larger tile beats them
+// by 10 %, a larger one unless beaten by 6 %.  (With 10 % for all sizes the small tile was
+// picked on large problems where 256x256 measured 20-40 % faster; with no margin on mid-sized fp8
+// problems where the small tile measured 7-15 % faster.  Mean regret over 124 measured problems: 0.9 %.)
 int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes) {
   const double e256 = estimate_us(256, M, N, K, elem_bytes);
   const double e128 = estimate_us(128, M, N, K, elem_bytes);
   const double e2 = estimate_us(kRingTile256x128, M, N, K, elem_bytes);
   const double best_large = e256 <= 1.05 * e2 ? e256 : e2;
-  if (e128 <= 1.1 * best_large) return 128;
+  const double margin = tiles_of(M, N, 128) <= kSmallProblemTiles ? 1.1 : 1.06;
+  if (e128 <= margin * best_large) return 128;
   return e256 <= 1.05 * e2 ? 256 : kRingTile256x128;
 }
 
