@@ -141,31 +141,41 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   const uint32_t total_tiles = tiles_m * tiles_n;  // the launcher keeps items below 2^31
   // Work items are (tile, split) pairs, split-major, so that workgroups running together read the
   // same range of K.  With a uniform K split every tile has g.splits items; with a tail split only
-  // the last g.tail_tiles tiles are cut (g.tail_splits ways) and come after all whole tiles.
+  // the last g.tail_tiles tiles are cut (g.tail_splits ways, into ranges of k-steps that differ by
+  // at most one when the k-steps do not divide) and come after all whole tiles.
   // steps is the number of k-steps of the current item.
   const uint32_t tail_tiles = (uint32_t)g.tail_tiles, tail_splits = (uint32_t)g.tail_splits;
   const uint32_t whole_tiles = total_tiles - tail_tiles;  // tail_tiles == 0 unless g.splits == 1
   const uint32_t total_items = tail_tiles ? whole_tiles + tail_tiles * tail_splits : total_tiles * (uint32_t)g.splits;
-  const uint32_t steps_split = __builtin_amdgcn_readfirstlane(k_steps / (uint32_t)(tail_tiles ? tail_splits : g.splits));
+  const uint32_t steps_split = __builtin_amdgcn_readfirstlane(k_steps / (uint32_t)g.splits);  // uniform split: divides
   uint32_t steps = 0;
-  // item -> (tile number in tile-map order, split, whether it writes fp32 partials); sets steps.
-  auto decode_item = [&](uint32_t it, uint32_t* tile, uint32_t* split_of) __attribute__((always_inline)) -> bool {
+  // item -> (tile number in tile-map order, split, first k-step, whether it writes fp32 partials);
+  // sets steps.
+  auto decode_item = [&](uint32_t it, uint32_t* tile, uint32_t* split_of, uint32_t* first_step)
+      __attribute__((always_inline)) -> bool {
     if (tail_tiles) {
       if (it < whole_tiles) {
         *tile = it;
         *split_of = 0;
+        *first_step = 0;
         steps = k_steps;
         return false;
       }
       const uint32_t j = it - whole_tiles;
+      const uint32_t sp = j / tail_tiles;
       *tile = whole_tiles + j % tail_tiles;
-      *split_of = j / tail_tiles;
-      steps = steps_split;
+      *split_of = sp;
+      // k-steps [sp*k/S, (sp+1)*k/S): every step once, lengths within one of each other
+      const uint32_t begin = __builtin_amdgcn_readfirstlane(sp * k_steps / tail_splits);
+      const uint32_t end = __builtin_amdgcn_readfirstlane((sp + 1) * k_steps / tail_splits);
+      *first_step = begin;
+      steps = end - begin;
       return true;
     }
     *tile = it % total_tiles;
     *split_of = it / total_tiles;
     steps = steps_split;
+    *first_step = __builtin_amdgcn_readfirstlane(*split_of * steps_split);
     return g.splits > 1;
   };
 
@@ -351,9 +361,9 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
 
   uint32_t item = blockIdx.x;
   uint32_t tile_m, tile_n, tile_no, split;
-  bool partial_item = decode_item(item, &tile_no, &split);
+  uint32_t step0;  // first k-step of the current item
+  bool partial_item = decode_item(item, &tile_no, &split, &step0);
   tile_coord_t<uint32_t>(tile_no, tiles_m, tiles_n, &tile_m, &tile_n);
-  uint32_t step0 = __builtin_amdgcn_readfirstlane(split * steps);  // first k-step of the current item
   __amdgpu_buffer_rsrc_t rsrc_a = panel_a((int64_t)tile_m * kTile), rsrc_b = panel_b((int64_t)tile_n * kTileN);
   if constexpr (kMx) mx_open_tile(tile_m, tile_n, step0);  // before the copies: see the waits
   open_tile(rsrc_a, rsrc_b, step0);
@@ -505,9 +515,8 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     item += gridDim.x;
     const bool more = item < total_items;
     if (more) {
-      partial_item = decode_item(item, &tile_no, &split);
+      partial_item = decode_item(item, &tile_no, &split, &step0);
       tile_coord_t<uint32_t>(tile_no, tiles_m, tiles_n, &tile_m, &tile_n);
-      step0 = __builtin_amdgcn_readfirstlane(split * steps);
       rsrc_a = panel_a((int64_t)tile_m * kTile);
       rsrc_b = panel_b((int64_t)tile_n * kTileN);
       if constexpr (kMx) mx_open_tile(tile_m, tile_n, step0);

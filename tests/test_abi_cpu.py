@@ -301,7 +301,7 @@ def test_plan_invariants_over_random_shapes(abi):
                 if tail_tiles:
                     assert (rows, cols) == (256, 256) and splits == 1 and tail_splits > 1
                     assert 256 <= tiles <= 3 * 256 and tail_tiles == tiles % 256
-                    assert tail_tiles * tail_splits <= 256 and steps % tail_splits == 0 and steps // tail_splits >= 16
+                    assert tail_tiles * tail_splits <= 256 and steps // tail_splits >= 16      # uneven cuts allowed
                     want = tail_tiles * tail_splits * 256 * 256 * 4
                 seen.add((rows, cols, splits > 1, tail_tiles > 0))
             assert abi.mi355_gemm_workspace_bytes(M, N, K, dt, ac.AUTO) == want, (M, N, K)

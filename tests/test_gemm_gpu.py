@@ -301,12 +301,17 @@ def test_basic_kernel_with_128_tiles_and_k_splits(abi, dt, M, N, K):
     (torch.bfloat16, 4352, 4352, 4096),        # 289 tiles: one full round + 33 tiles cut in four
     (torch.float8_e4m3fn, 4096, 6144, 8192),
     (torch.float16, 4000, 6100, 4200),         # ragged M, N and last k-step: 384 tiles of 256, 66 k-steps cut in two
+    (torch.bfloat16, 5746, 5832, 5648),        # 529 tiles: 17 cut in five, 89 k-steps (the last ragged): items of 17 and 18
+    (torch.bfloat16, 4096, 4352, 3008),        # 272 tiles: 16 cut in two, 47 k-steps: 23 + 24
+    (torch.float8_e4m3fn, 4352, 4352, 6784),   # 33 tiles cut in three, 53 k-steps: 17 + 18 + 18
 ])
 def test_tail_split(abi, dt, M, N, K):
     """More tiles than workgroup slots with a last round at most half full: the tiles of that round
     are cut along K.  Checked against the oracle, element by element against the one-thread-per-
     output kernel, for determinism, and without a workspace (the split is then skipped)."""
     assert abi.mi355_gemm_workspace_bytes(M, N, K, ac.torch_code(dt), ac.BASIC) > 0
+    plan = ac.plan(abi, M, N, K, ac.torch_code(dt), ac.BASIC)
+    assert plan[1:4] == (256, 256, 1) and plan[4] > 0 and plan[5] > 1, plan
     A = rand((M, K), M, torch.float32).clamp_(-50, 50).to(dt)
     B = rand((N, K), N, torch.float32).clamp_(-50, 50).to(dt)
     scale = 2.0 ** -4
