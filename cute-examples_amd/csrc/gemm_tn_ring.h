@@ -141,14 +141,20 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   const uint32_t total_tiles = tiles_m * tiles_n;  // the launcher keeps items below 2^31
   // Work items are (tile, split) pairs, split-major, so that workgroups running together read the
   // same range of K.  With a uniform K split every tile has g.splits items; with a tail split only
-  // the last g.tail_tiles tiles are cut (g.tail_splits ways, into ranges of k-steps that differ by
-  // at most one when the k-steps do not divide) and come after all whole tiles.
+  // the last g.tail_tiles tiles are cut (g.tail_splits ways) and come after all whole tiles.  Either
+  // way a tile is cut into ranges of k-steps that differ by at most one when the k-steps do not divide.
   // steps is the number of k-steps of the current item.
   const uint32_t tail_tiles = (uint32_t)g.tail_tiles, tail_splits = (uint32_t)g.tail_splits;
   const uint32_t whole_tiles = total_tiles - tail_tiles;  // tail_tiles == 0 unless g.splits == 1
   const uint32_t total_items = tail_tiles ? whole_tiles + tail_tiles * tail_splits : total_tiles * (uint32_t)g.splits;
-  const uint32_t steps_split = __builtin_amdgcn_readfirstlane(k_steps / (uint32_t)g.splits);  // uniform split: divides
   uint32_t steps = 0;
+  // k-steps [sp*k/S, (sp+1)*k/S) of split sp of S: every step once, lengths within one of each other
+  auto cut = [&](uint32_t sp, uint32_t of, uint32_t* first_step) __attribute__((always_inline)) {
+    const uint32_t begin = __builtin_amdgcn_readfirstlane(sp * k_steps / of);
+    const uint32_t end = __builtin_amdgcn_readfirstlane((sp + 1) * k_steps / of);
+    *first_step = begin;
+    steps = end - begin;
+  };
   // item -> (tile number in tile-map order, split, first k-step, whether it writes fp32 partials);
   // sets steps.
   auto decode_item = [&](uint32_t it, uint32_t* tile, uint32_t* split_of, uint32_t* first_step)
@@ -165,17 +171,12 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
       const uint32_t sp = j / tail_tiles;
       *tile = whole_tiles + j % tail_tiles;
       *split_of = sp;
-      // k-steps [sp*k/S, (sp+1)*k/S): every step once, lengths within one of each other
-      const uint32_t begin = __builtin_amdgcn_readfirstlane(sp * k_steps / tail_splits);
-      const uint32_t end = __builtin_amdgcn_readfirstlane((sp + 1) * k_steps / tail_splits);
-      *first_step = begin;
-      steps = end - begin;
+      cut(sp, tail_splits, first_step);
       return true;
     }
     *tile = it % total_tiles;
     *split_of = it / total_tiles;
-    steps = steps_split;
-    *first_step = __builtin_amdgcn_readfirstlane(*split_of * steps_split);
+    cut(*split_of, (uint32_t)g.splits, first_step);
     return g.splits > 1;
   };
 

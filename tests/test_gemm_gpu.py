@@ -337,14 +337,42 @@ def test_tail_split(abi, dt, M, N, K):
     assert 0.5 < same < 1.0 or dt == torch.float8_e4m3fn, same
 
 
+@pytest.mark.parametrize("dt,M,N,K,tile,splits", [
+    (torch.bfloat16, 512, 6144, 5696, (256, 256), 5),        # 48 tiles, 89 k-steps: 17 + 18 + 18 + 18 + 18
+    (torch.bfloat16, 500, 6100, 5648, (256, 256), 5),        # the same with ragged rows, columns and last k-step
+    (torch.float8_e4m3fn, 256, 4096, 13568, (128, 128), 4),  # 64 small tiles, 106 k-steps cut in four
+    (torch.float16, 200, 2048, 4160, (128, 128), 4),         # 32 small tiles, 65 k-steps: 16 + 16 + 16 + 17
+])
+def test_k_split_that_does_not_divide_the_k_steps(abi, dt, M, N, K, tile, splits):
+    """A K split cuts a tile's k-steps into ranges whose lengths differ by one when they do not divide:
+    every k-step must be used exactly once.  Oracle, element-by-element comparison with the
+    one-thread-per-output kernel, determinism."""
+    plan = ac.plan(abi, M, N, K, ac.torch_code(dt), ac.BASIC)
+    assert plan[1:4] == tile + (splits,), plan
+    assert (-(-K * (1 if dt == torch.float8_e4m3fn else 2) // 128)) % splits != 0
+    A = rand((M, K), M, torch.float32).clamp_(-50, 50).to(dt)
+    B = rand((N, K), N, torch.float32).clamp_(-50, 50).to(dt)
+    scale = 2.0 ** -4
+    C = run_abi(abi, A, B, ac.BASIC, scale)
+    check(C, A, B, scale)
+    S = torch.empty((M, N), dtype=out_dtype_of(dt), device="cuda")
+    assert ac.gemm_tn(abi, A.cuda(), B.cuda(), S, scale, ac.SIMPLE) == 0
+    torch.cuda.synchronize()
+    d = (C.float() - S.cpu().float()).abs()
+    bad = d > 2e-2 * S.cpu().float().abs() + 2e-2 * (K ** 0.5) * scale
+    assert int(bad.sum()) == 0, (int(bad.sum()), float(d.max()))
+    assert torch.equal(run_abi(abi, A, B, ac.BASIC, scale).view(torch.int16), C.view(torch.int16))
+
+
 @pytest.mark.parametrize("dt,M,N,K", [
     (torch.bfloat16, 512, 14336, 4096),        # 2 x 112 tiles
-    (torch.bfloat16, 500, 14000, 4104),        # ragged rows, columns and last k-step
+    (torch.bfloat16, 500, 14000, 1960),        # ragged rows, columns and last k-step
+    (torch.bfloat16, 250, 6100, 4104),         # ragged, 48 tiles, 65 k-steps cut in four: 16 + 16 + 16 + 17
     (torch.float16, 256, 4096, 14336),         # 32 tiles, K split 8 ways
     (torch.float8_e4m3fn, 1024, 6144, 4096),
     (torch.float8_e4m3fn, 1000, 6100, 4112),   # ragged; 4112 fp8 bytes = 32 k-steps + 16 bytes
     (torch.float8_e4m3fn, 256, 4096, 14336),   # K split 7 ways
-    (torch.bfloat16, 768, 768, 8192),          # 3 x 6 tiles, K split 8 ways
+    (torch.bfloat16, 500, 2000, 8200),         # 2 x 16 tiles, 129 k-steps (the last ragged) cut in eight
 ])
 def test_rectangular_tile(abi, dt, M, N, K):
     """Problems the planner gives the 256x128 tile: against the oracle and, element by element,
