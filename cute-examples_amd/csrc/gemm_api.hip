@@ -83,6 +83,10 @@ int resolve(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t l
 struct Repack {
   bool a, b, c;
   int64_t Kp, Np;                 // padded K (elements) and N
+  int64_t ld_ab, ld_c;            // row strides (elements) of the repacked operands and of the padded C:
+                                  // multiples of 128 bytes, so that no 128-byte piece of a row straddles
+                                  // two cache lines (4096x4096x4104 bf16: 123 us with 8208-byte rows, 98 us
+                                  // with 8320-byte rows)
   size_t bytes_a, bytes_b, bytes_c;
 };
 
@@ -100,11 +104,13 @@ bool repack_plan(const void* A, const void* B, const void* C, int64_t M, int64_t
   r->b = r->Kp != K || (ldb * es) % 16 != 0 || (uintptr_t)B % 16 != 0 || r->Np != N;
   r->c = r->Np != N || ldc % 4 != 0 || (uintptr_t)C % 8 != 0;
   if (!r->a && !r->b && !r->c) return false;
-  r->bytes_a = r->a ? round_up((size_t)M * (size_t)r->Kp * (size_t)es, 256) : 0;
-  r->bytes_b = r->b ? round_up((size_t)r->Np * (size_t)r->Kp * (size_t)es, 256) : 0;
-  r->bytes_c = r->c ? round_up((size_t)M * (size_t)r->Np * 2, 256) : 0;
+  r->ld_ab = (int64_t)round_up((size_t)(r->Kp * es), 128) / es;
+  r->ld_c = (int64_t)round_up((size_t)r->Np, 64);
+  r->bytes_a = r->a ? round_up((size_t)M * (size_t)r->ld_ab * (size_t)es, 256) : 0;
+  r->bytes_b = r->b ? round_up((size_t)r->Np * (size_t)r->ld_ab * (size_t)es, 256) : 0;
+  r->bytes_c = r->c ? round_up((size_t)M * (size_t)r->ld_c * 2, 256) : 0;
   // the repacked problem must be one the tiled kernels take
-  return tile256_ok(M, r->Np, r->Kp, r->a ? r->Kp : lda, r->b ? r->Kp : ldb, r->c ? r->Np : ldc, in_dtype);
+  return tile256_ok(M, r->Np, r->Kp, r->a ? r->ld_ab : lda, r->b ? r->ld_ab : ldb, r->c ? r->ld_c : ldc, in_dtype);
 }
 
 }  // namespace
@@ -388,13 +394,13 @@ int mi355_gemm_tn_scaled(const void* A, const void* B, void* C, int64_t M, int64
       uint8_t* wc = wb + r.bytes_b;
       uint8_t* rest = wc + r.bytes_c;
       const size_t rest_bytes = workspace_bytes - (r.bytes_a + r.bytes_b + r.bytes_c);
-      if (r.a && mi355::launch_repack_rows(A, M, K * es, lda * es, wa, M, r.Kp * es, (int)es, s) != 0) return MI355_ERR_LAUNCH;
-      if (r.b && mi355::launch_repack_rows(B, N, K * es, ldb * es, wb, r.Np, r.Kp * es, (int)es, s) != 0) return MI355_ERR_LAUNCH;
-      st = mi355_gemm_tn_scaled(r.a ? wa : A, r.b ? wb : B, r.c ? (void*)wc : C, M, r.Np, r.Kp, r.a ? r.Kp : lda,
-                                r.b ? r.Kp : ldb, r.c ? r.Np : ldc, in_dtype, out_dtype, scale, scale_a, scale_b,
+      if (r.a && mi355::launch_repack_rows(A, M, K * es, lda * es, wa, M, r.ld_ab * es, (int)es, s) != 0) return MI355_ERR_LAUNCH;
+      if (r.b && mi355::launch_repack_rows(B, N, K * es, ldb * es, wb, r.Np, r.ld_ab * es, (int)es, s) != 0) return MI355_ERR_LAUNCH;
+      st = mi355_gemm_tn_scaled(r.a ? wa : A, r.b ? wb : B, r.c ? (void*)wc : C, M, r.Np, r.Kp, r.a ? r.ld_ab : lda,
+                                r.b ? r.ld_ab : ldb, r.c ? r.ld_c : ldc, in_dtype, out_dtype, scale, scale_a, scale_b,
                                 MI355_VARIANT_AUTO, rest_bytes ? rest : nullptr, rest_bytes, stream);
       if (st != MI355_OK) return st;
-      if (r.c && mi355::launch_copy_out(wc, M, N, r.Np, C, ldc, s) != 0) return MI355_ERR_LAUNCH;
+      if (r.c && mi355::launch_copy_out(wc, M, N, r.ld_c, C, ldc, s) != 0) return MI355_ERR_LAUNCH;
       return MI355_OK;
     }
   }

@@ -195,11 +195,12 @@ def test_workspace_for_repacking_misaligned_problems(abi):
     and explicit variants get nothing."""
     f = abi.mi355_gemm_workspace_bytes
     r256 = lambda x: -(-x // 256) * 256
-    # N % 4 != 0: B gets 3 zero rows, C a padded copy; A stays where it is
-    assert f(1000, 50257, 768, ac.BF16, ac.AUTO) == r256(50260 * 768 * 2) + r256(1000 * 50260 * 2) + \
+    # N % 4 != 0: B gets 3 zero rows, C a padded copy with rows of a multiple of 64 elements; A stays where it is
+    assert f(1000, 50257, 768, ac.BF16, ac.AUTO) == r256(50260 * 768 * 2) + r256(1000 * 50304 * 2) + \
         f(1000, 50260, 768, ac.BF16, ac.AUTO)
-    # K*2 % 16 != 0: A and B repacked to K = 1008, N = 1003 -> 1004
-    assert f(1001, 1003, 1001, ac.BF16, ac.AUTO) == r256(1001 * 1008 * 2) + r256(1004 * 1008 * 2) + r256(1001 * 1004 * 2) + \
+    # K*2 % 16 != 0: A and B repacked to K = 1008 in rows of 1024 elements (a multiple of 128 bytes),
+    # N = 1003 -> 1004 in rows of 1024
+    assert f(1001, 1003, 1001, ac.BF16, ac.AUTO) == r256(1001 * 1024 * 2) + r256(1004 * 1024 * 2) + r256(1001 * 1024 * 2) + \
         f(1001, 1004, 1008, ac.BF16, ac.AUTO)
     assert f(100, 30, 77, ac.BF16, ac.AUTO) == 0                   # too small to bother
     assert f(1001, 1003, 1001, ac.BF16, ac.SIMPLE) == 0
