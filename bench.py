@@ -28,7 +28,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs of this script
 # (FETCH_SIZE, then WRITE_SIZE, each with --copy-calibration and scaled by what the same counter
 # reads for the 1 GiB copy: x2.000 and x1.000).  Workloads without a counter run report null.
-MEASURED_TRAFFIC_BYTES = {"bf16_8192": 1.793e9, "fp8_8192": 0.963e9, "mxfp8_8192": 0.965e9, "skinny_16_14336_4096": 1.265e8}
+MEASURED_TRAFFIC_BYTES = {"bf16_8192": 1.793e9, "fp8_8192": 0.963e9, "mxfp8_8192": 0.965e9, "skinny_16_14336_4096": 1.190e8}
 
 
 def parse():

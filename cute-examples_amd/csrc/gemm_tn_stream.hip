@@ -4,7 +4,8 @@
 // kernel is built around keeping many bytes of W in flight per CU rather than around MFMA issue:
 //
 //   * output tile TM x 64 with TM = 16/32/64/128/256 >= M; the grid is (N/64 tiles) x (K splits),
-//     several workgroups resident per CU (the LDS ring of one workgroup is 30-120 KiB);
+//     several workgroups resident per CU (the LDS ring of one workgroup is 30-120 KiB), or, when
+//     the tiles alone occupy most CUs, no K split and a deeper ring (see unsplit_deep);
 //   * per k-step (128 B of K per row) the TM rows of X and 64 rows of W go global -> LDS with
 //     full-cache-line direct-to-LDS loads into a ring of kDepth stages, kDepth-1 k-steps ahead;
 //   * the four waves read MFMA fragments from LDS (same 16-byte-chunk swizzle as the big-tile
@@ -203,9 +204,29 @@ int launch_cfg(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
 // Ring depth (k-steps) per tile height.  Depths 3..6 measured the same on the LLM projection
 // shapes; the shallow ones leave room for 3-4 workgroups per CU.
 constexpr int kDepth16 = 4, kDepth32 = 4, kDepth64 = 3, kDepth128 = 4, kDepth256 = 3;
+// Without a K split (enough tiles to give nearly every CU one) a workgroup has the CU to itself and
+// keeps its bytes in flight with a deep ring instead of with neighbours: 16x14336x4096 bf16
+// 27.7 us split four ways + reduce, 25.7 us unsplit with eight stages (27.1 us with fourteen).
+constexpr int kDepthUnsplit = 8;
+// That mode pays when the tiles occupy most of the 256 CUs and all of them are resident at once
+// with the deep ring (two workgroups per CU at M <= 16, one above): measured on N = 12800...28672,
+// bf16 and fp8, -7 to -20 % there; with more tiles than that (several rounds) the shallow ring with
+// three or four workgroups per CU is 5-20 % faster again.
+bool unsplit_deep(int64_t M, int64_t N) {
+  if (M > 64) return false;
+  const int64_t tm = M <= 16 ? 16 : M <= 32 ? 32 : 64;
+  const int64_t per_cu = 163840 / (kDepthUnsplit * (tm + kTileN) * kRowBytes);
+  const int64_t tiles = (N + kTileN - 1) / kTileN;
+  return tiles >= 200 && tiles <= 256 * per_cu;
+}
 
 template <class T, class OutT>
 int launch_m(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
+  if (splits == 1 && unsplit_deep(g.M, g.N)) {
+    if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
+    if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
+    return launch_cfg<T, OutT, 4, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
+  }
   if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, kDepth16>(g, splits, ws, stream);   //  16x64, 10 KiB/step
   if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, kDepth32>(g, splits, ws, stream);   //  32x64, 12 KiB/step
   if (g.M <= 64) return launch_cfg<T, OutT, 4, 1, 1, 4, kDepth64>(g, splits, ws, stream);   //  64x64, 16 KiB/step
@@ -225,6 +246,7 @@ int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
   const int64_t slots = 256 * per_cu;  // MI355X has 256 CUs; a heuristic only, so no device query here
   const int64_t tiles = ((M + tm - 1) / tm) * ((N + kTileN - 1) / kTileN);
   const int64_t steps = (K * elem_bytes + kRowBytes - 1) / kRowBytes;
+  if (unsplit_deep(M, N)) return 1;
   int best = 1;
   for (int s = 1; s <= 32; ++s) {
     if (tiles * s > slots) break;

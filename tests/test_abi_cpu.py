@@ -176,8 +176,12 @@ def test_plan(abi):
     assert ac.plan(abi, 512, 14336, 4096, ac.BF16) == (ac.BASIC, 256, 128, 1, 0, 1)         # 224 rectangular tiles
     assert ac.plan(abi, 2048, 2048, 2048, ac.F16) == (ac.BASIC, 128, 128, 1, 0, 1)          # 256 small tiles
     assert ac.plan(abi, 512, 6144, 4096, ac.BF16) == (ac.BASIC, 256, 256, 4, 0, 1)          # 48 tiles cut in four
-    v, rows, cols, splits, _, _ = ac.plan(abi, 16, 14336, 4096, ac.BF16)
+    v, rows, cols, splits, _, _ = ac.plan(abi, 16, 6144, 4096, ac.BF16)
     assert (v, rows, cols) == (ac.SKINNY, 16, 64) and splits >= 2
+    # 224 tiles of 64 columns: (nearly) one per CU, so no K split (the kernel then runs a deeper ring)
+    assert ac.plan(abi, 16, 14336, 4096, ac.BF16) == (ac.SKINNY, 16, 64, 1, 0, 1)
+    assert ac.plan(abi, 64, 14336, 4096, ac.E4M3) == (ac.SKINNY, 64, 64, 1, 0, 1)
+    assert ac.plan(abi, 16, 28672, 4096, ac.BF16)[3] == 1        # 448 tiles: two per CU at this height
     assert ac.plan(abi, 100, 30, 77, ac.BF16)[0] == ac.SIMPLE
     assert ac.plan(abi, 256, 256, 68, ac.BF16, ac.BASIC)[0] == ac.ERR_SHAPE
     assert ac.plan(abi, 256, 256, 64, 7)[0] == ac.ERR_DTYPE
