@@ -63,12 +63,13 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
 
   const uint32_t ldx_b = (uint32_t)(g.lda * T::kBytes), ldw_b = (uint32_t)(g.ldb * T::kBytes);
   const uint32_t k_bytes = (uint32_t)(g.K * T::kBytes);
-  // The host only splits K when the k-steps divide evenly; a ragged last k-step (K*elem_bytes not
-  // a multiple of 128) is handled by fetching its missing chunks from an out-of-range offset.
+  // Split `split` of S takes k-steps [split*k/S, (split+1)*k/S): every step once, lengths within one
+  // of each other when S does not divide them.  A ragged last k-step (K*elem_bytes not a multiple
+  // of 128) is handled by fetching its missing chunks from an out-of-range offset.
   const uint32_t steps_total = (k_bytes + kRowBytes - 1) / kRowBytes;
   const uint32_t tail_bytes = __builtin_amdgcn_readfirstlane(k_bytes % kRowBytes);
-  const uint32_t steps = __builtin_amdgcn_readfirstlane(steps_total / (uint32_t)splits);
-  const uint32_t step0 = __builtin_amdgcn_readfirstlane(split * steps);
+  const uint32_t step0 = __builtin_amdgcn_readfirstlane(split * steps_total / (uint32_t)splits);
+  const uint32_t steps = __builtin_amdgcn_readfirstlane((split + 1) * steps_total / (uint32_t)splits) - step0;
   const int64_t rows_x = g.M - m0 < kTm ? g.M - m0 : kTm;
   const int64_t rows_w = g.N - n0 < kTn ? g.N - n0 : kTn;
   const __amdgpu_buffer_rsrc_t rsrc_x = make_raw_buffer(
@@ -82,8 +83,16 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
   // the descriptor's range and read as zeros.
   const uint32_t r8 = lane >> 3, c8 = lane & 7u;
   const uint32_t ring0 = __builtin_amdgcn_readfirstlane(lds_address(ring));
+  // Workgroups that run side by side walk their k-steps from different starting points (and wrap
+  // around): started together at the same k they would all be reading the same 128-byte column of
+  // rows that lie a power of two apart when K is one, i.e. the same few memory channels (fp8
+  // 16x8192x8192 cut in two: 19.6 us, against 16.2 us for K = 8320).  Only the order of the fp32
+  // additions inside a tile depends on it, and that order is fixed per tile.
+  const uint32_t rot = __builtin_amdgcn_readfirstlane((blockIdx.x * 7u + blockIdx.y * 3u) % steps);
   auto issue_step = [&](uint32_t stage, uint32_t kt) __attribute__((always_inline)) {
-    const uint32_t kk = kt < steps ? step0 + kt : step0 + steps - 1;
+    uint32_t at = (kt < steps ? kt : steps - 1) + rot;   // steps past the end repeat the last one
+    at = at >= steps ? at - steps : at;
+    const uint32_t kk = step0 + at;
     const uint32_t soff = kk * kRowBytes;
     const bool ragged = tail_bytes != 0 && kk == steps_total - 1;
 #pragma unroll
@@ -237,7 +246,7 @@ int launch_m(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
 }  // namespace
 
 // K splits for a skinny problem: as many workgroups as can be resident at once (one wave of
-// workgroups, no tail), each with enough k-steps, and the k-steps must divide evenly.
+// workgroups, no tail), each with enough k-steps.
 int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
   const int64_t tm = M <= 16 ? 16 : M <= 32 ? 32 : M <= 64 ? 64 : M <= 128 ? 128 : 256;
   const int depth = M <= 16 ? 4 : M <= 32 ? 4 : M <= 64 ? 3 : M <= 128 ? 4 : 3;  // kDepth16 .. kDepth256
@@ -247,15 +256,22 @@ int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
   const int64_t tiles = ((M + tm - 1) / tm) * ((N + kTileN - 1) / kTileN);
   const int64_t steps = (K * elem_bytes + kRowBytes - 1) / kRowBytes;
   if (unsplit_deep(M, N)) return 1;
-  // At least 16 k-steps per workgroup (filling and draining the ring costs about four), fewer, down
-  // to 8, only while the workgroups do not yet cover the 256 CUs.  (With 8 everywhere, 36 bf16 and
-  // fp8 problems with N = 2048...11008 measured 5 % slower on average, up to 21 %.)
+  // The workgroups of a CU share its bandwidth, and one of them already keeps it busy, so what counts
+  // is the CU with the most k-steps to stream: ceil(workgroups / 256) workgroups of ceil(steps / S)
+  // k-steps, each paying about four more to fill and drain its ring; splits beyond that only add
+  // partial tiles.  Measured on 18 bf16 problems (M = 16 and 64, N = 2048...11008) with every S
+  // forced: the choice is within 1 % of the best S on average (a rule that maximised the number
+  // of workgroups: 10 %).  At least 8 k-steps per workgroup.
   int best = 1;
+  double best_cost = 0;
   for (int s = 1; s <= 32; ++s) {
     if (tiles * s > slots) break;
-    if (steps % s != 0) continue;
-    const int64_t per_item = steps / s;
-    if (per_item >= 16 || (per_item >= 8 && tiles * best < 256)) best = s;
+    if (s > 1 && steps / s < 8) break;
+    const double cost = (double)((tiles * s + 255) / 256) * (double)((steps + s - 1) / s + 4) + 0.5 * s;
+    if (s == 1 || cost < best_cost) {
+      best = s;
+      best_cost = cost;
+    }
   }
   return best;
 }

@@ -296,7 +296,7 @@ def test_plan_invariants_over_random_shapes(abi):
             tiles = -(-M // rows) * -(-N // cols)
             assert splits >= 1 and tail_splits >= 1 and tail_tiles >= 0
             if splits > 1:
-                assert tail_tiles == 0 and (v == ac.BASIC or steps % splits == 0), (M, N, K, splits)   # the tiled kernel cuts unevenly
+                assert tail_tiles == 0, (M, N, K, splits)      # the k-steps need not divide: cuts differ by one k-step
                 assert steps // splits >= (16 if v == ac.BASIC else 8), (M, N, K, splits)
             want = splits * M * N * 4 if splits > 1 else 0
             if v == ac.BASIC:

@@ -641,6 +641,21 @@ def test_skinny_kernel_every_tile_height_and_split(abi, dt, M, N, K):
     assert oracle.rel_frobenius(C, oracle.c_gemm_tn_f32(A, B, 0.25)) <= TOL[dt]
 
 
+@pytest.mark.parametrize("dt,M,N,K", [(torch.bfloat16, 16, 4096, 5696), (torch.bfloat16, 48, 4100, 11016),
+                                      (torch.float8_e4m3fn, 64, 2048, 13584), (torch.float16, 200, 1024, 5768)])
+def test_skinny_k_split_that_does_not_divide_the_k_steps(abi, dt, M, N, K):
+    """89, 173 (the last ragged), 107 and 91 k-steps with split counts that do not divide them."""
+    es = 1 if dt == torch.float8_e4m3fn else 2
+    splits = ac.plan(abi, M, N, K, ac.torch_code(dt), ac.SKINNY)[3]
+    assert splits > 1 and (-(-K * es // 128)) % splits != 0, splits
+    A = rand((M, K), M, torch.float32).clamp_(-50, 50).to(dt)
+    B = rand((N, K), N, torch.float32).clamp_(-50, 50).to(dt)
+    C = run_abi(abi, A, B, ac.SKINNY, 0.25)
+    check(C, A, B, 0.25)
+    assert oracle.rel_frobenius(C, oracle.c_gemm_tn_f32(A, B, 0.25)) <= TOL[dt]
+    assert torch.equal(run_abi(abi, A, B, ac.SKINNY, 0.25).view(torch.int16), C.view(torch.int16))
+
+
 def test_skinny_split_k_is_deterministic_and_needs_its_workspace(abi):
     M, N, K = 16, 256, 4096
     A, B = rand((M, K), 1, torch.bfloat16).cuda(), rand((N, K), 2, torch.bfloat16).cuda()
