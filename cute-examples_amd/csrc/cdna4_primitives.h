@@ -52,6 +52,18 @@ __device__ __forceinline__ void dma_16B_to_lds(uint32_t lds_base, uint32_t voffs
       : "memory");
 }
 
+// The same with 4 bytes per lane: lane l's dword lands at LDS byte address lds_base + 4*l.
+__device__ __forceinline__ void dma_4B_to_lds(uint32_t lds_base, uint32_t voffset,
+                                              __amdgpu_buffer_rsrc_t rsrc, uint32_t soffset) {
+  asm volatile(
+      "s_mov_b32 m0, %0\n\t"
+      "buffer_load_dword %1, %2, %3 offen lds"
+      :
+      : "s"(__builtin_amdgcn_readfirstlane(lds_base)), "v"(voffset), "s"(rsrc),
+        "s"(__builtin_amdgcn_readfirstlane(soffset))
+      : "memory");
+}
+
 // The same copy with the LDS base given as a scalar register plus a compile-time constant, folded
 // into the one instruction that writes M0 (it also writes SCC).
 template <uint32_t kLdsAdd>

@@ -264,6 +264,12 @@ int mi355_gemm_mx_check(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ld
 
 namespace {
 // Partial results of the block-scaled GEMM's K split or tail split (the planner's, as for plain fp8).
+// Whether a block-scaled problem goes to the streaming kernel, and with how many K splits.
+int mx_stream_splits(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc) {
+  if (M > kSkinnyAutoMaxM || !skinny_ok(M, N, K, lda, ldb, ldc, MI355_E4M3)) return 0;
+  return mi355::stream_splits(M, N, K, 1);
+}
+
 size_t mx_partial_bytes(int64_t M, int64_t N, int64_t K, int* splits, int* tail_tiles, int* tail_splits) {
   int s = mi355::ring_splits(M, N, K, 1), tt = 0, ts = 1;
   size_t bytes = s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : mi355::ring_tail(M, N, K, 1, &tt, &ts);
@@ -276,8 +282,10 @@ size_t mx_partial_bytes(int64_t M, int64_t N, int64_t K, int* splits, int* tail_
 
 size_t mi355_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int scales_shuffled) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0 || !extents_ok(M, N, K, K, K, N)) return 0;
-  return mx_partial_bytes(M, N, K, nullptr, nullptr, nullptr) +
-         (scales_shuffled ? 0 : mi355::mx_shuffled_bytes(M, K) + mi355::mx_shuffled_bytes(N, K));
+  const int ss = mx_stream_splits(M, N, K, K, K, N);
+  const size_t partial = ss ? (ss > 1 ? (size_t)ss * (size_t)M * (size_t)N * sizeof(float) : 0)
+                            : mx_partial_bytes(M, N, K, nullptr, nullptr, nullptr);
+  return partial + (scales_shuffled ? 0 : mi355::mx_shuffled_bytes(M, K) + mi355::mx_shuffled_bytes(N, K));
 }
 
 int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, int64_t N, int64_t K, int64_t lda,
@@ -322,6 +330,15 @@ int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, in
     g.mx_a = wa;
     g.mx_b = wb;
     used = bytes_a + bytes_b;
+  }
+  // A few rows of activations: stream the weights, as for plain fp8 (when the workspace holds the
+  // partial results of its K split, if it has one; otherwise the tile kernel below takes it).
+  if (const int ss = mx_stream_splits(M, N, K, lda, ldb, ldc)) {
+    const size_t need = ss > 1 ? (size_t)ss * (size_t)M * (size_t)N * sizeof(float) : 0;
+    if (!need || (workspace && (uintptr_t)workspace % 16 == 0 && workspace_bytes >= used + need)) {
+      g.tiles_m = g.tiles_n = 0;
+      return mi355::launch_stream_mx(g, out_dtype, ss, (uint8_t*)workspace + used, s) == 0 ? MI355_OK : MI355_ERR_LAUNCH;
+    }
   }
   // K split or tail split when the rest of the workspace holds the partial results (optional, as
   // for the other tiled kernels: without it the tiles run unsplit).

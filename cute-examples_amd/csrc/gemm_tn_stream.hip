@@ -34,6 +34,15 @@ constexpr int kTileN = 64;
 // Geometry per input type: 16x16 blocks for all of them (fp8 on the 16x16x128 shape).
 template <class T> struct StreamGeo { typedef Geo<T> type; };
 template <> struct StreamGeo<E4M3> { typedef GeoE4M3Rows type; };
+template <> struct StreamGeo<MxE4M3> { typedef GeoMxE4M3Rows type; };
+
+// Block scales (MxE4M3) come in the layout the tile kernel reads too (mx_scales.hip): one 512-byte
+// unit per (group of 128 rows, k-step), in which lane l owns the 8 bytes at 8*l: byte i is the scale
+// of row 16*i + l%16 for K block 4*kstep + l/16, i.e. exactly what lane l of the scaled MFMA has
+// to supply for the i-th 16-row block.  A 64-row tile is one half of a group, so one 4-byte copy
+// per lane and k-step brings the scales of all four blocks of W, and another those of X; they
+// travel through the ring like the operands (256 bytes each behind the rows of a stage).
+constexpr uint32_t kMxUnit = 512;
 
 template <class T, class OutT, int kMB, int kNB, int kWM, int kWN, int kDepth>
 __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* partial, int splits) {
@@ -44,11 +53,15 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
   constexpr int kSlices = 8 / kSliceChunks;            // MFMAs per k-step and block pair
   constexpr int kTm = 16 * kMB * kWM, kTn = 16 * kNB * kWN;
   static_assert(kTn == kTileN, "grid assumes 64-row W tiles");
-  constexpr int kStageBytes = (kTm + kTn) * kRowBytes;
+  constexpr bool kMx = G::kMx;
+  static_assert(!kMx || (kWM == 1 && kWN == 4 && kNB == 1), "block scales: one 64-row half group per operand");
+  constexpr int kDataBytes = (kTm + kTn) * kRowBytes;
+  constexpr int kStageBytes = kDataBytes + (kMx ? 512 : 0);   // + the scales of W, then of X
   constexpr int kCopies = (kTm + kTn) / 8;          // 8-row copies per k-step
   constexpr int kCpw = (kCopies + 3) / 4;           // per wave (padded with repeats)
   constexpr int kXCopies = kTm / 8;
-  static_assert(kCpw * (kDepth - 1) < 64, "vmcnt is a 6-bit counter");
+  constexpr int kVm = kCpw + (kMx ? 1 : 0);         // vector-memory instructions per wave and k-step
+  static_assert(kVm * (kDepth - 1) < 64, "vmcnt is a 6-bit counter");
   __shared__ __attribute__((aligned(1024))) uint8_t ring[kDepth * kStageBytes];
 
   const uint32_t tid = threadIdx.x;
@@ -76,6 +89,15 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
       (const uint8_t*)g.A + m0 * (int64_t)ldx_b, (uint32_t)((rows_x - 1) * ldx_b + k_bytes));
   const __amdgpu_buffer_rsrc_t rsrc_w = make_raw_buffer(
       (const uint8_t*)g.B + n0 * (int64_t)ldw_b, (uint32_t)((rows_w - 1) * ldw_b + k_bytes));
+
+  // Scales: even waves copy those of W, odd waves those of X (twice each, so that every wave
+  // issues the same number of instructions).
+  const uint32_t scale_units = kMx ? (uint32_t)((g.M + 255) / 256) * 2u * steps_total * kMxUnit : 0u;
+  const uint32_t scale_units_w = kMx ? (uint32_t)((g.N + 255) / 256) * 2u * steps_total * kMxUnit : 0u;
+  const __amdgpu_buffer_rsrc_t rsrc_sx = make_raw_buffer(g.mx_a, scale_units);
+  const __amdgpu_buffer_rsrc_t rsrc_sw = make_raw_buffer(g.mx_b, scale_units_w);
+  const uint32_t voff_sx = (uint32_t)(m0 / 128) * steps_total * kMxUnit + lane * 8 + (uint32_t)(m0 % 128) / 64 * 4;
+  const uint32_t voff_sw = (uint32_t)(n0 / 128) * steps_total * kMxUnit + lane * 8 + (uint32_t)(n0 % 128) / 64 * 4;
 
   // Copy c (0..kCopies-1) of a k-step moves 8 rows x 128 B: X rows first, then W rows; wave w
   // issues copies w, w+4, ...  (indices past the end repeat earlier copies so that every wave
@@ -105,6 +127,11 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
       if (c < kXCopies) dma_16B_to_lds(dst, (row * ldx_b + chunk * 16) | drop, rsrc_x, soff);   // c is wave-uniform
       else dma_16B_to_lds(dst, ((row - kTm) * ldw_b + chunk * 16) | drop, rsrc_w, soff);
     }
+    if constexpr (kMx) {
+      const uint32_t dst = ring0 + stage * kStageBytes + kDataBytes;
+      if ((wave & 1u) == 0) dma_4B_to_lds(dst, voff_sw, rsrc_sw, kk * kMxUnit);
+      else dma_4B_to_lds(dst + 256, voff_sx, rsrc_sx, kk * kMxUnit);
+    }
   };
 
   // Fragment geometry: lane l supplies row l%16 of a block, lane group l/16 picks the chunk.
@@ -116,6 +143,11 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
     const uint8_t* p = rows + blk * 16 * kRowBytes;
     if constexpr (G::kCpl == 1) {
       return *(const i32x4*)(p + (((uint32_t)(s * kSliceChunks) + grp) ^ swz) * 16);
+    } else if constexpr (kMx) {
+      // the order of K inside the scaled MFMA matters: lane group g supplies chunks g and 4+g
+      const i32x4 lo = *(const i32x4*)(p + ((grp ^ swz) * 16));
+      const i32x4 hi = *(const i32x4*)(p + (((grp + 4) ^ swz) * 16));
+      return (i32x8){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     } else {
       const i32x4 lo = *(const i32x4*)(p + (((uint32_t)(s * kSliceChunks) + grp * 2) ^ swz) * 16);
       const i32x4 hi = *(const i32x4*)(p + (((uint32_t)(s * kSliceChunks) + grp * 2 + 1) ^ swz) * 16);
@@ -134,7 +166,7 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
 
   uint32_t stage = 0;
   for (uint32_t kt = 0; kt < steps; ++kt) {
-    wait_vmcnt<kCpw * (kDepth - 2)>();  // my copies of k-step kt have landed
+    wait_vmcnt<kVm * (kDepth - 2)>();   // my copies of k-step kt have landed
     wait_lgkmcnt0();                    // my LDS reads of k-step kt-1 are back
     __builtin_amdgcn_s_barrier();       // everybody's are: stage of kt is full, stage of kt-1 is free
     const uint32_t refill = stage == 0 ? kDepth - 1 : stage - 1;
@@ -147,14 +179,26 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
       for (int j = 0; j < kNB; ++j) fw[j] = frag(st_base + w_lane, j, s);
 #pragma unroll
       for (int i = 0; i < kMB; ++i) fx[i] = frag(st_base + x_lane, i, s);
+      if constexpr (kMx) {
+        // this lane's four scale bytes of W (block wn is this wave's) and of X (block i)
+        const uint32_t sw = *(const uint32_t*)(st_base + kDataBytes + lane * 4) >> (wn * 8);
+        const uint32_t sx = *(const uint32_t*)(st_base + kDataBytes + 256 + lane * 4);
+        static_for<kMB>([&](auto ic) __attribute__((always_inline)) {
+          constexpr int i = decltype(ic)::value;
+          G::template mfma_scaled_inplace<0, i>(fw[0], fx[i], acc[i][0], sw, sx);
+        });
+      } else {
 #pragma unroll
-      for (int i = 0; i < kMB; ++i)
+        for (int i = 0; i < kMB; ++i)
 #pragma unroll
-        for (int j = 0; j < kNB; ++j) acc[i][j] = G::mfma(fw[j], fx[i], acc[i][j]);
+          for (int j = 0; j < kNB; ++j) acc[i][j] = G::mfma(fw[j], fx[i], acc[i][j]);
+      }
     }
     stage = stage + 1 == kDepth ? 0 : stage + 1;
   }
   wait_vmcnt<0>();
+  // the scaled MFMAs are inline assembly: the compiler does not know how long their results take
+  if constexpr (kMx) asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
   // acc[i][j][r] of lane l is the (partial) sum for
   //   m = m0 + (wm*kMB + i)*16 + l%16,   n = n0 + (wn*kNB + j)*16 + 4*(l/16) + r.
@@ -239,8 +283,12 @@ int launch_m(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
   if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, kDepth16>(g, splits, ws, stream);   //  16x64, 10 KiB/step
   if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, kDepth32>(g, splits, ws, stream);   //  32x64, 12 KiB/step
   if (g.M <= 64) return launch_cfg<T, OutT, 4, 1, 1, 4, kDepth64>(g, splits, ws, stream);   //  64x64, 16 KiB/step
-  if (g.M <= 128) return launch_cfg<T, OutT, 4, 2, 2, 2, kDepth128>(g, splits, ws, stream);  // 128x64, 24 KiB/step
-  return launch_cfg<T, OutT, 4, 4, 4, 1, kDepth256>(g, splits, ws, stream);                  // 256x64, 40 KiB/step
+  if constexpr (std::is_same<T, MxE4M3>::value) {
+    return -1;   // block scales: up to 64 rows (the host routes taller problems to the tile kernel)
+  } else {
+    if (g.M <= 128) return launch_cfg<T, OutT, 4, 2, 2, 2, kDepth128>(g, splits, ws, stream);  // 128x64, 24 KiB/step
+    return launch_cfg<T, OutT, 4, 4, 4, 1, kDepth256>(g, splits, ws, stream);                  // 256x64, 40 KiB/step
+  }
 }
 
 }  // namespace
@@ -282,6 +330,13 @@ int launch_splitk_reduce(const float* partial, const GemmArgs& g, int out_dtype,
   if (out_dtype == 0) hipLaunchKernelGGL((splitk_reduce<BF16>), grid, dim3(256), 0, stream, partial, g);
   else hipLaunchKernelGGL((splitk_reduce<F16>), grid, dim3(256), 0, stream, partial, g);
   return hipGetLastError() == hipSuccess ? 0 : -1;
+}
+
+// Block-scaled fp8 (g.mx_a / g.mx_b in the shuffled layout), M <= 64.
+int launch_stream_mx(const GemmArgs& g, int out_dtype, int splits, void* workspace, hipStream_t stream) {
+  if (g.M > 64) return -1;
+  return out_dtype == 0 ? launch_m<MxE4M3, BF16>(g, splits, (float*)workspace, stream)
+                        : launch_m<MxE4M3, F16>(g, splits, (float*)workspace, stream);
 }
 
 int launch_stream(const GemmArgs& g, int in_dtype, int out_dtype, int splits, void* workspace, hipStream_t stream) {

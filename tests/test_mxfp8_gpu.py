@@ -336,3 +336,70 @@ def test_torch_op_quantisers_agree_with_the_kernels_on_the_device(dtype, std):
     q, s = gemm_kernels.quantize_e4m3(x)
     qt, st = quantize_e4m3_torch(x)
     assert float(s) == float(st) and same_codes(q, qt)
+
+
+# ---------------------------------------------------------------- a few rows of activations: the streaming kernel
+
+@pytest.mark.parametrize("shuffled", [False, True])
+@pytest.mark.parametrize("shape", [(1, 256, 128), (16, 14336, 4096), (17, 2052, 1024), (33, 6144, 4096), (64, 4096, 5760),
+                                   (48, 14340, 2048), (64, 28672, 1024), (7, 260, 14336)])
+def test_few_rows_stream_the_weights(abi, shape, shuffled):
+    """M <= 64 goes to the weight-streaming kernel: every tile height, with and without a K split (and
+    splits that do not divide the k-steps), ragged N, both scale layouts; deterministic."""
+    M, N, K = shape
+    A, sa = random_mx(M, K, 31, 120, 132)
+    B, sb = random_mx(N, K, 32, 120, 132)
+    C = run_mx(abi, A, sa, B, sb, shuffled=shuffled, ldc=N + 4)
+    err, _ = check(C, A, sa, B, sb)
+    assert err < 5e-3
+    assert torch.equal(run_mx(abi, A, sa, B, sb, shuffled=shuffled, ldc=N + 4).view(torch.int16), C.view(torch.int16))
+
+
+@pytest.mark.parametrize("M", [1, 16, 40, 64])
+def test_each_scale_byte_reaches_its_block_only_with_few_rows(abi, M):
+    """One doubled scale byte changes exactly its row (or column) by exactly +32, for rows in every
+    16-row block of the tile and columns in every block of every wave, across several k-steps and
+    K splits of the streaming kernel."""
+    N, K = 4096, 2048
+    ones_a = torch.ones(M, K).to(torch.float8_e4m3fn)
+    ones_b = torch.ones(N, K).to(torch.float8_e4m3fn)
+    base_a = torch.full((M, K // 32), 127, dtype=torch.uint8)
+    base_b = torch.full((N, K // 32), 127, dtype=torch.uint8)
+    rows = sorted({0, M // 3, M // 2, M - 1, min(M - 1, 15), min(M - 1, 16), min(M - 1, 47)})
+    sa = base_a.clone()
+    for i, r in enumerate(rows):
+        sa[r, (5 * i + 3) % (K // 32)] = 128
+    C = run_mx(abi, ones_a, sa, ones_b, base_b).float()
+    want = torch.full((M, N), float(K))
+    want[rows, :] += 32.0
+    assert torch.equal(C, want)
+    cols = [0, 15, 16, 31, 32, 47, 48, 63, 64, 100, 127, 128, 191, 255, 300, N - 65, N - 1]
+    sb = base_b.clone()
+    for i, c in enumerate(cols):
+        sb[c, (7 * i + 1) % (K // 32)] = 128
+    for shuffled in (False, True):
+        C = run_mx(abi, ones_a, base_a, ones_b, sb, shuffled=shuffled).float()
+        want = torch.full((M, N), float(K))
+        want[:, cols] += 32.0
+        assert torch.equal(C, want), shuffled
+
+
+def test_few_rows_without_room_for_the_k_split_fall_back_to_the_tile_kernel(abi):
+    """The streaming kernel needs the workspace of its K split; a call that brings only the room for
+    the shuffled scales still succeeds (on the tile kernel, whose split is optional)."""
+    M, N, K = 16, 4096, 14336
+    A, sa = random_mx(M, K, 41, 120, 132)
+    B, sb = random_mx(N, K, 42, 120, 132)
+    full = abi.mi355_gemm_mx_workspace_bytes(M, N, K, 0)
+    only_scales = abi.mi355_mx_shuffled_bytes(M, K) + abi.mi355_mx_shuffled_bytes(N, K)
+    assert full > only_scales
+    Ad, Bd, sad, sbd = A.cuda(), B.cuda(), sa.cuda(), sb.cuda()
+    ws = torch.empty(only_scales, dtype=torch.uint8, device="cuda")
+    C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    rc = abi.mi355_gemm_tn_mxfp8(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, K, N, sad.data_ptr(), K // 32,
+                                 sbd.data_ptr(), K // 32, 0, ac.BF16, ws.data_ptr(), only_scales,
+                                 torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    err, _ = check(C.cpu(), A, sa, B, sb)
+    assert err < 5e-3
