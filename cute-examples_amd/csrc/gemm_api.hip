@@ -267,7 +267,7 @@ namespace {
 // Whether a block-scaled problem goes to the streaming kernel, and with how many K splits.
 int mx_stream_splits(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc) {
   if (M > kSkinnyAutoMaxM || !skinny_ok(M, N, K, lda, ldb, ldc, MI355_E4M3)) return 0;
-  return mi355::stream_splits(M, N, K, 1);
+  return mi355::stream_splits(M, N, K, 1, true);
 }
 
 size_t mx_partial_bytes(int64_t M, int64_t N, int64_t K, int* splits, int* tail_tiles, int* tail_splits) {

@@ -265,17 +265,17 @@ constexpr int kDepthUnsplit = 8;
 // with the deep ring (two workgroups per CU at M <= 16, one above): measured on N = 12800...28672,
 // bf16 and fp8, -7 to -20 % there; with more tiles than that (several rounds) the shallow ring with
 // three or four workgroups per CU is 5-20 % faster again.
-bool unsplit_deep(int64_t M, int64_t N) {
+bool unsplit_deep(int64_t M, int64_t N, bool mx) {
   if (M > 64) return false;
   const int64_t tm = M <= 16 ? 16 : M <= 32 ? 32 : 64;
-  const int64_t per_cu = 163840 / (kDepthUnsplit * (tm + kTileN) * kRowBytes);
+  const int64_t per_cu = 163840 / (kDepthUnsplit * ((tm + kTileN) * kRowBytes + (mx ? 512 : 0)));
   const int64_t tiles = (N + kTileN - 1) / kTileN;
   return tiles >= 200 && tiles <= 256 * per_cu;
 }
 
 template <class T, class OutT>
 int launch_m(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
-  if (splits == 1 && unsplit_deep(g.M, g.N)) {
+  if (splits == 1 && unsplit_deep(g.M, g.N, std::is_same<T, MxE4M3>::value)) {
     if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
     if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
     return launch_cfg<T, OutT, 4, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
@@ -295,15 +295,15 @@ int launch_m(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
 
 // K splits for a skinny problem: as many workgroups as can be resident at once (one wave of
 // workgroups, no tail), each with enough k-steps.
-int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
+int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
   const int64_t tm = M <= 16 ? 16 : M <= 32 ? 32 : M <= 64 ? 64 : M <= 128 ? 128 : 256;
   const int depth = M <= 16 ? 4 : M <= 32 ? 4 : M <= 64 ? 3 : M <= 128 ? 4 : 3;  // kDepth16 .. kDepth256
-  const int64_t ring_bytes = depth * (tm + kTileN) * kRowBytes;
+  const int64_t ring_bytes = depth * ((tm + kTileN) * kRowBytes + (mx ? 512 : 0));
   const int64_t per_cu = 163840 / ring_bytes < 8 ? 163840 / ring_bytes : 8;   // LDS-bound residency
   const int64_t slots = 256 * per_cu;  // MI355X has 256 CUs; a heuristic only, so no device query here
   const int64_t tiles = ((M + tm - 1) / tm) * ((N + kTileN - 1) / kTileN);
   const int64_t steps = (K * elem_bytes + kRowBytes - 1) / kRowBytes;
-  if (unsplit_deep(M, N)) return 1;
+  if (unsplit_deep(M, N, mx)) return 1;
   // The workgroups of a CU share its bandwidth, and one of them already keeps it busy, so what counts
   // is the CU with the most k-steps to stream: ceil(workgroups / 256) workgroups of ceil(steps / S)
   // k-steps, each paying about four more to fill and drain its ring; splits beyond that only add
