@@ -65,9 +65,10 @@ enum mi355_status {
  *             (1.0f for bf16/fp16; scale_a*scale_b for per-tensor-scaled fp8)
  *   variant   enum mi355_variant
  *   workspace device scratch of at least mi355_gemm_workspace_bytes(...) bytes, or NULL when
- *             that function returns 0; contents need not be initialised.  The skinny variant
- *             needs it for its K split (MI355_ERR_WORKSPACE otherwise); the tiled variant runs
- *             without its K split or tail split, i.e. slower, when it is NULL or too small.
+ *             that function returns 0; contents need not be initialised.  An explicit skinny
+ *             variant needs it for its K split (MI355_ERR_WORKSPACE otherwise); the tiled variant
+ *             runs without its K split or tail split, i.e. slower, when it is NULL or too small,
+ *             and MI355_VARIANT_AUTO then uses the tiled variant also where it would stream.
  *             MI355_VARIANT_AUTO also uses it (256-byte aligned) to repack a large problem the
  *             tiled kernels cannot address (K*elem_bytes % 16, N % 4, strides, pointers) into
  *             an aligned one; without it such a problem runs on the slow generic kernel

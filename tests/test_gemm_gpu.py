@@ -656,6 +656,24 @@ def test_skinny_k_split_that_does_not_divide_the_k_steps(abi, dt, M, N, K):
     assert torch.equal(run_abi(abi, A, B, ac.SKINNY, 0.25).view(torch.int16), C.view(torch.int16))
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 4096, 14336), (90, 6144, 4096)])
+def test_auto_without_a_workspace_takes_the_tile_kernel_for_few_rows(abi, M, N, K):
+    """The streaming kernel's K split needs a workspace; MI355_VARIANT_AUTO called without one still
+    succeeds (on the tile kernel, unsplit), an explicit MI355_VARIANT_SKINNY does not."""
+    A, B = rand((M, K), 7, torch.bfloat16), rand((N, K), 8, torch.bfloat16)
+    assert abi.mi355_gemm_select_variant(M, N, K, ac.BF16) == ac.SKINNY
+    assert abi.mi355_gemm_workspace_bytes(M, N, K, ac.BF16, ac.AUTO) > 0
+    Ad, Bd = A.cuda(), B.cuda()
+    C = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    call = lambda v: abi.mi355_gemm_tn(Ad.data_ptr(), Bd.data_ptr(), C.data_ptr(), M, N, K, K, K, N, ac.BF16, ac.BF16, 1.0, v,
+                                       None, 0, s)
+    assert call(ac.SKINNY) == ac.ERR_WORKSPACE
+    assert call(ac.AUTO) == 0
+    torch.cuda.synchronize()
+    check(C.cpu(), A, B)
+
+
 def test_skinny_split_k_is_deterministic_and_needs_its_workspace(abi):
     M, N, K = 16, 256, 4096
     A, B = rand((M, K), 1, torch.bfloat16).cuda(), rand((N, K), 2, torch.bfloat16).cuda()

@@ -107,7 +107,7 @@ def test_every_tile_shape(abi, shape, tile):
     """The block-scaled kernel runs on the tile the planner picks for plain e4m3; a wave with 64 rows
     of an operand reads half a 128-row scale unit."""
     M, N, K = shape
-    assert ac.plan(abi, M, N, K, ac.E4M3)[1:3] == tile
+    assert ac.plan(abi, M, N, K, ac.E4M3, ac.BASIC)[1:3] == tile
     A, sa = random_mx(M, K, 21)
     B, sb = random_mx(N, K, 22)
     C = run_mx(abi, A, sa, B, sb, ldc=N + 4)
