@@ -105,6 +105,20 @@ def build_case(name, variant, device="cuda", seed=0):
         # rotate operand sets so weights come from HBM, not the Infinity Cache (256 MB)
         rot = max(2, int(600e6 // (N * K * 2)) + 1)
         sets, tag, fp8 = [w.skinny(M, N, K, seed + 10 * i, device) for i in range(rot)], "bf16", None
+    elif name.startswith("skinnyfp8_") or name.startswith("skinnymx_"):
+        # the same small-M shapes with e4m3 weights: unit per-tensor scales, or OCP MX block scales
+        # quantised by the library into the layout the kernels read
+        M, N, K = (int(x) for x in name.split("_")[1:])
+        rot = max(2, int(600e6 // (N * K)) + 1)
+        sets = []
+        for i in range(rot):
+            X, W = w.skinny(M, N, K, seed + 10 * i, device)
+            if name.startswith("skinnymx_"):
+                (xq, px), (wq, pw) = gemm_kernels.quantize_mxfp8(X, shuffled=True), gemm_kernels.quantize_mxfp8(W * 50.0, shuffled=True)
+                sets.append((xq, wq, px, pw))
+            else:
+                sets.append((X.to(torch.float8_e4m3fn), (W * 50.0).to(torch.float8_e4m3fn)))
+        tag, fp8 = "e4m3", (("mxsets",) if name.startswith("skinnymx_") else (1.0, 1.0))
     else:
         raise SystemExit("unknown workload " + name)
     M, K = sets[0][0].shape
@@ -114,9 +128,12 @@ def build_case(name, variant, device="cuda", seed=0):
     state = {"i": 0}
 
     def call():
-        A, B = sets[state["i"] % len(sets)]
+        A, B = sets[state["i"] % len(sets)][:2]
         state["i"] += 1
-        if fp8 and fp8[0] == "mx":
+        if fp8 and fp8[0] == "mxsets":
+            _, _, pa, pb = sets[(state["i"] - 1) % len(sets)]
+            gemm_kernels.gemm_tn_mxfp8(A, B, pa, pb, C, True)
+        elif fp8 and fp8[0] == "mx":
             gemm_kernels.gemm_tn_mxfp8(A, B, fp8[1], fp8[2], C, True)
         elif fp8:
             gemm_kernels.gemm_tn_fp8(A, B, fp8[0], fp8[1], C, variant)
@@ -125,7 +142,7 @@ def build_case(name, variant, device="cuda", seed=0):
 
     es = sets[0][0].element_size()
     nbytes = (M * K + N * K) * es + M * N * C.element_size()
-    if fp8 and fp8[0] == "mx":
+    if fp8 and fp8[0] in ("mx", "mxsets"):
         nbytes += (M + N) * (K // 32)
     return call, 2.0 * M * N * K, nbytes, tag, (M, N, K), sets, C, fp8
 
@@ -206,7 +223,7 @@ def main():
 
     head, keep = measure(a.workload, a.variant, a.steps, a.warmup)
     sets, C, fp8, flops, nbytes = keep
-    mfma_bound = not a.workload.startswith("skinny_")
+    mfma_bound = not a.workload.startswith("skinny")
     if mfma_bound:
         roof = {"bound": "mfma", "achieved": head["tflops"], "peak": PEAK_TFLOPS[head["dtype"]],
                 "unit": "TFLOP/s", "frac": round(head["tflops"] / PEAK_TFLOPS[head["dtype"]], 4),
@@ -229,7 +246,7 @@ def main():
     if not a.no_extras:
         names = ["bf16_8192", "fp8_8192", "mxfp8_8192", "bf16_4096", "fp16_512"] + \
                 ["skinny_%d_%d_%d" % (m, n, k) for (n, k) in ((14336, 4096), (4096, 14336), (6144, 4096))
-                 for m in (16, 64, 256)]
+                 for m in (16, 64, 256)] + ["skinnyfp8_16_14336_4096", "skinnymx_16_14336_4096"]
         for n in names:
             if n == a.workload:
                 continue
