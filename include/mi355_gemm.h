@@ -135,11 +135,13 @@ int mi355_quantize_e4m3(const void *x, int x_dtype, int64_t n, void *x_q,
  *   workspace          mi355_gemm_mx_workspace_bytes(M, N, K, scales_shuffled) bytes, 16-byte
  *                      aligned: the shuffled scales (required when scales_shuffled == 0) followed
  *                      by the partial results of a K split or tail split (optional: with less
- *                      room the tiles run unsplit).
+ *                      room the tiles run unsplit, and a problem of at most 64 rows runs on the
+ *                      tiled kernel instead of the weight-streaming one).
  * Constraints: K % 128 == 0; A, B 16-byte aligned with row strides that are multiples of 16;
- * N % 4 == 0, ldc % 4 == 0, C 8-byte aligned; the size limits of the tiled variants.  Always runs
- * the tiled kernel (MI355_VARIANT_BASIC) with the tile and splits mi355_gemm_plan reports for
- * MI355_E4M3 operands of this shape.
+ * N % 4 == 0, ldc % 4 == 0, C 8-byte aligned; the size limits of the tiled variants.  Runs the
+ * weight-streaming kernel (MI355_VARIANT_SKINNY) for M <= 64 and otherwise the tiled kernel
+ * (MI355_VARIANT_BASIC) with the tile and splits mi355_gemm_plan reports for MI355_E4M3 operands
+ * of this shape and that variant.
  * Counterpart in the reference: none (it has no fp8 path); same launcher contract as
  * mi355_gemm_tn (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92), block format per the OCP
  * Microscaling Formats (MX) specification v1.0.
