@@ -276,16 +276,25 @@ bool unsplit_deep(int64_t M, int64_t N, bool mx) {
   return tiles >= 200 && tiles <= 256 * per_cu;
 }
 
+// 64 x 64 tile: the four waves as 2 x 2 (32 x 32 each: two fragments of X and two of W per wave and
+// k-step instead of four and one; 3-9 % faster where the tile runs unsplit), except with block
+// scales, whose layout wants one 64-row half group per operand and wave.
+template <class T, class OutT, int kDepth>
+int launch_64(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
+  if constexpr (std::is_same<T, MxE4M3>::value) return launch_cfg<T, OutT, 4, 1, 1, 4, kDepth>(g, splits, ws, stream);
+  else return launch_cfg<T, OutT, 2, 2, 2, 2, kDepth>(g, splits, ws, stream);
+}
+
 template <class T, class OutT>
 int launch_m(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
   if (splits == 1 && unsplit_deep(g.M, g.N, std::is_same<T, MxE4M3>::value)) {
     if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
     if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
-    return launch_cfg<T, OutT, 4, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
+    return launch_64<T, OutT, kDepthUnsplit>(g, splits, ws, stream);
   }
   if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, kDepth16>(g, splits, ws, stream);   //  16x64, 10 KiB/step
   if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, kDepth32>(g, splits, ws, stream);   //  32x64, 12 KiB/step
-  if (g.M <= 64) return launch_cfg<T, OutT, 4, 1, 1, 4, kDepth64>(g, splits, ws, stream);   //  64x64, 16 KiB/step
+  if (g.M <= 64) return launch_64<T, OutT, kDepth64>(g, splits, ws, stream);                 //  64x64, 16 KiB/step
   if constexpr (std::is_same<T, MxE4M3>::value) {
     return -1;   // block scales: up to 64 rows (the host routes taller problems to the tile kernel)
   } else {
