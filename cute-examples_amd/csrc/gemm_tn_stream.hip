@@ -262,8 +262,9 @@ int launch_cfg(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
 constexpr int kDepth16 = 4, kDepth32 = 4, kDepth64 = 3, kDepth128 = 4, kDepth256 = 3;
 // Without a K split (enough tiles to give nearly every CU one) a workgroup has the CU to itself and
 // keeps its bytes in flight with a deep ring instead of with neighbours: 16x14336x4096 bf16
-// 27.7 us split four ways + reduce, 25.7 us unsplit with eight stages (27.1 us with fourteen).
-constexpr int kDepthUnsplit = 8;
+// 27.7 us split four ways + reduce, 25.7 us unsplit with eight stages (27.1 us with fourteen); with
+// the staggered start six stages are 2 % faster than eight over 36 problems.
+constexpr int kDepthUnsplit = 6;
 // That mode pays when the tiles occupy most of the 256 CUs and all of them are resident at once
 // with the deep ring (two workgroups per CU at M <= 16, one above): measured on N = 12800...28672,
 // bf16 and fp8, -7 to -20 % there; with more tiles than that (several rounds) the shallow ring with
