@@ -10,8 +10,11 @@
 //     full-cache-line direct-to-LDS loads into a ring of kDepth stages, kDepth-1 k-steps ahead;
 //   * the four waves read MFMA fragments from LDS (same 16-byte-chunk swizzle as the big-tile
 //     kernels) and run v_mfma_f32_16x16x32 (two per k-step and block pair) or, for fp8,
-//     v_mfma_f32_16x16x128_f8f6f4 (one); W blocks are the MFMA rows, so every lane ends up with
-//     four consecutive n of one m;
+//     v_mfma_f32_16x16x128_f8f6f4 (one; with OCP MX block scales its scaled form, the scale bytes
+//     riding through the ring behind the rows); W blocks are the MFMA rows, so every lane ends up
+//     with four consecutive n of one m;
+//   * workgroups start their k-steps at different points and wrap around, so that they do not all
+//     read the same column of rows a power of two apart (the same memory channels) at once;
 //   * with K split S ways the partial tiles go to an fp32 workspace [S][M][N] and a second kernel
 //     adds them in a fixed order (deterministic), scales and rounds; with S = 1 the tile is
 //     rounded and stored directly.
