@@ -43,12 +43,14 @@ bool tile256_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64
 
 // Constraints of the small-M streaming kernel.  It wins up to M = 64 ...
 constexpr int64_t kSkinnyAutoMaxM = 64;
-// ... and up to M = 96 while the 64-column tiles fit the 256 CUs in one round (N <= 16384): measured
-// on 40 bf16 and fp8 problems with M = 80 and 96 (N = 2048...28672), -6 % in the geometric mean, from
-// -25 % to +8 %; with more tiles than that the tile kernel is 14-20 % faster, and at M = 128 it wins
-// more often and by more (one problem by 32 %).
-bool auto_streams(int64_t M, int64_t N) {
-  return M <= kSkinnyAutoMaxM || (M <= 96 && (N + 63) / 64 <= 256);
+// ... and up to M = 128 while the 64-column tiles fit the 256 CUs in one round (N <= 16384) and the
+// rows of A, which every one of those tiles reads again, stay in an XCD's 4 MiB L2 beside the
+// streaming weights (M*K*elem_bytes <= 2.2 MB): measured on 72 bf16 and fp8 problems with M = 96 and
+// 128 (N = 2048...16384), -6 % in the geometric mean where the rule applies, from -22 % to +10 %;
+// with more tiles the tile kernel is 14-20 % faster, with more bytes of A up to 40 % faster.
+bool auto_streams(int64_t M, int64_t N, int64_t K, int64_t es) {
+  if (M <= kSkinnyAutoMaxM) return true;
+  return M <= 128 && (N + 63) / 64 <= 256 && M * K * es <= 2200000;
 }
 bool skinny_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int in_dtype) {
   if (M > 256) return false;
@@ -70,7 +72,7 @@ int resolve(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t l
   if (variant == MI355_VARIANT_AUTO) {
     if (!tile256_ok(M, N, K, lda, ldb, ldc, in_dtype)) return MI355_VARIANT_SIMPLE;
     // A few rows of activations against a large weight matrix: stream the weights.
-    if (auto_streams(M, N) && skinny_ok(M, N, K, lda, ldb, ldc, in_dtype)) return MI355_VARIANT_SKINNY;
+    if (auto_streams(M, N, K, elem_bytes(in_dtype)) && skinny_ok(M, N, K, lda, ldb, ldc, in_dtype)) return MI355_VARIANT_SKINNY;
     return MI355_VARIANT_BASIC;
   }
   if (variant == MI355_VARIANT_BASIC || variant == MI355_VARIANT_PINGPONG)

@@ -292,7 +292,7 @@ def test_plan_invariants_over_random_shapes(abi):
             v, rows, cols, splits, tail_tiles, tail_splits = ac.plan(abi, M, N, K, dt)
             steps = -(-K * es // 128)
             assert v in (ac.BASIC, ac.SKINNY), (M, N, K, v)
-            assert (v == ac.SKINNY) == (M <= 64 or (M <= 96 and -(-N // 64) <= 256))
+            assert (v == ac.SKINNY) == (M <= 64 or (M <= 128 and -(-N // 64) <= 256 and M * K * es <= 2200000))
             tiles = -(-M // rows) * -(-N // cols)
             assert splits >= 1 and tail_splits >= 1 and tail_tiles >= 0
             if splits > 1:
