@@ -268,7 +268,7 @@ constexpr int kDepth16 = 4, kDepth32 = 4, kDepth64 = 3, kDepth128 = 4, kDepth256
 // 27.7 us split four ways + reduce, 25.7 us unsplit with eight stages (27.1 us with fourteen); with
 // the staggered start six stages are 2 % faster than eight over 36 problems.
 constexpr int kDepthUnsplit = 6;
-// That mode pays when the tiles occupy most of the 256 CUs and all of them are resident at once
+// That mode pays when the tiles occupy more than half of the 256 CUs and all of them are resident at once
 // with the deep ring (two workgroups per CU at M <= 16, one above): measured on N = 12800...28672,
 // bf16 and fp8, -7 to -20 % there; with more tiles than that (several rounds) the shallow ring with
 // three or four workgroups per CU is 5-20 % faster again.
@@ -278,7 +278,9 @@ bool unsplit_deep(int64_t M, int64_t N, bool mx) {
   const int64_t per_cu = 163840 / (kDepthUnsplit * ((tm + kTileN) * kRowBytes + (mx ? 512 : 0)));
   const int64_t tiles = (N + kTileN - 1) / kTileN;
   // (two per CU only for the lowest tile: fp8 32x28672x4096 measured 5 % slower that way than split)
-  return tiles >= 200 && tiles <= 256 * (tm <= 16 ? per_cu : 1);
+  // From 150 tiles on for the two lower tiles (N = 11008 and 12288 at M <= 32: -16 to -18 % against the
+  // split; with 128 tiles +25 %), from 200 for the 64-row tile (150...199 tiles: -10 % to +14 %).
+  return tiles >= (tm <= 32 ? 150 : 200) && tiles <= 256 * (tm <= 16 ? per_cu : 1);
 }
 
 // 64 x 64 tile: the four waves as 2 x 2 (32 x 32 each: two fragments of X and two of W per wave and
