@@ -2,11 +2,26 @@
 """Benchmark of the GEMM hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-extras] [--no-cpu]
+                    [--no-calibrate] [--no-fp8]
 
 A step is one gemm launch over one set of synthetic operands already resident in HBM.  The
 headline workload is bf16 M=N=K=8192, Normal(0,1) operands (the configuration the metric is
 quoted on); fp8 8192^3 (per-tensor scales and MX block scales), bf16 4096^3, fp16 512^3 and the
-skinny projection shapes are timed with fewer steps and reported under "extras".  Prints ONE JSON line.
+skinny projection shapes are timed with fewer steps and reported under "extras".  The metric names
+two configurations, so fp8 e4m3 8192^3 gets a block of its own ("fp8": value, roofline, cpu_baseline)
+measured with the same protocol and the same K and W as the headline.  Prints ONE JSON line.
+
+Clock settling.  The shader clock of an idle GPU needs tens of milliseconds of load to reach the
+level it then sustains (an 8192^3 GEMM runs ~13 % slower in the first few milliseconds after an
+idle period, ~5 % slower over the first 60 launches).  Every measurement therefore begins with a settle phase that is
+not part of W or K: the same launch repeated, in batches timed with HIP events, for at least
+150 ms and until three consecutive batches agree within 1 % (at most 2 s).  It is reported as
+settle_launches / settle_ms; the W warm-up and K timed launches follow it back to back.
+
+Calibration (on by default, --no-calibrate skips it): the library's MFMA-only kernel on the
+workload's own operands and its plain read kernel give roofline.measured_mfma_ceiling and
+roofline.measured_hbm_read, what this GPU sustains with nothing but matrix-core work / nothing but
+loads.  roofline.frac stays against the published peak.
 
 Protocol follows the reference's benchmark (kernels/tests/gemm_bench.py:285-295, :502-506):
 warm-up, then timed launches, TFLOP/s = 2*M*N*K / t — with HIP events on the launch stream
@@ -29,6 +44,10 @@ PEAK_HBM_GBS = 8000.0
 # (FETCH_SIZE, then WRITE_SIZE, each with --copy-calibration and scaled by what the same counter
 # reads for the 1 GiB copy: x2.000 and x1.000).  Workloads without a counter run report null.
 MEASURED_TRAFFIC_BYTES = {"bf16_8192": 1.793e9, "fp8_8192": 0.963e9, "mxfp8_8192": 0.965e9, "skinny_16_14336_4096": 1.190e8}
+TRAFFIC_PROFILE = {"bf16_8192": "profiles/gemm_tn_tile_ring__bf16_8192.md", "fp8_8192": "profiles/gemm_tn_tile_ring__fp8_8192.md",
+                   "mxfp8_8192": "profiles/gemm_tn_tile_ring__mxfp8_8192.md",
+                   "skinny_16_14336_4096": "profiles/gemm_tn_stream__skinny_16_14336_4096.md"}
+SETTLE_MIN_MS, SETTLE_MAX_MS, SETTLE_BATCH_MS = 150.0, 2000.0, 10.0
 
 
 def parse():
@@ -42,6 +61,10 @@ def parse():
     p.add_argument("--variant", default="auto")
     p.add_argument("--no-extras", action="store_true")
     p.add_argument("--no-cpu", action="store_true")
+    p.add_argument("--no-fp8", action="store_true", help="skip the fp8 8192^3 block of the metric")
+    p.add_argument("--calibrate", action="store_true", help="(default) measure the MFMA-only and plain-read ceilings")
+    p.add_argument("--no-calibrate", action="store_true")
+    p.add_argument("--no-settle", action="store_true", help="skip the clock-settle phase in front of every measurement")
     p.add_argument("--copy-calibration", action="store_true",
                    help="also run three 1 GiB device-to-device copies (known traffic: 1 GiB read + 1 GiB "
                         "written each) so that a rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this "
@@ -49,9 +72,43 @@ def parse():
     return p.parse_args()
 
 
-def time_calls(call, steps, warmup):
-    """HIP events on the current stream around `steps` back-to-back launches -> ms per launch."""
+def settle(call, enabled=True):
+    """Clock-settle phase: repeat the launch in event-timed batches of ~10 ms for at least
+    SETTLE_MIN_MS and until three consecutive batches agree within 1 %, at most SETTLE_MAX_MS.
+    Returns (launches, total ms, ms per launch of the last batch)."""
     import torch
+    if not enabled:
+        return 0, 0.0, None
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    call()
+    e1.record()
+    torch.cuda.synchronize()
+    per = max(e0.elapsed_time(e1), 1e-3)
+    batch = max(1, min(2000, int(SETTLE_BATCH_MS / per)))
+    launches, total, history = 1, per, []
+    while total < SETTLE_MAX_MS:
+        e0.record()
+        for _ in range(batch):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        launches += batch
+        total += ms
+        history.append(ms / batch)
+        if total >= SETTLE_MIN_MS and len(history) >= 3:
+            last = history[-3:]
+            if max(last) <= 1.01 * min(last):
+                break
+    return launches, total, history[-1] if history else per
+
+
+def time_calls(call, steps, warmup, do_settle=True):
+    """Settle phase, then `warmup` untimed launches, then HIP events on the current stream around
+    `steps` back-to-back launches -> (ms per launch, wall ms per launch, settle launches, settle ms)."""
+    import torch
+    n_settle, settle_ms, _ = settle(call, do_settle)
     for _ in range(warmup):
         call()
     torch.cuda.synchronize()
@@ -63,7 +120,7 @@ def time_calls(call, steps, warmup):
     e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return e0.elapsed_time(e1) / steps, wall_ms
+    return e0.elapsed_time(e1) / steps, wall_ms, n_settle, settle_ms
 
 
 def per_launch_ms(call, steps):
@@ -147,12 +204,13 @@ def build_case(name, variant, device="cuda", seed=0):
     return call, 2.0 * M * N * K, nbytes, tag, (M, N, K), sets, C, fp8
 
 
-def measure(name, variant, steps, warmup):
+def measure(name, variant, steps, warmup, do_settle=True):
     call, flops, nbytes, tag, mnk, sets, C, fp8 = build_case(name, variant)
-    ms, wall_ms = time_calls(call, steps, warmup)
+    ms, wall_ms, n_settle, settle_ms = time_calls(call, steps, warmup, do_settle)
     med, mn = per_launch_ms(call, steps)
     tflops = flops / ms / 1e9
-    row = {"workload": name, "M": mnk[0], "N": mnk[1], "K": mnk[2], "dtype": tag, "steps": steps,
+    row = {"workload": name, "M": mnk[0], "N": mnk[1], "K": mnk[2], "dtype": tag, "steps": steps, "warmup": warmup,
+           "settle_launches": n_settle, "settle_ms": round(settle_ms, 1),
            "ms": round(ms, 5), "wall_ms": round(wall_ms, 5), "launch_ms_median": round(med, 5),
            "launch_ms_min": round(mn, 5), "tflops": round(tflops, 2),
            "pct_mfma_peak": round(100 * tflops / PEAK_TFLOPS[tag], 2),
@@ -160,20 +218,83 @@ def measure(name, variant, steps, warmup):
     return row, (sets, C, fp8, flops, nbytes)
 
 
-def cpu_baseline(A, B, total_rows, budget_s=12.0, native_budget_s=5.0):
+def roofline_of(row, workload, variant, sets, flops, nbytes):
+    """The roofline object of one measured workload (the dominant kernel is its only GEMM kernel)."""
+    import gemm_kernels
+    traffic = MEASURED_TRAFFIC_BYTES.get(workload)
+    if not workload.startswith("skinny"):
+        roof = {"bound": "mfma", "achieved": row["tflops"], "peak": PEAK_TFLOPS[row["dtype"]],
+                "unit": "TFLOP/s", "frac": round(row["tflops"] / PEAK_TFLOPS[row["dtype"]], 4), "traffic": traffic}
+    else:
+        roof = {"bound": "hbm", "achieved": row["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": round(row["gbs"] / PEAK_HBM_GBS, 4), "traffic": traffic}
+    # the counters are not read in this run: the figure is the one of the committed profile of this command
+    roof["traffic_source"] = (TRAFFIC_PROFILE[workload] + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this "
+                              "script, scaled by a 1 GiB copy; not re-measured in this run)") if traffic else None
+    roof["kernel"] = gemm_kernels.select_variant(row["M"], row["N"], row["K"], sets[0][0].dtype) \
+        if variant == "auto" else variant
+    roof["flops_per_launch"] = flops
+    roof["algorithmic_bytes_per_launch"] = nbytes
+    roof["avg_launch_ms"] = row["ms"]
+    roof["launch_ms_median"], roof["launch_ms_min"] = row["launch_ms_median"], row["launch_ms_min"]
+    return roof
+
+
+def calibrate(A, B, do_settle=True):
+    """The library's two ceiling kernels through its C ABI: matrix cores only, on the workload's own
+    operands (dtype of A), and a plain read of 1 GiB.  Returns the two roofline entries."""
+    import ctypes
+    import torch
+    lib = ctypes.CDLL(os.path.join(ROOT, "cute-examples_amd", "gemm_kernels", "libmi355gemm.so"))
+    vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    lib.mi355_calibrate_sink_bytes.restype = sz
+    lib.mi355_calibrate_mfma.argtypes = [ci, vp, sz, vp, sz, ci, vp, ctypes.POINTER(ctypes.c_double), vp]
+    lib.mi355_calibrate_read.argtypes = [vp, sz, vp, vp]
+    code = {torch.bfloat16: 0, torch.float16: 1, torch.float8_e4m3fn: 2}[A.dtype]
+    sink = torch.empty(lib.mi355_calibrate_sink_bytes(), dtype=torch.uint8, device=A.device)
+    flops = ctypes.c_double()
+    iters = 4000   # ~2 ms per launch
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def mfma():
+        rc = lib.mi355_calibrate_mfma(code, A.data_ptr(), A.numel() * A.element_size(), B.data_ptr(),
+                                      B.numel() * B.element_size(), iters, sink.data_ptr(), ctypes.byref(flops), stream)
+        assert rc == 0, rc
+    ms, _, n_settle, settle_ms = time_calls(mfma, 40, 5, do_settle)
+    mfma_entry = {"value": round(flops.value / ms / 1e9, 1), "unit": "TFLOP/s", "ms_per_launch": round(ms, 4),
+                  "settle_launches": n_settle, "settle_ms": round(settle_ms, 1),
+                  "what": "mi355_calibrate_mfma: 4 waves per CU, the tile kernel's MFMA pattern on fragments of this "
+                          "workload's operands held in registers; no LDS, no copies, no barriers"}
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=A.device)
+    src.view(torch.int32).random_()
+
+    def read():
+        rc = lib.mi355_calibrate_read(src.data_ptr(), src.numel(), sink.data_ptr(), stream)
+        assert rc == 0, rc
+    ms, _, n_settle, settle_ms = time_calls(read, 100, 10, do_settle)
+    read_entry = {"value": round(src.numel() / ms / 1e6, 1), "unit": "GB/s", "ms_per_launch": round(ms, 4),
+                  "settle_launches": n_settle, "settle_ms": round(settle_ms, 1),
+                  "what": "mi355_calibrate_read: 16-byte loads over 1 GiB (four times the Infinity Cache), nothing else"}
+    del src, sink
+    torch.cuda.empty_cache()
+    return mfma_entry, read_entry
+
+
+def cpu_baseline(A, B, total_rows, scale=1.0, budget_s=12.0, native_budget_s=5.0):
     """The oracle's fp32 matmul (the reference's ground truth, gemm_test.py:36) timed on the host
-    cores on a bounded sample: as many row blocks of A against all of B as fit the budget."""
+    cores on a bounded sample: as many row blocks of A against all of B as fit the budget.  For fp8
+    operands this is the fp32 product of the dequantised operands times scale_a * scale_b."""
     import torch
     from oracle import oracle
     Bc = B.cpu()
     N, K = Bc.shape
     rows = min(1024, A.shape[0])
     Ac = A[:rows].cpu()   # the caller may hand over just these rows (already on the host)
-    oracle.gemm_tn_fp32(Ac[:64], Bc)            # warm-up (thread pool, conversions)
+    oracle.gemm_tn_fp32(Ac[:64], Bc, scale)            # warm-up (thread pool, conversions)
     t0 = time.perf_counter()
     done = 0
     while True:
-        oracle.gemm_tn_fp32(Ac, Bc)
+        oracle.gemm_tn_fp32(Ac, Bc, scale)
         done += rows
         el = time.perf_counter() - t0
         if el > budget_s or done >= 16 * total_rows:
@@ -181,7 +302,7 @@ def cpu_baseline(A, B, total_rows, budget_s=12.0, native_budget_s=5.0):
     tflops = 2.0 * done * N * K / el / 1e12
     # The same product in the operands' own 16-bit type, where torch has a CPU kernel for it.
     native = None
-    if Ac.dtype in (torch.bfloat16, torch.float16):
+    if Ac.dtype in (torch.bfloat16, torch.float16) and native_budget_s > 0:
         try:
             torch.matmul(Ac[:64], Bc.T)
             t0, n_done = time.perf_counter(), 0
@@ -194,11 +315,12 @@ def cpu_baseline(A, B, total_rows, budget_s=12.0, native_budget_s=5.0):
             native = round(2.0 * n_done * N * K / el_n / 1e12, 4)
         except RuntimeError:
             native = None
+    kind = "e4m3->fp32" if Ac.dtype == torch.float8_e4m3fn else "%s->fp32" % str(Ac.dtype).split(".")[-1]
     return {"value": round(tflops, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
             "kind": "port", "native_16bit_value": native,
-            "sample": "torch.matmul fp32 (incl. bf16->fp32 casts) of %d-row blocks of A against all of B "
+            "sample": "torch.matmul fp32 (incl. the %s casts) of %d-row blocks of A against all of B "
                       "(N=%d, K=%d), %d rows in %.1f s; host has %d logical cpus"
-                      % (rows, N, K, done, el, os.cpu_count())}
+                      % (kind, rows, N, K, done, el, os.cpu_count())}
 
 
 def main():
@@ -210,7 +332,7 @@ def main():
     import torch
     if not torch.cuda.is_available():
         raise SystemExit("bench.py needs a GPU")
-    import gemm_kernels
+    import gemm_kernels  # noqa: F401  (fails loudly when the extension is not built)
 
     if a.copy_calibration:
         src = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda").normal_()
@@ -221,26 +343,42 @@ def main():
         del src, dst
         torch.cuda.empty_cache()
 
-    head, keep = measure(a.workload, a.variant, a.steps, a.warmup)
+    do_settle = not a.no_settle
+    head, keep = measure(a.workload, a.variant, a.steps, a.warmup, do_settle)
     sets, C, fp8, flops, nbytes = keep
-    mfma_bound = not a.workload.startswith("skinny")
-    if mfma_bound:
-        roof = {"bound": "mfma", "achieved": head["tflops"], "peak": PEAK_TFLOPS[head["dtype"]],
-                "unit": "TFLOP/s", "frac": round(head["tflops"] / PEAK_TFLOPS[head["dtype"]], 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload)}
-    else:
-        roof = {"bound": "hbm", "achieved": head["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": round(head["gbs"] / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(a.workload)}
-    roof["kernel"] = gemm_kernels.select_variant(head["M"], head["N"], head["K"], sets[0][0].dtype) \
-        if a.variant == "auto" else a.variant
-    roof["flops_per_launch"] = flops
-    roof["algorithmic_bytes_per_launch"] = nbytes
-    roof["avg_launch_ms"] = head["ms"]
-    roof["launch_ms_median"], roof["launch_ms_min"] = head["launch_ms_median"], head["launch_ms_min"]
+    roof = roofline_of(head, a.workload, a.variant, sets, flops, nbytes)
+    if not a.no_calibrate:
+        roof["measured_mfma_ceiling"], roof["measured_hbm_read"] = calibrate(sets[0][0], sets[0][1], do_settle)
+        if roof["bound"] == "mfma":
+            roof["frac_of_measured_ceiling"] = round(head["tflops"] / roof["measured_mfma_ceiling"]["value"], 4)
+        else:
+            roof["frac_of_measured_ceiling"] = round(head["gbs"] / roof["measured_hbm_read"]["value"], 4)
 
-    cpu_operands = (sets[0][0][:1024].cpu(), sets[0][1].cpu(), sets[0][0].shape[0]) if not a.no_cpu else None
+    head_scale = float(fp8[0]) * float(fp8[1]) if fp8 and isinstance(fp8[0], float) else 1.0
+    cpu_operands = (sets[0][0][:1024].cpu(), sets[0][1].cpu(), sets[0][0].shape[0], head_scale) if not a.no_cpu else None
     del sets, C, keep
     torch.cuda.empty_cache()
+
+    # The second configuration of the metric: fp8 e4m3 8192^3, same protocol, same K and W.
+    fp8_block, fp8_cpu_operands = None, None
+    if a.workload == "bf16_8192" and not a.no_fp8:
+        row, keep = measure("fp8_8192", a.variant, a.steps, a.warmup, do_settle)
+        sets8, C8, sc8, flops8, nbytes8 = keep
+        roof8 = roofline_of(row, "fp8_8192", a.variant, sets8, flops8, nbytes8)
+        if not a.no_calibrate:
+            roof8["measured_mfma_ceiling"], _ = calibrate(sets8[0][0], sets8[0][1], do_settle)
+            roof8["frac_of_measured_ceiling"] = round(row["tflops"] / roof8["measured_mfma_ceiling"]["value"], 4)
+        fp8_block = {"value": row["tflops"], "unit": "TFLOP/s", "ms_per_step": row["ms"], "steps": a.steps,
+                     "warmup": a.warmup, "settle_launches": row["settle_launches"], "settle_ms": row["settle_ms"],
+                     "dtype": "e4m3", "pct_of_dense_mfma_peak": row["pct_mfma_peak"],
+                     "config": {"workload": "fp8_8192: M=N=K=8192 e4m3 operands quantised from Normal(0,1) with per-tensor "
+                                            "fp32 scales amax/448, fp32 accumulate, bf16 output after scale",
+                                "variant": roof8["kernel"]},
+                     "roofline": roof8, "cpu_baseline": None}
+        if not a.no_cpu:
+            fp8_cpu_operands = (sets8[0][0][:1024].cpu(), sets8[0][1].cpu(), sets8[0][0].shape[0], float(sc8[0]) * float(sc8[1]))
+        del sets8, C8, keep
+        torch.cuda.empty_cache()
 
     extras = []
     if not a.no_extras:
@@ -248,16 +386,16 @@ def main():
                 ["skinny_%d_%d_%d" % (m, n, k) for (n, k) in ((14336, 4096), (4096, 14336), (6144, 4096))
                  for m in (16, 64, 256)] + ["skinnyfp8_16_14336_4096", "skinnymx_16_14336_4096"]
         for n in names:
-            if n == a.workload:
+            if n == a.workload or (n == "fp8_8192" and fp8_block):
                 continue
             steps = 60 if "8192" in n else 200
-            row, keep = measure(n, "auto", steps, steps)
+            row, keep = measure(n, "auto", steps, steps, do_settle)
             extras.append(row)
             del keep
             torch.cuda.empty_cache()
         if a.workload == "bf16_8192" and a.variant == "auto":
             for v in ("basic", "pingpong"):
-                row, keep = measure("bf16_8192", v, 60, 60)
+                row, keep = measure("bf16_8192", v, 60, 60, do_settle)
                 row["variant"] = v
                 extras.append(row)
                 del keep
@@ -265,16 +403,19 @@ def main():
 
     # Last, so that the GPU does not idle (and drop its clocks) in the middle of the measurements.
     cpu = cpu_baseline(*cpu_operands) if cpu_operands else None
+    if fp8_block and fp8_cpu_operands:
+        fp8_block["cpu_baseline"] = cpu_baseline(*fp8_cpu_operands, budget_s=8.0, native_budget_s=0.0)
 
     out = {
         "metric": METRIC, "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1,
-        "steps": a.steps, "warmup": a.warmup, "ms_per_step": head["ms"], "higher_is_better": True,
+        "steps": a.steps, "warmup": a.warmup, "settle_launches": head["settle_launches"], "settle_ms": head["settle_ms"],
+        "ms_per_step": head["ms"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic",
         "config": {"workload": "%s: M=%d N=%d K=%d, A (M,K) and B (N,K) K-contiguous, fp32 accumulate"
                                % (a.workload, head["M"], head["N"], head["K"]),
                    "variant": roof["kernel"], "parallelism": "single GPU"},
         "pct_of_dense_mfma_peak": head["pct_mfma_peak"],
-        "roofline": roof, "cpu_baseline": cpu, "extras": extras,
+        "roofline": roof, "cpu_baseline": cpu, "fp8": fp8_block, "extras": extras,
     }
     print(json.dumps(out))
 

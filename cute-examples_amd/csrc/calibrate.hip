@@ -1,0 +1,116 @@
+// Measured ceilings of one GPU, for the benchmark's roofline line: what the matrix cores sustain
+// with nothing else going on, and what a plain read of HBM reaches.  The published peaks assume the
+// nominal clock; under the board power limit the sustained figures are lower and depend on the data
+// (all-zero operands draw far less power than random ones), so both kernels work on the caller's
+// own operands.
+//
+//   mfma_ceiling   every wave holds 8 + 8 operand fragments in registers (loaded once from the
+//                  caller's A and B) and runs the tile kernel's MFMA pattern on them -- 64
+//                  accumulator blocks, acc[i][j] += a[i] * b[j], the same instruction and the same
+//                  dependency distance as a k-step of gemm_tn_tile_ring -- with no LDS traffic, no
+//                  copies, no barriers.  One workgroup of four waves per CU.
+//   read_ceiling   16-byte loads, grid-stride over the buffer, xor-reduced so nothing is elided.
+//
+// Counterpart in the reference: none (its benchmark takes the peak from a table,
+// kernels/tests/gemm_bench.py:592-599).
+#include "../../include/mi355_gemm.h"
+
+#include "ring_common.h"
+
+namespace mi355 {
+namespace {
+
+template <class G>
+__global__ __launch_bounds__(256, 1) void mfma_ceiling(const uint8_t* a, const uint8_t* b, size_t a_bytes,
+                                                       size_t b_bytes, int iters, float* sink) {
+  typedef typename G::Frag Frag;
+  typedef typename G::Acc Acc;
+  constexpr int kN = 8;
+  Frag fa[kN], fb[kN];
+  Acc acc[kN][kN];
+  // Fragment i of this lane: sizeof(Frag) bytes of the operand, a different place for every lane,
+  // wave, workgroup and i (wrapping around inside the buffer).
+  const size_t lane_id = (size_t)blockIdx.x * 256 + threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < kN; ++i) {
+    const size_t at = (lane_id * kN + i) * sizeof(Frag);
+    fa[i] = *(const Frag*)(a + at % (a_bytes - sizeof(Frag) + 1) / sizeof(Frag) * sizeof(Frag));
+    fb[i] = *(const Frag*)(b + at % (b_bytes - sizeof(Frag) + 1) / sizeof(Frag) * sizeof(Frag));
+  }
+#pragma unroll
+  for (int i = 0; i < kN; ++i)
+#pragma unroll
+    for (int j = 0; j < kN; ++j)
+#pragma unroll
+      for (int r = 0; r < (int)(sizeof(Acc) / 4); ++r) acc[i][j][r] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+    static_for<kN * kN>([&](auto uc) __attribute__((always_inline)) {
+      constexpr int u = decltype(uc)::value;
+      G::mfma_inplace(fb[u % kN], fa[u / kN], acc[u / kN][u % kN]);
+    });
+  }
+  // The MFMAs are inline assembly: the compiler does not know how long their results take.
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < kN; ++i)
+#pragma unroll
+    for (int j = 0; j < kN; ++j) {
+      Acc c = acc[i][j];
+      asm volatile("" : "+a"(c));
+      s += c[0];
+    }
+  sink[lane_id] = s;
+}
+
+__global__ __launch_bounds__(256) void read_ceiling(const u32x4* src, size_t chunks, uint32_t* sink) {
+  u32x4 x = {0, 0, 0, 0};
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < chunks; i += stride) x ^= __builtin_nontemporal_load(src + i);
+  sink[(size_t)blockIdx.x * 256 + threadIdx.x] = x[0] ^ x[1] ^ x[2] ^ x[3];
+}
+
+}  // namespace
+}  // namespace mi355
+
+extern "C" {
+
+size_t mi355_calibrate_sink_bytes(void) { return (size_t)4096 * 256 * 4; }
+
+int mi355_calibrate_mfma(int in_dtype, const void* a, size_t a_bytes, const void* b, size_t b_bytes, int iters,
+                         void* sink, double* flops, void* stream) {
+  using namespace mi355;
+  if (!a || !b || !sink || !flops) return MI355_ERR_NULL;
+  if (in_dtype != MI355_BF16 && in_dtype != MI355_F16 && in_dtype != MI355_E4M3) return MI355_ERR_DTYPE;
+  if (iters <= 0 || a_bytes < 4096 || b_bytes < 4096) return MI355_ERR_SHAPE;
+  if ((uintptr_t)a % 32 != 0 || (uintptr_t)b % 32 != 0 || (uintptr_t)sink % 4 != 0) return MI355_ERR_ALIGN;
+  const int cus = compute_units();
+  if (cus > 4096) return MI355_ERR_LAUNCH;
+  hipStream_t s = (hipStream_t)stream;
+  const uint8_t* pa = (const uint8_t*)a;
+  const uint8_t* pb = (const uint8_t*)b;
+  // flop per MFMA: 2 * 16 * 16 * K, K = 32 (16-bit) or 128 (fp8)
+  const double per_mfma = in_dtype == MI355_E4M3 ? 2.0 * 16 * 16 * 128 : 2.0 * 16 * 16 * 32;
+  *flops = per_mfma * 64.0 * (double)iters * 4.0 * (double)cus;
+  if (in_dtype == MI355_BF16)
+    hipLaunchKernelGGL(mfma_ceiling<Geo<BF16>>, dim3(cus), dim3(256), 0, s, pa, pb, a_bytes, b_bytes, iters, (float*)sink);
+  else if (in_dtype == MI355_F16)
+    hipLaunchKernelGGL(mfma_ceiling<Geo<F16>>, dim3(cus), dim3(256), 0, s, pa, pb, a_bytes, b_bytes, iters, (float*)sink);
+  else
+    hipLaunchKernelGGL(mfma_ceiling<GeoE4M3Rows>, dim3(cus), dim3(256), 0, s, pa, pb, a_bytes, b_bytes, iters, (float*)sink);
+  return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ERR_LAUNCH;
+}
+
+int mi355_calibrate_read(const void* src, size_t bytes, void* sink, void* stream) {
+  using namespace mi355;
+  if (!src || !sink) return MI355_ERR_NULL;
+  if (bytes < 16) return MI355_ERR_SHAPE;
+  if ((uintptr_t)src % 16 != 0 || (uintptr_t)sink % 4 != 0) return MI355_ERR_ALIGN;
+  const int cus = compute_units();
+  const unsigned blocks = (unsigned)(cus * 16 < 4096 ? cus * 16 : 4096);
+  hipLaunchKernelGGL(read_ceiling, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const u32x4*)src, bytes / 16,
+                     (uint32_t*)sink);
+  return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ERR_LAUNCH;
+}
+
+}  // extern "C"

@@ -290,9 +290,15 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   const uint32_t a_lane = (wm * kWaveTileM + rblk) * kRowBytes;
   const uint32_t b_lane = (wn * kWaveTileN + rblk) * kRowBytes;
   // Byte offset inside a row of the e-th chunk this lane reads in slice s.
-  // With block scales the order of K inside the MFMA matters: group g supplies chunks g and 4+g.
+  // When one MFMA spans the k-step, group g supplies chunks g and 4+g.  With block scales the order
+  // of K inside the MFMA demands it; without them any order that is the same for both operands gives
+  // the same dot product, and this one is free of LDS bank conflicts: a ds_read_b128 is served 16
+  // lanes per cycle, lanes {0-3, 12-15, 20-23, 24-27} first (then {4-11, 16-19, 28-31}, then the same
+  // of the upper 32), i.e. rows from two neighbouring groups together, and the chunks 2g, 2g+1 of
+  // neighbouring groups differ in bit 1, which the row swizzle maps onto the same banks (counted:
+  // one conflict cycle per access cycle), while g and g+1 differ in bit 0 and do not collide.
   auto chunk_off = [&](int s, int e) __attribute__((always_inline)) -> uint32_t {
-    if constexpr (kMx) return ((uint32_t)(grp + 4 * e) ^ swz) << 4;
+    if constexpr (kRowSliced) return ((uint32_t)(grp + 4 * e) ^ swz) << 4;
     else return ((uint32_t)(s * kSliceChunks + grp * G::kCpl + e) ^ swz) << 4;
   };
   auto load_frag = [&](const uint8_t* slot_rows, int blk, int s) __attribute__((always_inline)) -> Frag {

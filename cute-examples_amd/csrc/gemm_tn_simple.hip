@@ -12,14 +12,19 @@ namespace {
 
 template <class T, class OutT>
 __global__ __launch_bounds__(256) void gemm_tn_simple(GemmArgs g) {
-  const int64_t n = (int64_t)blockIdx.x * 16 + (threadIdx.x & 15);
-  const int64_t m = (int64_t)blockIdx.y * 16 + (threadIdx.x >> 4);
-  if (m >= g.M || n >= g.N) return;
-  const int64_t a0 = m * g.lda, b0 = n * g.ldb;
-  float acc = 0.f;
-  for (int64_t k = 0; k < g.K; ++k)
-    acc = __builtin_fmaf(Decode<T>::run(g.A, a0 + k), Decode<T>::run(g.B, b0 + k), acc);
-  ((uint16_t*)g.C)[m * g.ldc + n] = Pack4<OutT>::one(acc * output_scale(g));
+  // 16 x 16 outputs per workgroup; the workgroups walk the blocks of C in one dimension (the y and z
+  // dimensions of a grid hold 65535 entries only), striding when there are more than 2^31 - 1.
+  const int64_t blocks_n = (g.N + 15) / 16, blocks = blocks_n * ((g.M + 15) / 16);
+  for (int64_t b = blockIdx.x; b < blocks; b += gridDim.x) {
+    const int64_t n = (b % blocks_n) * 16 + (threadIdx.x & 15);
+    const int64_t m = (b / blocks_n) * 16 + (threadIdx.x >> 4);
+    if (m >= g.M || n >= g.N) continue;
+    const int64_t a0 = m * g.lda, b0 = n * g.ldb;
+    float acc = 0.f;
+    for (int64_t k = 0; k < g.K; ++k)
+      acc = __builtin_fmaf(Decode<T>::run(g.A, a0 + k), Decode<T>::run(g.B, b0 + k), acc);
+    ((uint16_t*)g.C)[m * g.ldc + n] = Pack4<OutT>::one(acc * output_scale(g));
+  }
 }
 
 // One thread per 16-byte chunk of the destination.  The source has only element alignment, so it is
@@ -62,8 +67,9 @@ __global__ __launch_bounds__(256) void copy_out(const uint16_t* __restrict__ src
 
 template <class T, class OutT>
 int launch(const GemmArgs& g, hipStream_t stream) {
-  dim3 grid((unsigned)((g.N + 15) / 16), (unsigned)((g.M + 15) / 16));
-  hipLaunchKernelGGL((gemm_tn_simple<T, OutT>), grid, dim3(256), 0, stream, g);
+  const int64_t blocks = ((g.N + 15) / 16) * ((g.M + 15) / 16);
+  const int64_t grid = blocks < 0x7fffffff ? blocks : 0x7fffffff;
+  hipLaunchKernelGGL((gemm_tn_simple<T, OutT>), dim3((unsigned)grid), dim3(256), 0, stream, g);
   return hipGetLastError() == hipSuccess ? 0 : -1;
 }
 

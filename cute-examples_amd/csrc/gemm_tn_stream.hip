@@ -149,14 +149,13 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
     const uint8_t* p = rows + blk * 16 * kRowBytes;
     if constexpr (G::kCpl == 1) {
       return *(const i32x4*)(p + (((uint32_t)(s * kSliceChunks) + grp) ^ swz) * 16);
-    } else if constexpr (kMx) {
-      // the order of K inside the scaled MFMA matters: lane group g supplies chunks g and 4+g
+    } else {
+      // One MFMA spans the k-step: lane group g supplies chunks g and 4+g.  The scaled MFMA needs that
+      // order of K; the plain one takes any order common to both operands, and this one has no LDS
+      // bank conflicts where chunks 2g, 2g+1 have one per access (see chunk_off in gemm_tn_ring.h).
+      static_assert(kSlices == 1, "a fragment of two chunks covers the whole k-step");
       const i32x4 lo = *(const i32x4*)(p + ((grp ^ swz) * 16));
       const i32x4 hi = *(const i32x4*)(p + (((grp + 4) ^ swz) * 16));
-      return (i32x8){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    } else {
-      const i32x4 lo = *(const i32x4*)(p + (((uint32_t)(s * kSliceChunks) + grp * 2) ^ swz) * 16);
-      const i32x4 hi = *(const i32x4*)(p + (((uint32_t)(s * kSliceChunks) + grp * 2 + 1) ^ swz) * 16);
       return (i32x8){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
   };

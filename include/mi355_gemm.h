@@ -220,6 +220,26 @@ int mi355_gemm_check(int64_t M, int64_t N, int64_t K,
 int mi355_gemm_tile_coord(int64_t block, int64_t tiles_m, int64_t tiles_n,
                           int64_t *tile_m, int64_t *tile_n);
 
+/*
+ * Measured ceilings of the GPU the call runs on, for a benchmark's roofline line.  No counterpart
+ * in the reference, whose benchmark reads the peak from a table (kernels/tests/gemm_bench.py:592-599).
+ *
+ * mi355_calibrate_mfma enqueues ONE launch of a kernel that does nothing but matrix-core work: one
+ * workgroup of four waves per compute unit, every wave running the tile kernel's MFMA pattern
+ * (v_mfma_f32_16x16x32 for MI355_BF16 / MI355_F16, v_mfma_f32_16x16x128_f8f6f4 for MI355_E4M3;
+ * 64 accumulator blocks) `iters` times on operand fragments it loads once from `a` and `b` (any
+ * device data of that type, e.g. the operands of the GEMM being measured: the sustained clock
+ * depends on the data; at least 4096 bytes each, 32-byte aligned).  *flops receives the flop count
+ * of the launch; the caller times it.  `sink` is device memory of mi355_calibrate_sink_bytes().
+ *
+ * mi355_calibrate_read enqueues one launch that reads `bytes` bytes at `src` (16-byte aligned)
+ * with plain 16-byte loads and nothing else.
+ */
+size_t mi355_calibrate_sink_bytes(void);
+int mi355_calibrate_mfma(int in_dtype, const void *a, size_t a_bytes, const void *b, size_t b_bytes,
+                         int iters, void *sink, double *flops, void *stream);
+int mi355_calibrate_read(const void *src, size_t bytes, void *sink, void *stream);
+
 /* Human-readable text for a status code; never NULL.  Replaces the TORCH_CHECK messages of
  * gemm_test.cu:15-41 and the stderr print of :88-90. */
 const char *mi355_gemm_strerror(int status);

@@ -55,6 +55,12 @@ def load():
     L.mi355_gemm_check.restype = ci
     L.mi355_gemm_tile_coord.argtypes = [i64, i64, i64, ctypes.POINTER(i64), ctypes.POINTER(i64)]
     L.mi355_gemm_tile_coord.restype = ci
+    L.mi355_calibrate_sink_bytes.argtypes = []
+    L.mi355_calibrate_sink_bytes.restype = sz
+    L.mi355_calibrate_mfma.argtypes = [ci, vp, sz, vp, sz, ci, vp, ctypes.POINTER(ctypes.c_double), vp]
+    L.mi355_calibrate_mfma.restype = ci
+    L.mi355_calibrate_read.argtypes = [vp, sz, vp, vp]
+    L.mi355_calibrate_read.restype = ci
     L.mi355_gemm_strerror.argtypes = [ci]
     L.mi355_gemm_strerror.restype = ctypes.c_char_p
     L.mi355_gemm_version.argtypes = []

@@ -1,0 +1,68 @@
+"""The shape-sweep harness (cute-examples_amd/gemm_bench.py, the counterpart of the reference's
+kernels/tests/gemm_bench.py) runs end to end on its two smallest shapes: both implementations are
+timed with both protocols, they agree on the same operands, and the summary table and the JSON file
+come out."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_gemm_bench_two_smallest_shapes(tmp_path):
+    out = tmp_path / "sweep.json"
+    env = dict(os.environ, PYTHONPATH=os.path.join(ROOT, "cute-examples_amd"))
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "cute-examples_amd", "gemm_bench.py"), "--runs", "3",
+                           "--shapes", "1024x1024,2048x2048", "--out", str(out)],
+                          capture_output=True, text=True, env=env, timeout=300)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+    assert "PERFORMANCE SUMMARY" in proc.stdout and "1024x1024" in proc.stdout and "2048x2048" in proc.stdout
+    data = json.loads(out.read_text())
+    assert data["comparator"].startswith("torch.mm") and len(data["rows"]) == 2
+    for row in data["rows"]:
+        assert row["rel_diff"] <= 1e-2, row                     # ours and torch.mm on the same operands
+        for key in ("ours_wall_ms", "blas_wall_ms", "ours_event_ms", "blas_event_ms"):
+            assert 0.0 < row[key] < 1e3, (key, row)
+        assert row["ours_tflops"] > 1.0 and row["blas_tflops"] > 1.0
+
+
+def test_calibration_kernels_run_and_report_plausible_ceilings(abi):
+    """mi355_calibrate_mfma / mi355_calibrate_read through the C ABI: they launch, write their sink,
+    and the rates they give are those of a GPU (above 100 TFLOP/s and 1 TB/s) and below the published
+    peaks.  Argument errors come back before any launch."""
+    import ctypes
+    import torch
+    from tests import abi_ctypes as ac
+
+    sink = torch.zeros(abi.mi355_calibrate_sink_bytes(), dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    flops = ctypes.c_double()
+    assert abi.mi355_calibrate_mfma(ac.BF16, None, 4096, None, 4096, 10, sink.data_ptr(), ctypes.byref(flops), stream) == ac.ERR_NULL
+    for code, dt, peak in ((ac.BF16, torch.bfloat16, 2500.0), (ac.E4M3, torch.float8_e4m3fn, 5000.0)):
+        A = torch.randn(1024, 1024, device="cuda").to(dt)
+        B = torch.randn(1024, 1024, device="cuda").to(dt)
+        nbytes = A.numel() * A.element_size()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for timed in (False, True):
+            e0.record()
+            rc = abi.mi355_calibrate_mfma(code, A.data_ptr(), nbytes, B.data_ptr(), nbytes, 2000, sink.data_ptr(),
+                                          ctypes.byref(flops), stream)
+            e1.record()
+            assert rc == ac.OK
+            torch.cuda.synchronize()
+        tflops = flops.value / e0.elapsed_time(e1) / 1e9
+        assert 100.0 < tflops <= 1.02 * peak, tflops
+    src = torch.empty(1 << 28, dtype=torch.uint8, device="cuda")
+    src.view(torch.int32).random_()
+    for timed in (False, True):
+        e0.record()
+        assert abi.mi355_calibrate_read(src.data_ptr(), src.numel(), sink.data_ptr(), stream) == ac.OK
+        e1.record()
+        torch.cuda.synchronize()
+    gbs = src.numel() / e0.elapsed_time(e1) / 1e6
+    assert 1000.0 < gbs, gbs

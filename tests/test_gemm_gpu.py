@@ -144,10 +144,8 @@ def test_reference_test_shapes_bf16_randn(abi, size, variant):
     C = run_abi(abi, A, B, variant)
     err, ref = check(C, A, B)
     assert err < 4e-3  # bf16 output rounding alone is ~1.7e-3
-    # The reference asserts allclose(atol=1e-2, rtol=1e-2) on N(0,1) inputs; with |C| up to
-    # ~5*sqrt(K) a correctly rounded bf16 result misses rtol=1e-2 only through bf16's own
-    # 2^-9 spacing, so the check is applied to the rounding-free part: C vs bf16(ref).
-    assert oracle.reference_accepts(C, ref.bfloat16())
+    # gemm_test.py:10, :36 as written: allclose(atol=1e-2, rtol=1e-2) against the fp32 product
+    assert oracle.reference_accepts(C, ref)
 
 
 @pytest.mark.parametrize("variant", TILED)
@@ -764,7 +762,8 @@ def test_python_module_is_the_reference_call(abi):
     C.fill_(float("nan"))
     out = gemm_tn_test(A, B, C)
     assert out.data_ptr() == C.data_ptr()
-    check(C, A, B)
+    err, ref = check(C, A, B)
+    assert oracle.reference_accepts(C, ref)   # gemm_test.py:10 against the fp32 product of :36
 
 
 def test_python_module_repacks_odd_shapes():
