@@ -7,6 +7,8 @@
 #include "gemm_launch.h"
 #include "tile_map.h"
 
+#include <atomic>
+
 namespace {
 
 int elem_bytes(int dtype) { return dtype == MI355_E4M3 ? 1 : 2; }
@@ -121,11 +123,49 @@ bool repack_plan(const void* A, const void* B, const void* C, int64_t M, int64_t
   return tile256_ok(M, r->Np, r->Kp, r->a ? r->ld_ab : lda, r->b ? r->ld_ab : ldb, r->c ? r->ld_c : ldc, in_dtype);
 }
 
+// How a call treats a workspace that is too small for what the plan wants.
+//   kLenient    run without (tiles unsplit, generic kernel instead of repacking, ...), as documented
+//               for mi355_gemm_tn
+//   kStrict     refuse with MI355_ERR_SCRATCH: the workspace is the library's own fixed buffer, and
+//               a caller who cannot allocate should hear that the problem is beyond it
+//   kStrictDry  the same decisions and return codes, stopping before the first HIP call
+enum WorkspaceMode { kLenient, kStrict, kStrictDry };
+
+}  // namespace
+
+// Scratch of mi355_gemm_tn_noalloc: one copy per GPU, held from the moment the code object is
+// loaded on that GPU until the process ends.  In host code this name is only a handle for
+// hipGetSymbolAddress; the device address differs per GPU and is kept in scratch_address[].
+constexpr size_t kScratchBytes = (size_t)MI355_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<void*> scratch_address[kMaxDevices];
+
+// Device address of `scratch` on the current device, looked up once per device.
+int scratch_of_current_device(void** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return MI355_ERR_LAUNCH;
+  void* p = scratch_address[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return MI355_ERR_LAUNCH;
+    scratch_address[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return MI355_OK;
+}
+
+int run_gemm(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+             int64_t ldc, int in_dtype, int out_dtype, float scale, const float* scale_a, const float* scale_b,
+             int variant, void* workspace, size_t workspace_bytes, void* stream, WorkspaceMode mode);
+
 }  // namespace
 
 extern "C" {
 
-int mi355_gemm_version(void) { return (0 << 16) | 1; }
+int mi355_gemm_version(void) { return (0 << 16) | 2; }
 
 const char* mi355_gemm_strerror(int status) {
   switch (status) {
@@ -140,6 +180,10 @@ const char* mi355_gemm_strerror(int status) {
     case MI355_ERR_WORKSPACE: return "workspace is NULL or smaller than mi355_gemm_workspace_bytes()";
     case MI355_ERR_LAUNCH: return "HIP runtime rejected the kernel launch";
     case MI355_ERR_ALIGN: return "A and B must be 16-byte aligned and C 8-byte aligned for the tiled variants";
+    case MI355_ERR_SCRATCH:
+      return "mi355_gemm_tn_noalloc: the problem wants more scratch than the library's built-in buffer of "
+             "MI355_NOALLOC_SCRATCH_BYTES holds; call mi355_gemm_tn with a workspace of "
+             "mi355_gemm_workspace_bytes() instead";
   }
   return "unknown status code";
 }
@@ -375,6 +419,34 @@ int mi355_gemm_tn_scaled(const void* A, const void* B, void* C, int64_t M, int64
                          int64_t lda, int64_t ldb, int64_t ldc, int in_dtype, int out_dtype, float scale,
                          const float* scale_a, const float* scale_b, int variant, void* workspace,
                          size_t workspace_bytes, void* stream) {
+  return run_gemm(A, B, C, M, N, K, lda, ldb, ldc, in_dtype, out_dtype, scale, scale_a, scale_b, variant, workspace,
+                  workspace_bytes, stream, kLenient);
+}
+
+int mi355_gemm_tn_noalloc(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
+                          int64_t lda, int64_t ldb, int64_t ldc, int in_dtype, int out_dtype, float scale,
+                          int variant, void* stream) {
+  // First the whole decision path without a HIP call (argument errors and MI355_ERR_SCRATCH come from
+  // here, so they can be provoked on a machine without a GPU); the stand-in address only has to
+  // be non-null and aligned like the real one.
+  int st = run_gemm(A, B, C, M, N, K, lda, ldb, ldc, in_dtype, out_dtype, scale, nullptr, nullptr, variant,
+                    (void*)(uintptr_t)256, kScratchBytes, stream, kStrictDry);
+  if (st != MI355_OK || M == 0 || N == 0) return st;
+  void* ws = nullptr;
+  st = scratch_of_current_device(&ws);
+  if (st != MI355_OK) return st;
+  return run_gemm(A, B, C, M, N, K, lda, ldb, ldc, in_dtype, out_dtype, scale, nullptr, nullptr, variant, ws,
+                  kScratchBytes, stream, kStrict);
+}
+
+}  // extern "C"
+
+namespace {
+
+int run_gemm(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+             int64_t ldc, int in_dtype, int out_dtype, float scale, const float* scale_a, const float* scale_b,
+             int variant, void* workspace, size_t workspace_bytes, void* stream, WorkspaceMode mode) {
+  const bool strict = mode != kLenient, dry = mode == kStrictDry;
   int st = check_common(M, N, K, lda, ldb, ldc, in_dtype, out_dtype, variant);
   if (st != MI355_OK) return st;
   if (M == 0 || N == 0) return MI355_OK;  // nothing to write
@@ -405,28 +477,31 @@ int mi355_gemm_tn_scaled(const void* A, const void* B, void* C, int64_t M, int64
   }
   if (v == MI355_VARIANT_SIMPLE && variant == MI355_VARIANT_AUTO && workspace && (uintptr_t)workspace % 256 == 0) {
     Repack r;
-    // The streaming kernel insists on the workspace of its K split, so the rest must cover it.
-    const auto inner_ok = [&](const Repack& p) {
-      const size_t rest = workspace_bytes - (p.bytes_a + p.bytes_b + p.bytes_c);
-      return mi355_gemm_select_variant(M, p.Np, p.Kp, in_dtype) != MI355_VARIANT_SKINNY ||
-             rest >= mi355_gemm_workspace_bytes(M, p.Np, p.Kp, in_dtype, MI355_VARIANT_AUTO);
-    };
-    if (repack_plan(A, B, C, M, N, K, lda, ldb, ldc, in_dtype, &r) &&
-        workspace_bytes >= r.bytes_a + r.bytes_b + r.bytes_c && inner_ok(r)) {
-      const int64_t es = elem_bytes(in_dtype);
-      uint8_t* wa = (uint8_t*)workspace;
-      uint8_t* wb = wa + r.bytes_a;
-      uint8_t* wc = wb + r.bytes_b;
-      uint8_t* rest = wc + r.bytes_c;
-      const size_t rest_bytes = workspace_bytes - (r.bytes_a + r.bytes_b + r.bytes_c);
-      if (r.a && mi355::launch_repack_rows(A, M, K * es, lda * es, wa, M, r.ld_ab * es, (int)es, s) != 0) return MI355_ERR_LAUNCH;
-      if (r.b && mi355::launch_repack_rows(B, N, K * es, ldb * es, wb, r.Np, r.ld_ab * es, (int)es, s) != 0) return MI355_ERR_LAUNCH;
-      st = mi355_gemm_tn_scaled(r.a ? wa : A, r.b ? wb : B, r.c ? (void*)wc : C, M, r.Np, r.Kp, r.a ? r.ld_ab : lda,
-                                r.b ? r.ld_ab : ldb, r.c ? r.ld_c : ldc, in_dtype, out_dtype, scale, scale_a, scale_b,
-                                MI355_VARIANT_AUTO, rest_bytes ? rest : nullptr, rest_bytes, stream);
-      if (st != MI355_OK) return st;
-      if (r.c && mi355::launch_copy_out(wc, M, N, r.ld_c, C, ldc, s) != 0) return MI355_ERR_LAUNCH;
-      return MI355_OK;
+    if (repack_plan(A, B, C, M, N, K, lda, ldb, ldc, in_dtype, &r)) {
+      const size_t packed = r.bytes_a + r.bytes_b + r.bytes_c;
+      // What the repacked (aligned) problem wants for its own splits.  The streaming kernel insists
+      // on the workspace of its K split, so a lenient call repacks only when the rest covers it.
+      const size_t inner = mi355_gemm_workspace_bytes(M, r.Np, r.Kp, in_dtype, MI355_VARIANT_AUTO);
+      const bool inner_streams = mi355_gemm_select_variant(M, r.Np, r.Kp, in_dtype) == MI355_VARIANT_SKINNY;
+      const bool fits = workspace_bytes >= packed && (workspace_bytes - packed >= inner || (!strict && !inner_streams));
+      if (strict && !fits) return MI355_ERR_SCRATCH;
+      if (fits) {
+        if (dry) return MI355_OK;
+        const int64_t es = elem_bytes(in_dtype);
+        uint8_t* wa = (uint8_t*)workspace;
+        uint8_t* wb = wa + r.bytes_a;
+        uint8_t* wc = wb + r.bytes_b;
+        uint8_t* rest = wc + r.bytes_c;
+        const size_t rest_bytes = workspace_bytes - packed;
+        if (r.a && mi355::launch_repack_rows(A, M, K * es, lda * es, wa, M, r.ld_ab * es, (int)es, s) != 0) return MI355_ERR_LAUNCH;
+        if (r.b && mi355::launch_repack_rows(B, N, K * es, ldb * es, wb, r.Np, r.ld_ab * es, (int)es, s) != 0) return MI355_ERR_LAUNCH;
+        st = run_gemm(r.a ? wa : A, r.b ? wb : B, r.c ? (void*)wc : C, M, r.Np, r.Kp, r.a ? r.ld_ab : lda,
+                      r.b ? r.ld_ab : ldb, r.c ? r.ld_c : ldc, in_dtype, out_dtype, scale, scale_a, scale_b,
+                      MI355_VARIANT_AUTO, rest_bytes ? rest : nullptr, rest_bytes, stream, mode);
+        if (st != MI355_OK) return st;
+        if (r.c && mi355::launch_copy_out(wc, M, N, r.ld_c, C, ldc, s) != 0) return MI355_ERR_LAUNCH;
+        return MI355_OK;
+      }
     }
   }
   int rc;
@@ -437,10 +512,12 @@ int mi355_gemm_tn_scaled(const void* A, const void* B, void* C, int64_t M, int64
   const int stream_s = v == MI355_VARIANT_SKINNY ? mi355::stream_splits(M, N, K, elem_bytes(in_dtype)) : 1;
   const size_t stream_need = stream_s > 1 ? (size_t)stream_s * (size_t)M * (size_t)N * sizeof(float) : 0;
   if (stream_need && (!workspace || workspace_bytes < stream_need || (uintptr_t)workspace % 16 != 0)) {
+    if (strict) return MI355_ERR_SCRATCH;
     if (variant != MI355_VARIANT_AUTO) return MI355_ERR_WORKSPACE;
     v = MI355_VARIANT_BASIC;   // whatever the streaming kernel takes the tile kernel takes too
   }
   if (v == MI355_VARIANT_SKINNY) {
+    if (dry) return MI355_OK;
     const int splits = stream_s;
     g.tiles_m = g.tiles_n = 0;
     rc = mi355::launch_stream(g, in_dtype, out_dtype, splits, workspace, s);
@@ -448,31 +525,38 @@ int mi355_gemm_tn_scaled(const void* A, const void* B, void* C, int64_t M, int64
     const int tile = v == MI355_VARIANT_PINGPONG ? 256 : mi355::ring_tile_edge(M, N, K, elem_bytes(in_dtype));
     if (v == MI355_VARIANT_BASIC) {
       // Both kinds of K split are optional for this kernel: without a (large enough, aligned)
-      // workspace the same tiles run unsplit, slower but with the same result contract.
+      // workspace a lenient call runs the same tiles unsplit, slower but with the same result contract.
       const auto usable = [&](size_t need) {
         return need && workspace && workspace_bytes >= need && (uintptr_t)workspace % 16 == 0;
       };
       const int splits = mi355::ring_splits(M, N, K, elem_bytes(in_dtype));
       g.partial = (float*)workspace;
       if (splits > 1) {
-        if (usable((size_t)splits * (size_t)M * (size_t)N * sizeof(float))) g.splits = splits;
+        const size_t need = (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
+        if (usable(need)) g.splits = splits;
+        else if (strict) return MI355_ERR_SCRATCH;
       } else {
         int tail_tiles, tail_splits;
-        if (usable(mi355::ring_tail(M, N, K, elem_bytes(in_dtype), &tail_tiles, &tail_splits))) {
+        const size_t need = mi355::ring_tail(M, N, K, elem_bytes(in_dtype), &tail_tiles, &tail_splits);
+        if (usable(need)) {
           g.tail_tiles = tail_tiles;
           g.tail_splits = tail_splits;
+        } else if (strict && need) {
+          return MI355_ERR_SCRATCH;
         }
       }
     }
+    if (dry) return MI355_OK;
     g.tiles_m = (M + mi355::ring_tile_rows(tile) - 1) / mi355::ring_tile_rows(tile);
     g.tiles_n = (N + mi355::ring_tile_cols(tile) - 1) / mi355::ring_tile_cols(tile);
     rc = v == MI355_VARIANT_PINGPONG ? mi355::launch_tile256_pingpong(g, in_dtype, out_dtype, s)
                                      : mi355::launch_tile_ring(g, in_dtype, out_dtype, tile, s);
   } else {
+    if (dry) return MI355_OK;
     g.tiles_m = g.tiles_n = 0;
     rc = mi355::launch_simple(g, in_dtype, out_dtype, s);
   }
   return rc == 0 ? MI355_OK : MI355_ERR_LAUNCH;
 }
 
-}  // extern "C"
+}  // namespace

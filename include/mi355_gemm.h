@@ -50,7 +50,8 @@ enum mi355_status {
   MI355_ERR_VARIANT = -4,   /* unknown variant, or variant cannot run this shape/dtype      */
   MI355_ERR_WORKSPACE = -5, /* workspace missing or smaller than mi355_gemm_workspace_bytes */
   MI355_ERR_LAUNCH = -6,    /* the HIP runtime refused the launch                           */
-  MI355_ERR_ALIGN = -7      /* a pointer or leading dimension is not 16-byte aligned        */
+  MI355_ERR_ALIGN = -7,     /* a pointer or leading dimension is not 16-byte aligned        */
+  MI355_ERR_SCRATCH = -8    /* mi355_gemm_tn_noalloc: the problem is beyond the built-in scratch */
 };
 
 /*
@@ -102,6 +103,36 @@ int mi355_gemm_tn_scaled(const void *A, const void *B, void *C,
                          int in_dtype, int out_dtype, float scale,
                          const float *scale_a, const float *scale_b, int variant,
                          void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * mi355_gemm_tn for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the same computation, kernels and plan,
+ * with the workspace replaced by a buffer of MI355_NOALLOC_SCRATCH_BYTES that is part of the
+ * library's code object.  The call allocates and frees nothing and hands over no workspace.
+ * No counterpart in the reference (its launcher, kernels/gemm_kernels/sm90a/gemm_test.cu:12-92,
+ * has no workspace at all).
+ *
+ *   - Each GPU the library runs on holds its own copy of the buffer from the first use of the
+ *     library on that GPU until the process ends.  Its address on a GPU is looked up on the first
+ *     call made with that GPU current (no allocation, but a one-time runtime query: make one call
+ *     outside a graph capture first).
+ *   - A problem whose plan wants more than the buffer holds is refused with MI355_ERR_SCRATCH; it
+ *     is never silently run on a slower path.  K-split partial planes and tail-split partial tiles
+ *     always fit (a plan has at most 256 split items of at most 256 x 256 floats = 64 MiB), and
+ *     problems that want no workspace have no size limit, so in practice the limit applies to the
+ *     repacked operands of a large misaligned problem (K*elem_bytes % 16, N % 4, strides, pointers;
+ *     mi355_gemm_workspace_bytes reports the figure for contiguous operands).
+ *   - All calls on one GPU share that GPU's buffer, which keeps the last call's contents (nothing
+ *     in it needs to start at zero).  Calls that may overlap on one GPU (different streams, or
+ *     several host threads) race on it: serialise them, or use mi355_gemm_tn with a workspace each.
+ * Argument checks and their status codes are those of mi355_gemm_tn and run before any HIP call.
+ */
+#define MI355_NOALLOC_SCRATCH_BYTES 67108864 /* 64 MiB */
+int mi355_gemm_tn_noalloc(const void *A, const void *B, void *C,
+                          int64_t M, int64_t N, int64_t K,
+                          int64_t lda, int64_t ldb, int64_t ldc,
+                          int in_dtype, int out_dtype, float scale, int variant,
+                          void *stream);
 
 /*
  * Per-tensor fp8 quantisation, the step in front of the fp8 GEMM: amax = max|x|,

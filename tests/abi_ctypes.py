@@ -10,7 +10,8 @@ HEADER = os.path.join(ROOT, "include", "mi355_gemm.h")
 
 BF16, F16, E4M3, F32 = 0, 1, 2, 3
 AUTO, BASIC, PINGPONG, SKINNY, SIMPLE = 0, 1, 2, 3, 4
-OK, ERR_NULL, ERR_DTYPE, ERR_SHAPE, ERR_VARIANT, ERR_WORKSPACE, ERR_LAUNCH, ERR_ALIGN = 0, -1, -2, -3, -4, -5, -6, -7
+OK, ERR_NULL, ERR_DTYPE, ERR_SHAPE, ERR_VARIANT, ERR_WORKSPACE, ERR_LAUNCH, ERR_ALIGN, ERR_SCRATCH = 0, -1, -2, -3, -4, -5, -6, -7, -8
+NOALLOC_SCRATCH_BYTES = 64 << 20
 
 
 def declared_symbols():
@@ -29,6 +30,8 @@ def load():
     L.mi355_gemm_tn.restype = ci
     L.mi355_gemm_tn_scaled.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, f32, vp, vp, ci, vp, sz, vp]
     L.mi355_gemm_tn_scaled.restype = ci
+    L.mi355_gemm_tn_noalloc.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, f32, ci, vp]
+    L.mi355_gemm_tn_noalloc.restype = ci
     L.mi355_quantize_e4m3.argtypes = [vp, ci, i64, vp, vp, vp]
     L.mi355_quantize_e4m3.restype = ci
     u8p = vp
@@ -86,6 +89,16 @@ def gemm_tn(L, A, B, C, scale=1.0, variant=AUTO, stream=None):
                          C.stride(0), in_dt, out_dt, scale, variant,
                          ws.data_ptr() if ws is not None else None, ws_bytes, s)
     return rc
+
+
+def gemm_tn_noalloc(L, A, B, C, scale=1.0, variant=AUTO, stream=None):
+    """Call mi355_gemm_tn_noalloc on torch device tensors: no workspace crosses the boundary."""
+    import torch
+    M, K = A.shape
+    N = B.shape[0]
+    s = stream if stream is not None else torch.cuda.current_stream().cuda_stream
+    return L.mi355_gemm_tn_noalloc(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, A.stride(0), B.stride(0),
+                                   C.stride(0), torch_code(A.dtype), torch_code(C.dtype), scale, variant, s)
 
 
 def gemm_tn_mxfp8(L, A_q, B_q, sa, sb, C, shuffled=False, stream=None):

@@ -311,3 +311,25 @@ def test_plan_invariants_over_random_shapes(abi):
                 seen.add((rows, cols, splits > 1, tail_tiles > 0))
             assert abi.mi355_gemm_workspace_bytes(M, N, K, dt, ac.AUTO) == want, (M, N, K)
     assert len(seen) >= 7, seen
+
+
+def test_noalloc_entry_point_decides_before_any_hip_call(abi):
+    """mi355_gemm_tn_noalloc runs its argument checks and the does-it-fit decision before it touches
+    the device, so both can be provoked here: the pointers only need to look aligned."""
+    p = 1 << 20
+    f = abi.mi355_gemm_tn_noalloc
+    assert f(None, p, p, 256, 256, 64, 64, 64, 256, ac.BF16, ac.BF16, 1.0, ac.AUTO, None) == ac.ERR_NULL
+    assert f(p, p, p, 256, 256, 64, 32, 64, 256, ac.BF16, ac.BF16, 1.0, ac.AUTO, None) == ac.ERR_SHAPE
+    assert f(p, p, p, 256, 256, 64, 64, 64, 256, ac.BF16, ac.BF16, 1.0, 9, None) == ac.ERR_VARIANT
+    assert f(p, p, p, 0, 256, 64, 64, 64, 256, ac.BF16, ac.BF16, 1.0, ac.AUTO, None) == ac.OK      # nothing to do
+    # a misaligned problem whose repacked operands (400 MB) are beyond the 64 MiB buffer
+    assert abi.mi355_gemm_workspace_bytes(8191, 8193, 8190, ac.BF16, ac.AUTO) > ac.NOALLOC_SCRATCH_BYTES
+    assert f(p, p, p, 8191, 8193, 8190, 8190, 8190, 8193, ac.BF16, ac.BF16, 1.0, ac.AUTO, None) == ac.ERR_SCRATCH
+    assert b"MI355_NOALLOC_SCRATCH_BYTES" in abi.mi355_gemm_strerror(ac.ERR_SCRATCH)
+    # split partials never exceed the buffer: at most 256 split items of at most 256 x 256 floats
+    import random
+    rng = random.Random(11)
+    for _ in range(2000):
+        M, N, K = rng.randint(1, 20000), 4 * rng.randint(1, 8000), 16 * rng.randint(1, 2048)   # aligned: no repacking
+        for dt in (ac.BF16, ac.E4M3):
+            assert abi.mi355_gemm_workspace_bytes(M, N, K, dt, ac.AUTO) <= ac.NOALLOC_SCRATCH_BYTES, (M, N, K, dt)
