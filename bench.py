@@ -406,6 +406,14 @@ def main():
     if fp8_block and fp8_cpu_operands:
         fp8_block["cpu_baseline"] = cpu_baseline(*fp8_cpu_operands, budget_s=8.0, native_budget_s=0.0)
 
+    if fp8_block:
+        # the second configuration of the metric in brief, beside the headline's roofline
+        r8 = fp8_block["roofline"]
+        roof["fp8_8192"] = {"value": fp8_block["value"], "unit": "TFLOP/s", "ms_per_step": fp8_block["ms_per_step"],
+                            "peak": r8["peak"], "frac": r8["frac"], "traffic": r8["traffic"],
+                            "measured_mfma_ceiling": (r8.get("measured_mfma_ceiling") or {}).get("value"),
+                            "cpu_baseline_value": (fp8_block["cpu_baseline"] or {}).get("value"),
+                            "see": "the top-level \"fp8\" object of this line"}
     out = {
         "metric": METRIC, "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "settle_launches": head["settle_launches"], "settle_ms": head["settle_ms"],
@@ -415,7 +423,7 @@ def main():
                                % (a.workload, head["M"], head["N"], head["K"]),
                    "variant": roof["kernel"], "parallelism": "single GPU"},
         "pct_of_dense_mfma_peak": head["pct_mfma_peak"],
-        "roofline": roof, "cpu_baseline": cpu, "fp8": fp8_block, "extras": extras,
+        "roofline": roof, "cpu_baseline": cpu, "extras": extras, "fp8": fp8_block,
     }
     print(json.dumps(out))
 

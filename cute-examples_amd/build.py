@@ -23,6 +23,9 @@ HIP_SOURCES = ["gemm_api.hip", "gemm_tn_simple.hip", "gemm_tn_ring_bf16.hip", "g
 # LDS base in all of them, the asynchronous scale loads in the block-scaled one.
 CHECKED_SOURCES = ["gemm_tn_ring_bf16.hip", "gemm_tn_ring_f16.hip", "gemm_tn_ring_e4m3.hip", "gemm_tn_ring_mx.hip"]
 CHECKED_SOURCE = "gemm_tn_ring_mx.hip"
+# Sources whose kernels must keep the hardware's distances the compiler does not enforce (wide
+# stores and their data registers, inline-assembly MFMAs and their results): every GEMM kernel.
+HAZARD_SOURCES = CHECKED_SOURCES + ["gemm_tn_pingpong.hip", "gemm_tn_stream.hip", "calibrate.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -56,7 +59,7 @@ def build_lib():
     with tempfile.TemporaryDirectory() as tmp:
         def compile_one(src):
             obj = os.path.join(tmp, src.replace(".hip", ".o"))
-            extra = ["-save-temps=obj"] if src in CHECKED_SOURCES else []
+            extra = ["-save-temps=obj"] if src in HAZARD_SOURCES else []
             _run([hipcc] + HIPCC_FLAGS + ["-c"] + extra + ["-o", obj, os.path.join(CSRC, src)])
             return obj
 
@@ -71,6 +74,16 @@ def build_lib():
             if src == CHECKED_SOURCE:
                 print("check_async_loads: %d scale operands ok" % check_async_loads.check(asm[0]), flush=True)
         print("check_async_loads: %d direct-to-LDS copies ok" % copies, flush=True)
+        stores = mfmas = 0
+        for src in HAZARD_SOURCES:
+            asm = glob.glob(os.path.join(tmp, src.replace(".hip", "") + "-hip-amdgcn-*gfx950.s"))
+            if len(asm) != 1:
+                raise RuntimeError("expected one device assembly file for %s, found %r" % (src, asm))
+            n_st, n_mf = check_async_loads.check_hazard_distances(asm[0])
+            stores, mfmas = stores + n_st, mfmas + n_mf
+        print("check_async_loads: %d stores keep their data registers for %d wait states, %d inline MFMAs keep their "
+              "results untouched for %d" % (stores, check_async_loads.STORE_DATA_WINDOW, mfmas,
+                                             check_async_loads.MFMA_RESULT_WINDOW), flush=True)
         _run([hipcc] + HIPCC_FLAGS + ["-o", LIB] + objs)
     return LIB
 

@@ -117,6 +117,33 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(uintptr_t)p;
 }
 
+// Store data and the registers that hold it.  A vector-memory store of more than 8 bytes per lane
+// reads its data registers over several cycles after it has issued, and the ISA asks for idle wait
+// states between such a store and the next write of those registers.  The compiler provides them
+// only for stores without a scalar offset register; the stores here have one.  With nothing in
+// between, a few lanes of a store's first data register were seen to carry the NEXT store's value.
+// So the code keeps the hazard from arising instead of waiting it out: the data registers of store
+// n stay live, untouched, until the data of store n + 2 is complete (hold_previous names the new
+// data and that of the two stores before it in one empty assembly statement, which the compiler
+// can neither move in front of the conversion that produces the new data nor behind the store that
+// consumes it, and a scheduling barrier behind every store keeps the next conversion from being
+// hoisted above it), so the conversions of blocks n + 1 and n + 2 cannot be given the registers of
+// store n, and three register sets rotate.  The first write into the registers of store n is then
+// two whole conversions away (ten to thirty instructions each, depending on the kernel).
+// check_async_loads.check_hazard_distances verifies exactly that in the generated assembly of every
+// build: no write of a store's data registers within 12 wait states, on any path.
+template <class V>
+__device__ __forceinline__ void hold_previous(V& current, const V& previous, const V& before) {
+  asm volatile("" : "+v"(current) : "v"(previous), "v"(before));
+}
+// Where no conversion follows a store -- the last store of a tile, and the fp32 partial tiles of a
+// K split, whose data is the accumulator registers themselves -- the data registers are held over
+// idle wait states instead: the wait states the ISA asks for, counted, not a delay tuned by trial.
+template <class V>
+__device__ __forceinline__ void hold_last(const V& last) {
+  asm volatile("s_nop 11" ::"v"(last) : "memory");
+}
+
 // Four fp32 -> four 16-bit values (round to nearest even), packed into 8 bytes.
 template <class OutT> struct Pack4;
 template <> struct Pack4<BF16> {

@@ -215,12 +215,19 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
     for (int j = 0; j < kNB; ++j) {
       const int64_t n = n0 + (wn * kNB + j) * 16 + grp * 4;
       if (n + 4 > g.N) continue;
+      // A wave has at most sixteen of these stores: each one's data registers are simply held over
+      // the wait states a wide store wants before they may be rewritten (see hold_previous).
       if (partial) {
-        *(f32x4*)(partial + ((int64_t)split * g.M + m) * g.N + n) = acc[i][j];
+        u32x4 data = __builtin_bit_cast(u32x4, acc[i][j]);
+        asm volatile("" : "+v"(data));
+        *(u32x4*)(partial + ((int64_t)split * g.M + m) * g.N + n) = data;
+        hold_last(data);
       } else {
         const float sc = output_scale(g);
-        *(u32x2*)((uint16_t*)g.C + m * g.ldc + n) =
-            Pack4<OutT>::run(acc[i][j][0] * sc, acc[i][j][1] * sc, acc[i][j][2] * sc, acc[i][j][3] * sc);
+        u32x2 data = Pack4<OutT>::run(acc[i][j][0] * sc, acc[i][j][1] * sc, acc[i][j][2] * sc, acc[i][j][3] * sc);
+        asm volatile("" : "+v"(data));
+        *(u32x2*)((uint16_t*)g.C + m * g.ldc + n) = data;
+        hold_last(data);
       }
     }
   }

@@ -20,18 +20,6 @@ namespace mi355 {
 
 constexpr uint32_t kStoreOutOfRange = 0x80000000u;  // tiles of C span less than 2 GiB (host check)
 
-// A 16-byte buffer store followed by idle cycles.  The store reads its four data registers a few
-// cycles after it issues; the instructions that refill them for the next store come right behind
-// it, and with only the compiler's two wait states in between (as s_nop) a few lanes of the first
-// register were seen to pick up the new value.  Eight idle cycles per store are below measurement.
-// kAux: cache-policy bits of the store (1 = sc0, 2 = nt, 16 = sc1).
-template <int kAux>
-__device__ __forceinline__ void store_16B_guarded(u32x4 data, __amdgpu_buffer_rsrc_t rsrc, uint32_t voffset,
-                                                  uint32_t soffset) {
-  __builtin_amdgcn_raw_buffer_store_b128(data, rsrc, voffset, soffset, kAux);
-  asm volatile("s_nop 7");
-}
-
 // Called on an accumulator block right before it is read element by element.  kPinned: the kernel's
 // MFMAs are inline assembly on accumulation registers; the empty statement here keeps the block in
 // those registers up to this point of the program, so the register allocator moves it to VGPRs
@@ -107,19 +95,33 @@ __device__ __forceinline__ void store_output_tile(typename G::Acc (&acc)[kNbM][k
     });
   };
   if (cols == (uint32_t)tile_cols) {
+    u32x4 previous = {0u, 0u, 0u, 0u}, before = {0u, 0u, 0u, 0u};
     convert([&](auto ic, auto colc, u32x2 x, u32x2 y) __attribute__((always_inline)) {
       constexpr int i = decltype(ic)::value, col = decltype(colc)::value;
-      store_16B_guarded<kAux>((u32x4){x[0], x[1], y[0], y[1]}, rc, v0 + col * 2, i * block_step);
+      u32x4 data = {x[0], x[1], y[0], y[1]};
+      hold_previous(data, previous, before);
+      __builtin_amdgcn_raw_buffer_store_b128(data, rc, v0 + col * 2, i * block_step, kAux);
+      MI355_FENCE();   // the next block's conversion stays behind this store
+      before = previous;
+      previous = data;
     });
+    hold_last(previous);
   } else {
     // N is a multiple of 4 (host check), so each half of the 8 columns is in or out as a whole.
+    u32x4 previous = {0u, 0u, 0u, 0u}, before = {0u, 0u, 0u, 0u};
     convert([&](auto ic, auto colc, u32x2 x, u32x2 y) __attribute__((always_inline)) {
       constexpr int i = decltype(ic)::value, col = decltype(colc)::value;
       const uint32_t vx = col0 + col + 4 <= cols ? v0 + col * 2 : kStoreOutOfRange;
       const uint32_t vy = col0 + col + 8 <= cols ? v0 + col * 2 + 8 : kStoreOutOfRange;
-      __builtin_amdgcn_raw_buffer_store_b64(x, rc, vx, i * block_step, 0);
-      __builtin_amdgcn_raw_buffer_store_b64(y, rc, vy, i * block_step, 0);
+      u32x4 data = {x[0], x[1], y[0], y[1]};
+      hold_previous(data, previous, before);
+      __builtin_amdgcn_raw_buffer_store_b64((u32x2){data[0], data[1]}, rc, vx, i * block_step, 0);
+      __builtin_amdgcn_raw_buffer_store_b64((u32x2){data[2], data[3]}, rc, vy, i * block_step, 0);
+      MI355_FENCE();
+      before = previous;
+      previous = data;
     });
+    hold_last(previous);
   }
 }
 
@@ -147,8 +149,11 @@ __device__ __forceinline__ void store_partial_tile(typename G::Acc (&acc)[kNbM][
       if constexpr (q == 0) pin_acc_block<kAsmRead>(acc[i][j]);
       const typename G::Acc& c = acc[i][j];
       const f32x4 quad = {c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
+      u32x4 data = __builtin_bit_cast(u32x4, quad);
+      asm volatile("" : "+v"(data));   // the store reads these registers, the ones hold_last then holds
       // write-through: the partials are read back by another kernel, not by this one (+8 % measured)
-      store_16B_guarded<16>(__builtin_bit_cast(u32x4, quad), rp, v, i * block_step);
+      __builtin_amdgcn_raw_buffer_store_b128(data, rp, v, i * block_step, 16);
+      hold_last(data);   // 12 idle cycles per store: this path runs once per split item, not per k-step
     });
   });
 }

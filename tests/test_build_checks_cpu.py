@@ -174,3 +174,53 @@ def test_lds_base_check_accepts_a_write_one_mfma_ahead(tmp_path):
 def test_lds_base_check_rejects(tmp_path, body, msg):
     with pytest.raises(RuntimeError, match=msg):
         run_lds(tmp_path, body)
+
+
+# ---------------------------------------------------------------- store-data and MFMA-result distances
+
+K_HEAD = "_ZN5mi3554demoEv: ; @kernel\n"
+STORE = "\tbuffer_store_dwordx4 v[0:3], v150, s[20:23], s86 offen nt sc1\n"
+FILL = "\tv_add_u32_e32 v100, v101, v102\n"
+ASM_MFMA = "\t;;#ASMSTART\n\tv_mfma_f32_16x16x32_bf16 a[0:3], v[2:5], v[6:9], a[0:3]\n\t;;#ASMEND\n"
+
+
+def run_hazards(tmp_path, body):
+    f = tmp_path / "h.s"
+    f.write_text(K_HEAD + body + TAIL)
+    return check_async_loads.check_hazard_distances(str(f))
+
+
+def test_store_data_may_be_rewritten_after_the_window(tmp_path):
+    w = check_async_loads.STORE_DATA_WINDOW
+    assert run_hazards(tmp_path, STORE + FILL * w + "\tv_mov_b32_e32 v0, v9\n") == (1, 0)
+    assert run_hazards(tmp_path, STORE + "\ts_nop %d\n" % (w - 1) + "\tv_mov_b32_e32 v3, v9\n") == (1, 0)
+    # the address register and unrelated registers are free at once
+    assert run_hazards(tmp_path, STORE + "\tv_mov_b32_e32 v150, v9\n\tv_mov_b32_e32 v4, v9\n") == (1, 0)
+
+
+@pytest.mark.parametrize("body", [
+    STORE + FILL * 3 + "\tv_accvgpr_read_b32 v0, a248\n",                                  # a plain write, too early
+    STORE + "\ts_nop 7\n" + "\tv_cvt_pk_bf16_f32 v2, v4, v5\n",                               # eight idle cycles are not twelve
+    STORE + FILL * 2 + "\tv_permlane16_swap_b32_e32 v9, v1\n",                              # the swap writes both operands
+    STORE + FILL * 2 + "\ts_cbranch_scc1 .LBB0_2\n" + FILL * 20 + ".LBB0_2:\n\tv_mov_b32_e32 v1, v9\n",   # on the taken path
+    STORE + FILL * 2 + "\ts_branch .LBB0_3\n.LBB0_3:\n\tds_read_b128 v[0:3], v123\n",
+    "\tglobal_store_dwordx4 v[4:5], v[8:11], off\n" + FILL + "\tv_mov_b32_e32 v10, v9\n",   # data is the second operand there
+    "\tbuffer_store_dwordx2 v[2:3], v0, s[20:23], 0 offen\n" + FILL * 4 + "\tv_mov_b32_e32 v2, v9\n",
+])
+def test_store_data_rewritten_too_early_is_rejected(tmp_path, body):
+    with pytest.raises(RuntimeError, match="rewrites data of"):
+        run_hazards(tmp_path, body)
+
+
+def test_inline_mfma_results_are_left_alone_for_the_window(tmp_path):
+    w = check_async_loads.MFMA_RESULT_WINDOW
+    # accumulating in place into exactly the same registers is what the hardware is built for
+    assert run_hazards(tmp_path, ASM_MFMA + ASM_MFMA + FILL * w + "\tv_accvgpr_read_b32 v0, a0\n") == (0, 2)
+    with pytest.raises(RuntimeError, match="touches the result of"):
+        run_hazards(tmp_path, ASM_MFMA + FILL * 5 + "\tv_accvgpr_read_b32 v0, a2\n")
+    with pytest.raises(RuntimeError, match="touches the result of"):
+        run_hazards(tmp_path, ASM_MFMA + FILL * 5 + "\tbuffer_store_dwordx4 a[0:3], v1, s[20:23], 0 offen\n")
+    with pytest.raises(RuntimeError, match="touches the result of"):     # an overlapping, not identical, accumulator
+        run_hazards(tmp_path, ASM_MFMA + "\t;;#ASMSTART\n\tv_mfma_f32_16x16x32_bf16 a[2:5], v[2:5], v[6:9], a[2:5]\n\t;;#ASMEND\n")
+    # MFMAs the compiler emitted itself get their wait states from the compiler: not this check's business
+    assert run_hazards(tmp_path, "\tv_mfma_f32_16x16x32_bf16 v[0:3], v[12:15], v[16:19], v[0:3]\n\tv_mov_b32_e32 v20, v0\n") == (0, 0)
