@@ -49,7 +49,9 @@ int launch_tile256_pingpong(const GemmArgs& g, int in_dtype, int out_dtype, hipS
 // Single-wave-group ring kernel.  `tile` is 256 or 128 (square tiles) or kRingTile256x128 (256 rows
 // of A by 128 rows of B); ring_tile_edge, ring_splits and ring_tail are pure host heuristics.
 constexpr int kRingTile256x128 = 384;
-inline int ring_tile_rows(int tile) { return tile == 128 ? 128 : 256; }
+// 128 x 128 tile on the nine-slot ring (four k-steps of copies in flight, one workgroup per CU).
+constexpr int kRingTile128Deep = 129;
+inline int ring_tile_rows(int tile) { return tile == 128 || (tile >= kRingTile128Deep && tile < 140) ? 128 : 256; }
 inline int ring_tile_cols(int tile) { return tile == 256 ? 256 : 128; }
 int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes);
 int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes);

@@ -89,8 +89,15 @@ constexpr uint32_t kMxUnitBytes = 512;
 // kTileNT: rows of B per workgroup when they differ from kTileT: the 256x128 tile (128x64 per wave)
 // has three times as many tiles as 256x256 on shapes that leave most CUs without a 256x256 tile,
 // and moves 1.5 times the bytes per flop instead of the 128x128 tile's two times.
-template <class T, class OutT, bool kRaggedK, int kTileT, int kWavesN = 2, int kTileNT = kTileT>
-__global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void gemm_tn_tile_ring(GemmArgs g) {
+// kAhead (d): k-steps of copies kept in flight; the ring has 2d + 1 slots.  The ring described
+// above is d = 2.  d = 4 (nine 16 KiB slots of the 128-row tile, one workgroup per CU) is for
+// problems with one or two tile rows, whose rows of B are read by one or two workgroups only and so
+// come from HBM, not from the L2: with d = 2 an operand-step has about one k-step of flight time
+// before the barrier that waits for it (a third of a microsecond on the small tile), with d = 4
+// about three.
+template <class T, class OutT, bool kRaggedK, int kTileT, int kWavesN = 2, int kTileNT = kTileT, int kAhead = 2>
+__global__ __launch_bounds__(threads_of(kWavesN), (kTileT == 256 || kAhead > 2) ? 1 : 2) void gemm_tn_tile_ring(GemmArgs g) {
+  constexpr int kSlots = 2 * kAhead + 1;          // shadows the five of ring_common.h
   constexpr int kTile = kTileT;                   // rows of A per workgroup
   constexpr int kTileN = kTileNT;                 // rows of B per workgroup
   static_assert(kTileN <= kTile, "a slot is sized for the rows of A");
@@ -118,6 +125,8 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   // spans all of them, the two halves of the wave's rows of A.
   constexpr bool kRowSliced = G::kRowSliced;
   constexpr bool kMx = G::kMx;
+  static_assert(kSlots * kSlotBytes <= 160 * 1024, "the ring must fit the LDS of a CU");
+  static_assert(!kMx || kAhead == 2, "block scales: the scale registers are sized and timed for the five-slot ring");
   static_assert(!kMx || (kRowSliced && !kRaggedK && (kWaveTileM == 128 || kWaveTileM == 64) &&
                          (kWaveTileN == 128 || kWaveTileN == 64)),
                 "block scales: whole k-steps, a whole or half 128-row scale group per wave and operand");
@@ -247,8 +256,20 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     copy_rows(rsrc, jc, slotc, soff, voff_b, tail_b, b_step, dma_wave_b);
   };
   // Byte offset of k-step kt of the item that starts at global k-step step0, clamped to its last.
+  // kRotate (the deep ring, i.e. problems of one or two tile rows whose workgroups all read
+  // different rows of B): an item walks its k-steps from its own starting point `rot` and wraps
+  // around, so that the workgroups running side by side do not all read the same 128-byte column
+  // of rows that lie a power of two apart, i.e. the same few memory channels, at the same time.
+  // Only the order of the fp32 additions of a tile depends on it, and that order is fixed per item.
+  constexpr bool kRotate = kAhead > 2;
+  uint32_t rot = 0;
   auto soff_of = [&](uint32_t step0, uint32_t kt) __attribute__((always_inline)) -> uint32_t {
-    return __builtin_amdgcn_readfirstlane((step0 + (kt < steps ? kt : steps - 1)) * kRowBytes);
+    uint32_t at = kt < steps ? kt : steps - 1;
+    if constexpr (kRotate) {
+      at += rot;
+      at = at >= steps ? at - steps : at;
+    }
+    return __builtin_amdgcn_readfirstlane((step0 + at) * kRowBytes);
   };
   // Opening copies of a tile: A0 B0 A1 B1 A2 into slots 0..4.
   // Block scales (kMx only).  Set ph holds the scales of the k-step worked off in ring phase ph:
@@ -276,12 +297,14 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     load_8B_async(scb[1], rsrc_sb, voff_sb, mx_soff_of(1));
   };
   auto open_tile = [&](__amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb, uint32_t step0) __attribute__((always_inline)) {
-    const uint32_t s0 = soff_of(step0, 0), s1 = soff_of(step0, 1), s2 = soff_of(step0, 2);
-    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, std::integral_constant<uint32_t, 0>{}, s0); });
-    static_for<kCphB>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, std::integral_constant<uint32_t, 1>{}, s0); });
-    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, std::integral_constant<uint32_t, 2>{}, s1); });
-    static_for<kCphB>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, std::integral_constant<uint32_t, 3>{}, s1); });
-    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, std::integral_constant<uint32_t, 4>{}, s2); });
+    // operand-steps A0 B0 A1 B1 ... A(kAhead) into slots 0 .. 2 kAhead
+    static_for<kAhead + 1>([&](auto tc) __attribute__((always_inline)) {
+      constexpr int t = decltype(tc)::value;
+      const uint32_t st = soff_of(step0, t);
+      static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_a(ra, j, std::integral_constant<uint32_t, 2 * t>{}, st); });
+      if constexpr (t < kAhead)
+        static_for<kCphB>([&](auto j) __attribute__((always_inline)) { copy_b(rb, j, std::integral_constant<uint32_t, 2 * t + 1>{}, st); });
+    });
   };
 
   // Fragment geometry: lane l supplies row l%kBlk of a block; group l/kBlk picks the chunks.
@@ -370,6 +393,12 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
   uint32_t tile_m, tile_n, tile_no, split;
   uint32_t step0;  // first k-step of the current item
   bool partial_item = decode_item(item, &tile_no, &split, &step0);
+  // spread the starting points of the items evenly over their k-steps
+  auto rot_of = [&](uint32_t it) __attribute__((always_inline)) -> uint32_t {
+    // 32-bit arithmetic: a row panel is below 2 GiB (host check), so an item has fewer than 2^16 k-steps
+    return kRotate ? __builtin_amdgcn_readfirstlane((it & 0xffffu) * steps / total_items % steps) : 0u;
+  };
+  rot = rot_of(item);
   tile_coord_t<uint32_t>(tile_no, tiles_m, tiles_n, &tile_m, &tile_n);
   __amdgpu_buffer_rsrc_t rsrc_a = panel_a((int64_t)tile_m * kTile), rsrc_b = panel_b((int64_t)tile_n * kTileN);
   if constexpr (kMx) mx_open_tile(tile_m, tile_n, step0);  // before the copies: see the waits
@@ -383,8 +412,9 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
 #pragma unroll
         for (int r = 0; r < kAccLen; ++r) acc[i][j][r] = 0.f;
 
-    // A0 and B0 have landed; A1, B1, A2 may be in flight (the counter saturates at 63).
-    wait_vmcnt<(2 * kCph + kCphB < 63 ? 2 * kCph + kCphB : 63)>();
+    // A0 and B0 have landed; A1, B1, ... A(kAhead) may be in flight (the counter saturates at 63).
+    constexpr int kOpenInFlight = kAhead * kCph + (kAhead - 1) * kCphB;
+    wait_vmcnt<(kOpenInFlight < 63 ? kOpenInFlight : 63)>();
     __builtin_amdgcn_s_barrier();
     if constexpr (kRowSliced) {
 #pragma unroll
@@ -398,9 +428,10 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
 
     // The slot of A(t) walks 0, 2, 4, 1, 3 and repeats, so the loop is unrolled over five phases in
     // which every slot number, and with it every LDS offset, is a compile-time constant.
-    // Row offsets of the operand k-steps the loop copies next, B(t+2) and A(t+3).
+    // Row offsets of the operand k-steps the loop copies next, B(t+kAhead) and A(t+kAhead+1).
     const uint32_t soff_last = soff_of(step0, steps - 1);
-    uint32_t soff_b = soff_of(step0, 2), soff_a = soff_of(step0, 3);
+    uint32_t soff_b = soff_of(step0, kAhead), soff_a = soff_of(step0, kAhead + 1);
+    uint32_t kt_b = kAhead, kt_a = kAhead + 1;   // kRotate: k-steps (of the item) the loop copies next
     // Offset of the scales the loop loads next (those of k-step t+2).
     const uint32_t mx_soff_last = mx_soff_of(steps - 1);
     uint32_t mx_soff = mx_soff_of(2);
@@ -464,9 +495,12 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
         }
         if constexpr (s == 0 && u == kBarrierAt) {
           // My reads of this k-step's slots are back; B(t+1) (and A(t+1) before it) have
-          // landed; only this wave's copies of A(t+2) may still be in flight.
+          // landed; only this wave's copies of A(t+2) [... B(t+kAhead-1), A(t+kAhead)] may still be
+          // in flight.
           wait_lgkmcnt0();
-          wait_vmcnt<kCph + (kMx ? 2 : 0)>();  // the two scale requests of this k-step are younger still
+          constexpr int kLoopInFlight = (kAhead - 1) * kCph + (kAhead - 2) * kCphB;
+          static_assert(kLoopInFlight + 2 < 64, "vmcnt is a 6-bit counter");
+          wait_vmcnt<kLoopInFlight + (kMx ? 2 : 0)>();  // the two scale requests of this k-step are younger still
           __builtin_amdgcn_s_barrier();
         }
         // Copy c is "prepared" (its LDS base written to M0) one MFMA before it is issued when it
@@ -502,8 +536,13 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
         else mfma_u(s, u);
         MI355_FENCE();
       });
-      soff_b = soff_b + kRowBytes < soff_last ? soff_b + kRowBytes : soff_last;
-      soff_a = soff_a + kRowBytes < soff_last ? soff_a + kRowBytes : soff_last;
+      if constexpr (kRotate) {
+        soff_b = soff_of(step0, ++kt_b);
+        soff_a = soff_of(step0, ++kt_a);
+      } else {
+        soff_b = soff_b + kRowBytes < soff_last ? soff_b + kRowBytes : soff_last;
+        soff_a = soff_a + kRowBytes < soff_last ? soff_a + kRowBytes : soff_last;
+      }
       if constexpr (kMx) mx_soff = mx_soff + kMxUnitBytes < mx_soff_last ? mx_soff + kMxUnitBytes : mx_soff_last;
       ++kt;
       last = kt == steps;
@@ -523,6 +562,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), kTileT == 256 ? 1 : 2) void ge
     const bool more = item < total_items;
     if (more) {
       partial_item = decode_item(item, &tile_no, &split, &step0);
+      rot = rot_of(item);
       tile_coord_t<uint32_t>(tile_no, tiles_m, tiles_n, &tile_m, &tile_n);
       rsrc_a = panel_a((int64_t)tile_m * kTile);
       rsrc_b = panel_b((int64_t)tile_n * kTileN);
@@ -557,19 +597,18 @@ __global__ __launch_bounds__(256) void tail_reduce(GemmArgs g) {
   *(u32x2*)((uint16_t*)g.C + m * g.ldc + n) = Pack4<OutT>::run(sum[0] * scale, sum[1] * scale, sum[2] * scale, sum[3] * scale);
 }
 
-template <class T, class OutT, int kTileT, int kTileNT = kTileT>
+template <class T, class OutT, int kTileT, int kTileNT = kTileT, int kAhead = 2, int kWavesN = 2>
 int launch_tile(const GemmArgs& g, hipStream_t stream) {
   const int64_t items = g.tail_tiles ? g.tiles_m * g.tiles_n + (int64_t)g.tail_tiles * (g.tail_splits - 1)
                                      : g.tiles_m * g.tiles_n * g.splits;
   if (items >= ((int64_t)1 << 31)) return -1;  // the kernel counts items in 32 bits
-  const int64_t slots = (int64_t)compute_units() * (kTileT == 256 ? 1 : 2);  // resident workgroups (LDS-bound)
+  const int64_t slots = (int64_t)compute_units() * ((kTileT == 256 || kAhead > 2) ? 1 : 2);  // resident workgroups (LDS-bound)
   const int64_t blocks = items < slots ? items : slots;
-  constexpr int kWavesN = 2;
   if ((g.K * T::kBytes) % kRowBytes == 0) {
-    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, false, kTileT, kWavesN, kTileNT>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
+    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, false, kTileT, kWavesN, kTileNT, kAhead>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
   } else {
     if constexpr (std::is_same<T, MxE4M3>::value) return -1;  // block scales need whole k-steps (host check)
-    else hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, true, kTileT, kWavesN, kTileNT>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
+    else hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, true, kTileT, kWavesN, kTileNT, kAhead>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
   }
   if (hipGetLastError() != hipSuccess) return -1;
   if (g.splits > 1)
@@ -585,6 +624,14 @@ int launch_tile(const GemmArgs& g, hipStream_t stream) {
 template <class T, class OutT>
 int launch(const GemmArgs& g, int tile, hipStream_t stream) {
   if (tile == kRingTile256x128) return launch_tile<T, OutT, 256, 128>(g, stream);
+  if constexpr (!std::is_same<T, MxE4M3>::value)
+    if (tile == kRingTile128Deep) return launch_tile<T, OutT, 128, 128, 4>(g, stream);
+#ifdef MI355_EXPERIMENT
+  if constexpr (std::is_same<T, BF16>::value && std::is_same<OutT, BF16>::value) {
+    if (tile == 130) return launch_tile<T, OutT, 128, 128, 4, 4>(g, stream);
+    if (tile == 131) return launch_tile<T, OutT, 128, 128, 3, 2>(g, stream);
+  }
+#endif
   return tile == 128 ? launch_tile<T, OutT, 128>(g, stream) : launch_tile<T, OutT, 256>(g, stream);
 }
 

@@ -5,6 +5,9 @@
 // Scheduler's round structure (gemm.cuh:168-212).
 #include "gemm_launch.h"
 #include "ring_common.h"
+#ifdef MI355_EXPERIMENT
+#include <cstdlib>
+#endif
 
 namespace mi355 {
 
@@ -26,6 +29,9 @@ int64_t tiles_of(int64_t M, int64_t N, int tile) {
 // (two of which fit a CU): filling both places with K splits measured 7-13 % slower on
 // M = 128..256 against N = 14336.
 int uniform_splits(int64_t tiles, int64_t steps) {
+#ifdef MI355_EXPERIMENT
+  if (const char* f = getenv("MI355_FORCE_SPLITS")) return atoi(f);
+#endif
   int best = 1;
   for (int s = 2; s <= 16; ++s) {
     if (tiles * s > kSlots) break;
@@ -112,6 +118,9 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
 // picked on large problems where 256x256 measured 20-40 % faster; with no margin on mid-sized fp8
 // problems where the small tile measured 7-15 % faster.  Mean regret over 124 measured problems: 0.9 %.)
 int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes) {
+#ifdef MI355_EXPERIMENT
+  if (const char* f = getenv("MI355_FORCE_TILE")) return atoi(f);
+#endif
   const double e256 = estimate_us(256, M, N, K, elem_bytes);
   const double e128 = estimate_us(128, M, N, K, elem_bytes);
   const double e2 = estimate_us(kRingTile256x128, M, N, K, elem_bytes);
