@@ -81,6 +81,7 @@ def build_lib():
                 raise RuntimeError("expected one device assembly file for %s, found %r" % (src, asm))
             n_st, n_mf = check_async_loads.check_hazard_distances(asm[0])
             stores, mfmas = stores + n_st, mfmas + n_mf
+            check_async_loads.check_no_scratch(asm[0])
         print("check_async_loads: %d stores keep their data registers for %d wait states, %d inline MFMAs keep their "
               "results untouched for %d" % (stores, check_async_loads.STORE_DATA_WINDOW, mfmas,
                                              check_async_loads.MFMA_RESULT_WINDOW), flush=True)

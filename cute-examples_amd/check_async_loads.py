@@ -265,3 +265,19 @@ def check_hazard_distances(asm_path, kernel_filter=None):
     if not found:
         raise RuntimeError("no kernel matching %r in %s" % (kernel_filter, asm_path))
     return stores, mfmas
+
+
+def check_no_scratch(asm_path):
+    """The ring kernels count the vector-memory instructions in flight by hand (s_waitcnt vmcnt(N) with N
+    derived from the copies they issue); a register spill would add loads and stores of its own to
+    that count.  No kernel of the file may use scratch memory or spill a vector register.  Returns
+    the number of kernels checked."""
+    src = open(asm_path).read()
+    sizes = [int(x) for x in re.findall(r'^\s*\.private_segment_fixed_size:\s*(\d+)', src, re.M)]
+    spills = [int(x) for x in re.findall(r'^\s*\.vgpr_spill_count:\s*(\d+)', src, re.M)]
+    if not sizes or len(sizes) != len(spills):
+        raise RuntimeError("no kernel metadata found in " + asm_path)
+    if any(sizes) or any(spills):
+        raise RuntimeError("%s: a kernel uses scratch memory (bytes per lane %r, spilled registers %r)"
+                           % (asm_path, sizes, spills))
+    return len(sizes)

@@ -624,14 +624,10 @@ int launch_tile(const GemmArgs& g, hipStream_t stream) {
 template <class T, class OutT>
 int launch(const GemmArgs& g, int tile, hipStream_t stream) {
   if (tile == kRingTile256x128) return launch_tile<T, OutT, 256, 128>(g, stream);
-  if constexpr (!std::is_same<T, MxE4M3>::value)
-    if (tile == kRingTile128Deep) return launch_tile<T, OutT, 128, 128, 4>(g, stream);
-#ifdef MI355_EXPERIMENT
-  if constexpr (std::is_same<T, BF16>::value && std::is_same<OutT, BF16>::value) {
-    if (tile == 130) return launch_tile<T, OutT, 128, 128, 4, 4>(g, stream);
-    if (tile == 131) return launch_tile<T, OutT, 128, 128, 3, 2>(g, stream);
+  if (tile == kRingTile128Deep) {   // the planner picks it for 16-bit inputs only
+    if constexpr (T::kBytes == 2) return launch_tile<T, OutT, 128, 128, 4>(g, stream);
+    else return -1;
   }
-#endif
   return tile == 128 ? launch_tile<T, OutT, 128>(g, stream) : launch_tile<T, OutT, 256>(g, stream);
 }
 

@@ -5,16 +5,13 @@
 // Scheduler's round structure (gemm.cuh:168-212).
 #include "gemm_launch.h"
 #include "ring_common.h"
-#ifdef MI355_EXPERIMENT
-#include <cstdlib>
-#endif
 
 namespace mi355 {
 
 namespace {
 
-constexpr int64_t kSlots = 256;  // one work item per CU of an MI355X; heuristics only, so no device query
-constexpr int64_t kSmallProblemTiles = 2 * kSlots;  // 128x128 tiles that are resident all at once
+constexpr int64_t kCuSlots = 256;  // one work item per CU of an MI355X; heuristics only, so no device query
+constexpr int64_t kSmallProblemTiles = 2 * kCuSlots;  // 128x128 tiles that are resident all at once
 
 int64_t k_steps_of(int64_t K, int elem_bytes) { return (K * elem_bytes + kRowBytes - 1) / kRowBytes; }
 
@@ -29,12 +26,9 @@ int64_t tiles_of(int64_t M, int64_t N, int tile) {
 // (two of which fit a CU): filling both places with K splits measured 7-13 % slower on
 // M = 128..256 against N = 14336.
 int uniform_splits(int64_t tiles, int64_t steps) {
-#ifdef MI355_EXPERIMENT
-  if (const char* f = getenv("MI355_FORCE_SPLITS")) return atoi(f);
-#endif
   int best = 1;
   for (int s = 2; s <= 16; ++s) {
-    if (tiles * s > kSlots) break;
+    if (tiles * s > kCuSlots) break;
     if (steps / s < 16) continue;   // the k-steps need not divide: the items' lengths differ by at most one
     best = s;
   }
@@ -52,11 +46,11 @@ int uniform_splits(int64_t tiles, int64_t steps) {
 void tail_plan(int64_t tiles, int64_t steps, int* tail_tiles, int* tail_splits) {
   *tail_tiles = 0;
   *tail_splits = 1;
-  const int64_t rest = tiles % kSlots;
-  if (tiles < kSlots || tiles > 3 * kSlots || rest == 0) return;
+  const int64_t rest = tiles % kCuSlots;
+  if (tiles < kCuSlots || tiles > 3 * kCuSlots || rest == 0) return;
   int best = 1;
   for (int s = 2; s <= 16; ++s) {
-    if (rest * s > kSlots) break;
+    if (rest * s > kCuSlots) break;
     if (steps / s < 16) continue;   // the k-steps need not divide: the items' lengths differ by at most one
     best = s;
   }
@@ -83,7 +77,7 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
   const int64_t steps = k_steps_of(K, elem_bytes);
   const int s = uniform_splits(tiles, steps);
   const int64_t items = tiles * s;
-  double rounds = (double)((items + kSlots - 1) / kSlots);
+  double rounds = (double)((items + kCuSlots - 1) / kCuSlots);
   double step_us, fixed_us;
   if (tile == 256) {
     step_us = items >= 224 ? 1.45 : 1.2;
@@ -91,12 +85,12 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
     int tail_tiles, tail_splits;
     tail_plan(tiles, steps, &tail_tiles, &tail_splits);
     if (tail_tiles) {
-      rounds = (double)(tiles / kSlots) + 1.0 / tail_splits + 0.2;
-    } else if (s == 1 && items > kSlots) {
+      rounds = (double)(tiles / kCuSlots) + 1.0 / tail_splits + 0.2;
+    } else if (s == 1 && items > kCuSlots) {
       // full rounds, then a last round that runs at the higher clock unless it is (nearly) full too
-      const int64_t rest = items % kSlots;
+      const int64_t rest = items % kCuSlots;
       const double last = rest == 0 ? 0.0 : (double)steps * (rest >= 224 ? 1.45 : 1.2) + fixed_us;
-      return (double)(items / kSlots) * ((double)steps * 1.45 + fixed_us) + last;
+      return (double)(items / kCuSlots) * ((double)steps * 1.45 + fixed_us) + last;
     }
   } else if (tile == kRingTile256x128) {
     step_us = 0.85;
@@ -118,9 +112,17 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
 // picked on large problems where 256x256 measured 20-40 % faster; with no margin on mid-sized fp8
 // problems where the small tile measured 7-15 % faster.  Mean regret over 124 measured problems: 0.9 %.)
 int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes) {
-#ifdef MI355_EXPERIMENT
-  if (const char* f = getenv("MI355_FORCE_TILE")) return atoi(f);
-#endif
+  // One or two rows of 128 x 128 tiles that nearly fill the CUs in one round, and a short K: every
+  // workgroup streams its own rows of B from HBM, which the nine-slot ring keeps further ahead of the
+  // MFMAs than the five-slot one can, and unsplit tiles spare the partial planes of a K split.
+  // Instantiated and measured for the 16-bit input types: against the rest of this planner on bf16
+  // (256, 11008...14336, 2048...4096) and
+  // (192, 14336, 4096): 3-10 % less time; with longer rows of K (from 5120 elements), more tiles than
+  // CUs or fewer than two thirds of them it loses by 1-60 %.
+  const int64_t small_tiles = tiles_of(M, N, 128);
+  if (elem_bytes == 2 && M <= 256 && small_tiles >= 170 && small_tiles <= kCuSlots && k_steps_of(K, elem_bytes) >= 16 &&
+      k_steps_of(K, elem_bytes) <= 64)
+    return kRingTile128Deep;
   const double e256 = estimate_us(256, M, N, K, elem_bytes);
   const double e128 = estimate_us(128, M, N, K, elem_bytes);
   const double e2 = estimate_us(kRingTile256x128, M, N, K, elem_bytes);

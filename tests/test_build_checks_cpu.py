@@ -224,3 +224,13 @@ def test_inline_mfma_results_are_left_alone_for_the_window(tmp_path):
         run_hazards(tmp_path, ASM_MFMA + "\t;;#ASMSTART\n\tv_mfma_f32_16x16x32_bf16 a[2:5], v[2:5], v[6:9], a[2:5]\n\t;;#ASMEND\n")
     # MFMAs the compiler emitted itself get their wait states from the compiler: not this check's business
     assert run_hazards(tmp_path, "\tv_mfma_f32_16x16x32_bf16 v[0:3], v[12:15], v[16:19], v[0:3]\n\tv_mov_b32_e32 v20, v0\n") == (0, 0)
+
+
+def test_scratch_use_is_rejected(tmp_path):
+    meta = "    .private_segment_fixed_size: %d\n    .vgpr_spill_count: %d\n"
+    f = tmp_path / "m.s"
+    f.write_text(meta % (0, 0) + meta % (0, 0))
+    assert check_async_loads.check_no_scratch(str(f)) == 2
+    f.write_text(meta % (0, 0) + meta % (1420, 1756))
+    with pytest.raises(RuntimeError, match="uses scratch memory"):
+        check_async_loads.check_no_scratch(str(f))

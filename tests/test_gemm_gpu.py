@@ -623,6 +623,27 @@ def test_config4_skinny_projections(abi, M, N, K):
         assert oracle.rel_frobenius(run_abi(abi, X, W, v), ref) < 4e-3, v
 
 
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", [(256, 14336, 4096), (200, 11012, 2056), (130, 12288, 1032), (256, 10880, 1024)])
+def test_one_or_two_tile_rows_on_the_nine_slot_ring(abi, dt, M, N, K):
+    """Problems of one or two rows of 128 x 128 tiles that nearly fill the CUs run on the deep ring
+    (four k-steps of copies in flight, k-steps walked from a per-workgroup starting point): ragged
+    M, N and K, both 16-bit input types, every element against the oracle."""
+    code = ac.torch_code(dt)
+    v, rows, cols, splits, tail_tiles, tail_splits = ac.plan(abi, M, N, K, code)
+    assert (v, rows, cols, splits, tail_tiles) == (ac.BASIC, 128, 128, 1, 0)
+    assert 170 <= -(-M // 128) * -(-N // 128) <= 256
+    A, B = rand((M, K), M + 3, dt), rand((N, K), N + 4, dt)
+    C = run_abi(abi, A, B, ac.AUTO, 0.5)
+    err, ref = check(C, A, B, 0.5)
+    assert err < 4e-3
+    # and bit for bit what the unrotated, five-slot form of the same kernel gives on a problem with
+    # the same k range per tile but fewer tiles: only the order of the k-steps differs between the
+    # two, so the results agree to fp32 summation order
+    small = run_abi(abi, A, B[:2048].contiguous(), ac.BASIC, 0.5)
+    assert oracle.rel_frobenius(C[:, :2048], small) < 2e-3
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 512, 128), (16, 128, 8), (48, 260, 1096), (256, 64, 4104), (10, 260, 256), (17, 64, 1024), (33, 512, 4096),
                                    (64, 1024, 2048), (100, 640, 1024), (129, 72, 512), (256, 768, 2048)])
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
