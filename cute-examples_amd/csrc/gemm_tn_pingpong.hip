@@ -14,10 +14,18 @@
 //
 // A wave's MFMA and load phases never overlap, so its operand fragments are single-buffered: a
 // load phase refills the registers the preceding MFMA phase has just finished with, and the other
-// group's MFMA phase (32 MFMAs, ~512 cycles) hides the LDS latency.  MFMA phases run at raised
-// wave priority.  LDS ring, swizzle, copy geometry and tile walk are those of the single-group
-// kernel (ring_common.h, gemm_tn_ring.h): five 32 KiB slots, operand-steps queued as
-// A0 B0 A1 B1 A2 ..., the two slots of k-step t refilled with B(t+2), A(t+3) once both groups
+// group's MFMA phase (512 MFMA cycles) hides the LDS latency.  MFMA phases run at raised wave
+// priority.  For the 16-bit types the two slices of a k-step are the two halves of its 128 bytes
+// of K (v_mfma_f32_16x16x32, 32 MFMAs per phase); for fp8 one v_mfma_f32_16x16x128_f8f6f4 spans the
+// k-step, so the slices are the two halves of the wave's rows of A (16 MFMAs per phase) and the
+// fragments of B are loaded once per k-step, in L1.
+//
+// Everything else is the single-group kernel's (gemm_tn_ring.h): the five-slot LDS ring with
+// operand-steps queued as A0 B0 A1 B1 A2 ..., the row swizzle, the copy geometry, the k loop
+// unrolled over the five positions of the ring so that every LDS offset is an immediate, MFMAs as
+// inline assembly with the accumulator tied in place, the copies of a k-step spread between the
+// LDS reads of their phase, the next tile's opening copies in flight while the finished tile is
+// stored (tile_store.h).  The two slots of k-step t are refilled with B(t+2), A(t+3) once both groups
 // have read them (end of phase 4t+2).
 //
 // Counterpart in the reference: kernels/gemm_kernels/sm90a/gemm_pingpong.cuh:121-349, where two
@@ -37,20 +45,19 @@ constexpr int kSlotBytes = kTile * kRowBytes;  // 32 KiB: one operand, one k-ste
 
 // kRaggedK: K*elem_bytes is not a multiple of the 128-byte k-step.  Kept out of the common
 // instantiation because selecting the per-lane offset inside the loop puts a dependent VALU
-// chain in front of every copy and costs ~8 % at 8192^3.
+// chain in front of every copy.
 template <class T, class OutT, bool kRaggedK>
 __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_pingpong(GemmArgs g) {
   __shared__ __attribute__((aligned(1024))) uint8_t ring[kSlots * kSlotBytes];
-  typedef Geo<T> G;
+  typedef typename RingGeo<T>::type G;
   typedef typename G::Frag Frag;
   typedef typename G::Acc Acc;
-  constexpr int kBlk = G::kBlk;
-  constexpr int kNbA = 128 / kBlk;                      // A blocks per wave (128 rows)
-  constexpr int kNbB = 64 / kBlk;                       // B blocks per wave (64 columns)
+  static_assert(G::kBlk == 16 && !G::kMx, "16 x 16 blocks, no block scales");
+  constexpr bool kRowSliced = G::kRowSliced;            // fp8: one MFMA spans the k-step
+  constexpr int kNbA = 8;                               // 16-row blocks of A per wave (128 rows)
+  constexpr int kNbB = 4;                               // 16-row blocks of B per wave (64 columns)
+  constexpr int kHalfA = kNbA / 2;
   constexpr int kSliceChunks = G::kGroups * G::kCpl;
-  constexpr int kSlices = 8 / kSliceChunks;
-  constexpr int kAccLen = kBlk * kBlk / 64;
-  static_assert(kSlices == 2, "the phase table assumes two slices per k-step");
 
   const uint32_t tid = threadIdx.x;
   const uint32_t lane = tid & 63u;
@@ -78,55 +85,64 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_pingpong(GemmArgs
 
   // Copy geometry as in the single-group kernel, but each of the 8 waves moves 32 rows of an
   // operand per k-step: copies 4w..4w+3 of 8 rows x 128 B.
+  constexpr int kCph = 4;
   const uint32_t r8 = lane >> 3, c8 = lane & 7u;
   constexpr uint32_t kOutOfRange = 0x80000000u;  // row panels are smaller than 2 GiB (host check)
-  uint32_t voff_a[2], voff_b[2], tail_a[2], tail_b[2];
+  uint32_t voff_a[2], voff_b[2], tail_a[kRaggedK ? 2 : 1], tail_b[kRaggedK ? 2 : 1];
 #pragma unroll
   for (int par = 0; par < 2; ++par) {
     const uint32_t chunk = c8 ^ swizzle(par * 8 + r8);
     voff_a[par] = (wave * 32 + r8) * lda_b + chunk * 16;
     voff_b[par] = (wave * 32 + r8) * ldb_b + chunk * 16;
-    const bool tail_or_oob = tail_bytes != 0 && chunk * 16 >= tail_bytes;
-    tail_a[par] = tail_or_oob ? kOutOfRange : voff_a[par];
-    tail_b[par] = tail_or_oob ? kOutOfRange : voff_b[par];
+    if constexpr (kRaggedK) {
+      const bool tail_or_oob = tail_bytes != 0 && chunk * 16 >= tail_bytes;
+      tail_a[par] = tail_or_oob ? kOutOfRange : voff_a[par];
+      tail_b[par] = tail_or_oob ? kOutOfRange : voff_b[par];
+    }
   }
   const uint32_t a_step = __builtin_amdgcn_readfirstlane(8 * lda_b);
   const uint32_t b_step = __builtin_amdgcn_readfirstlane(8 * ldb_b);
   const uint32_t ring0 = __builtin_amdgcn_readfirstlane(lds_address(ring));
-  const uint32_t dma_wave = ring0 + wave * 4096;
+  const uint32_t dma_wave = ring0 + wave * (kCph * 1024);  // this wave's share of a slot
+  const uint32_t soff_tail = (k_steps - 1) * kRowBytes;     // the k-step that may be ragged
 
-  auto copy_a = [&](__amdgpu_buffer_rsrc_t rsrc, int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
-    const uint32_t kk = kt < k_steps ? kt : k_steps - 1;
-    const uint32_t voff = kRaggedK && kk == k_steps - 1 ? tail_a[j & 1] : voff_a[j & 1];
-    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff + j * a_step, rsrc, kk * kRowBytes);
+  // Copy j of an operand's k-step into slot `slot` (a compile-time number); soff is the k-step's
+  // byte offset inside a row.
+  auto copy_rows = [&](__amdgpu_buffer_rsrc_t rsrc, auto jc, auto slotc, uint32_t soff, const uint32_t* voff,
+                       const uint32_t* tail, uint32_t step) __attribute__((always_inline)) {
+    constexpr int j = decltype(jc)::value;
+    constexpr uint32_t slot = decltype(slotc)::value;
+    uint32_t v = voff[j & 1];
+    if constexpr (kRaggedK) v = soff == soff_tail ? tail[j & 1] : v;
+    dma_16B_to_lds_at<slot * kSlotBytes + j * 1024>(dma_wave, v + j * step, rsrc, soff);
   };
-  auto copy_b = [&](__amdgpu_buffer_rsrc_t rsrc, int j, uint32_t slot, uint32_t kt) __attribute__((always_inline)) {
-    const uint32_t kk = kt < k_steps ? kt : k_steps - 1;
-    const uint32_t voff = kRaggedK && kk == k_steps - 1 ? tail_b[j & 1] : voff_b[j & 1];
-    dma_16B_to_lds(dma_wave + slot * kSlotBytes + j * 1024, voff + j * b_step, rsrc, kk * kRowBytes);
+  // Byte offset of k-step kt, clamped to the last: copies past the end of K re-read it into a slot
+  // nobody reads, so the loop body stays branch-free.
+  auto soff_of = [&](uint32_t kt) __attribute__((always_inline)) -> uint32_t {
+    return __builtin_amdgcn_readfirstlane((kt < k_steps ? kt : k_steps - 1) * kRowBytes);
   };
   auto open_tile = [&](__amdgpu_buffer_rsrc_t ra, __amdgpu_buffer_rsrc_t rb) __attribute__((always_inline)) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) copy_a(ra, j, 0, 0);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) copy_b(rb, j, 1, 0);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) copy_a(ra, j, 2, 1);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) copy_b(rb, j, 3, 1);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) copy_a(ra, j, 4, 2);
+    const uint32_t s0 = soff_of(0), s1 = soff_of(1), s2 = soff_of(2);
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_rows(ra, j, std::integral_constant<uint32_t, 0>{}, s0, voff_a, tail_a, a_step); });
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_rows(rb, j, std::integral_constant<uint32_t, 1>{}, s0, voff_b, tail_b, b_step); });
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_rows(ra, j, std::integral_constant<uint32_t, 2>{}, s1, voff_a, tail_a, a_step); });
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_rows(rb, j, std::integral_constant<uint32_t, 3>{}, s1, voff_b, tail_b, b_step); });
+    static_for<kCph>([&](auto j) __attribute__((always_inline)) { copy_rows(ra, j, std::integral_constant<uint32_t, 4>{}, s2, voff_a, tail_a, a_step); });
   };
 
-  const uint32_t rblk = lane & (kBlk - 1), grp = lane / kBlk;
+  // Fragment geometry: lane l supplies row l%16 of a block; group l/16 picks the chunks.
+  const uint32_t rblk = lane & 15u, grp = lane >> 4;
   const uint32_t swz = swizzle(rblk);
   const uint32_t a_lane = (wm * 128 + rblk) * kRowBytes;
   const uint32_t b_lane = (wn * 64 + rblk) * kRowBytes;
+  // Byte offset inside a row of the e-th chunk this lane reads in slice s (row-sliced: chunks g
+  // and 4+g, the conflict-free order, see chunk_off in gemm_tn_ring.h).
   auto chunk_off = [&](int s, int e) __attribute__((always_inline)) -> uint32_t {
-    return ((uint32_t)(s * kSliceChunks + grp * G::kCpl + e) ^ swz) << 4;
+    if constexpr (kRowSliced) return ((uint32_t)(grp + 4 * e) ^ swz) << 4;
+    else return ((uint32_t)(s * kSliceChunks + grp * G::kCpl + e) ^ swz) << 4;
   };
   auto load_frag = [&](const uint8_t* slot_rows, int blk, int s) __attribute__((always_inline)) -> Frag {
-    const uint8_t* p = slot_rows + blk * kBlk * kRowBytes;
+    const uint8_t* p = slot_rows + blk * 16 * kRowBytes;
     if constexpr (G::kCpl == 1) {
       return *(const i32x4*)(p + chunk_off(s, 0));
     } else {
@@ -137,20 +153,42 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_pingpong(GemmArgs
   };
 
   Acc acc[kNbA][kNbB];
-  Frag fa[kNbA], fb[kNbB];
+  // K-sliced: all blocks of A and of B, one slice of K at a time.  Row-sliced: all of B for the
+  // k-step and half of the wave's rows of A at a time.
+  Frag fa[kRowSliced ? kHalfA : kNbA], fb[kNbB];
 
-  auto load_phase_reads = [&](const uint8_t* a_rows, const uint8_t* b_rows, int s) __attribute__((always_inline)) {
-#pragma unroll
-    for (int j = 0; j < kNbB; ++j) fb[j] = load_frag(b_rows, j, s);
-#pragma unroll
-    for (int i = 0; i < kNbA; ++i) fa[i] = load_frag(a_rows, i, s);
+  // Load number q of the load phase in front of slice s (a_rows / b_rows: the slot rows of the k-step
+  // that slice belongs to); returns the number of loads of that phase through kReads.
+  constexpr int kReads0 = kRowSliced ? kNbB + kHalfA : kNbB + kNbA;   // in front of slice 0 (phase L1)
+  constexpr int kReads1 = kRowSliced ? kHalfA : kNbB + kNbA;          // in front of slice 1 (phase L0)
+  auto read_q = [&](auto sc, auto qc, const uint8_t* a_rows, const uint8_t* b_rows) __attribute__((always_inline)) {
+    constexpr int s = decltype(sc)::value, q = decltype(qc)::value;
+    if constexpr (kRowSliced) {
+      if constexpr (s == 0) {
+        if constexpr (q < kNbB) fb[q] = load_frag(b_rows, q, 0);
+        else fa[q - kNbB] = load_frag(a_rows, q - kNbB, 0);
+      } else {
+        fa[q] = load_frag(a_rows, kHalfA + q, 0);
+      }
+    } else {
+      if constexpr (q < kNbB) fb[q] = load_frag(b_rows, q, s);
+      else fa[q - kNbB] = load_frag(a_rows, q - kNbB, s);
+    }
   };
-  auto mfma_phase = [&]() __attribute__((always_inline)) {
+  auto mfma_phase = [&](auto sc) __attribute__((always_inline)) {
+    constexpr int s = decltype(sc)::value;
     __builtin_amdgcn_s_setprio(1);
-#pragma unroll
-    for (int i = 0; i < kNbA; ++i)
-#pragma unroll
-      for (int j = 0; j < kNbB; ++j) acc[i][j] = G::mfma(fb[j], fa[i], acc[i][j]);
+    if constexpr (kRowSliced) {
+      static_for<kHalfA * kNbB>([&](auto uc) __attribute__((always_inline)) {
+        constexpr int r = decltype(uc)::value / kNbB, j = decltype(uc)::value % kNbB;
+        G::mfma_inplace(fb[j], fa[r], acc[s * kHalfA + r][j]);
+      });
+    } else {
+      static_for<kNbA * kNbB>([&](auto uc) __attribute__((always_inline)) {
+        constexpr int i = decltype(uc)::value / kNbB, j = decltype(uc)::value % kNbB;
+        G::mfma_inplace(fb[j], fa[i], acc[i][j]);
+      });
+    }
     __builtin_amdgcn_s_setprio(0);
   };
   // Phase boundary: nothing may move across it.
@@ -162,7 +200,7 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_pingpong(GemmArgs
 
   const float scale = output_scale(g);
   auto epilogue = [&](int64_t m0, int64_t n0) __attribute__((always_inline)) {
-    store_output_tile<G, OutT, kNbA, kNbB, false>(acc, g, m0, n0, kTile, kTile, wm * 128, wn * 64, lane, scale);
+    store_output_tile<G, OutT, kNbA, kNbB, true>(acc, g, m0, n0, kTile, kTile, wm * 128, wn * 64, lane, scale);
   };
 
   const uint32_t tiles_m = (uint32_t)g.tiles_m, tiles_n = (uint32_t)g.tiles_n;  // below 2^31 tiles (launcher)
@@ -178,44 +216,76 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_tn_tile256_pingpong(GemmArgs
 #pragma unroll
       for (int j = 0; j < kNbB; ++j)
 #pragma unroll
-        for (int r = 0; r < kAccLen; ++r) acc[i][j][r] = 0.f;
+        for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-    wait_vmcnt<12>();  // A0 and B0 have landed (A1, B1, A2 may be in flight: 3 x 4 copies)
+    wait_vmcnt<3 * kCph>();  // A0 and B0 have landed (A1, B1, A2 may be in flight)
     phase_barrier();
-    load_phase_reads(ring + a_lane, ring + kSlotBytes + b_lane, 0);
+    static_for<kReads0>([&](auto q) __attribute__((always_inline)) {
+      read_q(std::integral_constant<int, 0>{}, q, ring + a_lane, ring + kSlotBytes + b_lane);
+    });
     wait_lgkmcnt0();
     if (group == 1) phase_barrier();  // group 1 runs one phase behind group 0
 
-    uint32_t slot_a = 0;
-    for (uint32_t kt = 0; kt < k_steps; ++kt) {
-      const uint32_t slot_b = slot_a + 1 >= kSlots ? slot_a + 1 - kSlots : slot_a + 1;
-      const uint32_t slot_a1 = slot_a + 2 >= kSlots ? slot_a + 2 - kSlots : slot_a + 2;
-      const uint32_t slot_b1 = slot_a + 3 >= kSlots ? slot_a + 3 - kSlots : slot_a + 3;
+    // Row offsets of the operand k-steps the loop copies next, B(t+2) and A(t+3).
+    const uint32_t soff_last = soff_of(k_steps - 1);
+    uint32_t soff_b = soff_of(2), soff_a = soff_of(3);
+    uint32_t kt = 0;
+    bool last = false;
+    for (;;) {
+      // The slot of A(t) walks 0, 2, 4, 1, 3: unrolled over the five positions, every slot number and
+      // with it every LDS offset is a compile-time constant.
+      static_for<kSlots>([&](auto phase) __attribute__((always_inline)) {
+        if (last) return;
+        constexpr uint32_t slot_a = (2 * decltype(phase)::value) % kSlots;
+        constexpr uint32_t slot_b = (slot_a + 1) % kSlots, slot_a1 = (slot_a + 2) % kSlots, slot_b1 = (slot_a + 3) % kSlots;
+        const uint8_t* a_rows = ring + slot_a * kSlotBytes + a_lane;
+        const uint8_t* b_rows = ring + slot_b * kSlotBytes + b_lane;
+        const uint8_t* a1_rows = ring + slot_a1 * kSlotBytes + a_lane;
+        const uint8_t* b1_rows = ring + slot_b1 * kSlotBytes + b_lane;
 
-      // M0: slice 0 of this k-step.
-      mfma_phase();
-      phase_barrier();
-      // L0: slice 1 of this k-step.  For group 1 this phase ends at global phase 4t+2, the point
-      // by which B(t+1) must have landed everywhere (only the 4 copies of A(t+2) may be in flight).
-      load_phase_reads(ring + slot_a * kSlotBytes + a_lane, ring + slot_b * kSlotBytes + b_lane, 1);
-      wait_lgkmcnt0();
-      if (group == 1) wait_vmcnt<4>();
-      phase_barrier();
-      // M1: slice 1.  For group 0 this phase ends at global phase 4t+2.
-      mfma_phase();
-      if (group == 0) wait_vmcnt<4>();
-      phase_barrier();
-      // L1: slice 0 of the next k-step, and this wave's share of the refill.  Both groups have
-      // finished reading the slots of k-step t by now (group 1 did so in its L0, one phase ago
-      // from group 0's point of view, three phases ago from its own).
-      load_phase_reads(ring + slot_a1 * kSlotBytes + a_lane, ring + slot_b1 * kSlotBytes + b_lane, 0);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) copy_b(rsrc_b, j, slot_a, kt + 2);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) copy_a(rsrc_a, j, slot_b, kt + 3);
-      wait_lgkmcnt0();
-      phase_barrier();
-      slot_a = slot_a1;
+        // M0: slice 0 of this k-step.
+        mfma_phase(std::integral_constant<int, 0>{});
+        phase_barrier();
+        // L0: slice 1 of this k-step.  For group 1 this phase ends at global phase 4t+2, the point
+        // by which B(t+1) must have landed everywhere (only the copies of A(t+2) may be in flight).
+        static_for<kReads1>([&](auto q) __attribute__((always_inline)) {
+          read_q(std::integral_constant<int, 1>{}, q, a_rows, b_rows);
+        });
+        wait_lgkmcnt0();
+        if (group == 1) wait_vmcnt<kCph>();
+        phase_barrier();
+        // M1: slice 1.  For group 0 this phase ends at global phase 4t+2.
+        mfma_phase(std::integral_constant<int, 1>{});
+        if (group == 0) wait_vmcnt<kCph>();
+        phase_barrier();
+        // L1: slice 0 of the next k-step, and this wave's share of the refill, one copy after
+        // every second read so that the copies do not queue up behind each other in the
+        // texture-address unit.  Both groups have finished reading the slots of k-step t by now
+        // (group 1 did so in its L0, one phase ago from group 0's point of view, three phases ago
+        // from its own).
+        static_for<kReads0>([&](auto qc) __attribute__((always_inline)) {
+          constexpr int q = decltype(qc)::value;
+          read_q(std::integral_constant<int, 0>{}, qc, a1_rows, b1_rows);
+          constexpr int kCopies = 2 * kCph;
+          // copy c goes after read number (c + 1) * kReads0 / kCopies - 1
+          static_for<kCopies>([&](auto cc) __attribute__((always_inline)) {
+            constexpr int c = decltype(cc)::value;
+            if constexpr ((c + 1) * kReads0 / kCopies - 1 == q) {
+              if constexpr (c < kCph)
+                copy_rows(rsrc_b, std::integral_constant<int, c>{}, std::integral_constant<uint32_t, slot_a>{}, soff_b, voff_b, tail_b, b_step);
+              else
+                copy_rows(rsrc_a, std::integral_constant<int, c - kCph>{}, std::integral_constant<uint32_t, slot_b>{}, soff_a, voff_a, tail_a, a_step);
+            }
+          });
+        });
+        wait_lgkmcnt0();
+        phase_barrier();
+        soff_b = soff_b + kRowBytes < soff_last ? soff_b + kRowBytes : soff_last;
+        soff_a = soff_a + kRowBytes < soff_last ? soff_a + kRowBytes : soff_last;
+        ++kt;
+        last = kt == k_steps;
+      });
+      if (last) break;
     }
     if (group == 0) phase_barrier();  // let group 1 finish its last phase; barrier counts now match
     wait_vmcnt<0>();

@@ -69,11 +69,6 @@ constexpr int first_copy_at(int p, int first, int span, int n) {
   return c;
 }
 
-// Geometry the kernel uses for an input type: fp8 runs on the 16x16x128 shape here.
-template <class T> struct RingGeo { typedef Geo<T> type; };
-template <> struct RingGeo<E4M3> { typedef GeoE4M3Rows type; };
-template <> struct RingGeo<MxE4M3> { typedef GeoMxE4M3Rows type; };
-
 // Layout of block scales as the kernel reads them ("shuffled", written by mx_scales.hip): one
 // 512-byte unit per (group of 128 rows, k-step); lane l of the wave that owns those rows reads the
 // 8 bytes at 8*l: byte i is the scale of row 16*i + l%16 of the group for K block 4*kstep + l/16.

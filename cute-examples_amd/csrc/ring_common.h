@@ -113,6 +113,11 @@ struct GeoMxE4M3Rows : GeoE4M3Rows {
   }
 };
 
+// Geometry the ring-buffered tile kernels use for an input type: fp8 runs on the 16x16x128 shape.
+template <class T> struct RingGeo { typedef Geo<T> type; };
+template <> struct RingGeo<E4M3> { typedef GeoE4M3Rows type; };
+template <> struct RingGeo<MxE4M3> { typedef GeoMxE4M3Rows type; };
+
 // Compute units of the current device (256 on MI355X); queried once per device.
 inline int compute_units() {
   static std::atomic<int> cached[64];
