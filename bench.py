@@ -271,6 +271,16 @@ def calibrate(A, B, do_settle=True):
                   "settle_launches": n_settle, "settle_ms": round(settle_ms, 1),
                   "what": "mi355_calibrate_mfma: 4 waves per CU, the tile kernel's MFMA pattern on fragments of this "
                           "workload's operands held in registers; no LDS, no copies, no barriers"}
+    # The same loop on all-zero operands: no data toggling, so the board power limit does not bind
+    # and the clock stays near nominal.  The gap to the figure above is what the data costs in clock.
+    zeros = torch.zeros(1 << 20, dtype=torch.uint8, device=A.device)
+
+    def mfma_zero():
+        rc = lib.mi355_calibrate_mfma(code, zeros.data_ptr(), zeros.numel(), zeros.data_ptr(), zeros.numel(), iters,
+                                      sink.data_ptr(), ctypes.byref(flops), stream)
+        assert rc == 0, rc
+    ms0, _, _, _ = time_calls(mfma_zero, 40, 5, do_settle)
+    mfma_entry["value_zero_operands"] = round(flops.value / ms0 / 1e9, 1)
     src = torch.empty(1 << 30, dtype=torch.uint8, device=A.device)
     src.view(torch.int32).random_()
 
