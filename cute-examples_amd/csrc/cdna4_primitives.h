@@ -82,9 +82,17 @@ __device__ __forceinline__ void dma_16B_to_lds_at(uint32_t lds_base, uint32_t vo
 // compiler knowing that the result arrives later: the caller must pass the pair through
 // wait_vmcnt_for<N>() (N = vector-memory instructions issued after this one) before its first use,
 // and must check in the generated code that the pair is not copied in between.
+// MI355_MX_SYNC_SCALES: the fallback the build switches to when that check of the generated code
+// fails (a different compiler may copy such a register): the load then waits for itself, and with
+// it for every copy in flight, which costs time in every k-step but needs no promise from the
+// register allocator.
 __device__ __forceinline__ void load_8B_async(u32x2& dst, __amdgpu_buffer_rsrc_t rsrc, uint32_t voffset,
                                               uint32_t soffset) {
+#ifdef MI355_MX_SYNC_SCALES
+  asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen\n\ts_waitcnt vmcnt(0)"
+#else
   asm volatile("buffer_load_dwordx2 %0, %1, %2, %3 offen"
+#endif
                : "=v"(dst)
                : "v"(voffset), "s"(rsrc), "s"(__builtin_amdgcn_readfirstlane(soffset))
                : "memory");
