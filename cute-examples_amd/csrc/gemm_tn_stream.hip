@@ -244,8 +244,18 @@ __global__ __launch_bounds__(256) void splitk_reduce(const float* partial, GemmA
   const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (q >= M * quads_per_row) return;
   const int64_t m = q / quads_per_row, n = (q % quads_per_row) * 4;
-  f32x4 sum = *(const f32x4*)(partial + m * N + n);
-  for (int s = 1; s < splits; ++s) sum += *(const f32x4*)(partial + ((int64_t)s * M + m) * N + n);
+  // Four planes per round: their loads go out together (a plane past the last one repeats the last and
+  // is not added), the additions keep the order of the planes.
+  const float* mine = partial + m * N + n;
+  const int64_t plane = M * N;
+  f32x4 sum = *(const f32x4*)mine;
+  for (int s0 = 1; s0 < splits; s0 += 4) {
+    f32x4 t[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t[i] = *(const f32x4*)(mine + (int64_t)(s0 + i < splits ? s0 + i : splits - 1) * plane);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sum = s0 + i < splits ? sum + t[i] : sum;
+  }
   *(u32x2*)(C + m * ldc + n) = Pack4<OutT>::run(sum[0] * scale, sum[1] * scale, sum[2] * scale, sum[3] * scale);
 }
 
