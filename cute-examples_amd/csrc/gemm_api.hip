@@ -223,7 +223,7 @@ int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant, 
   const int es = elem_bytes(in_dtype);
   if (v == MI355_VARIANT_SKINNY) {
     rows = M <= 16 ? 16 : M <= 32 ? 32 : M <= 64 ? 64 : M <= 128 ? 128 : 256;
-    cols = 64;
+    cols = mi355::stream_tile_cols(M, N, K, es);
     splits = mi355::stream_splits(M, N, K, es);
   } else if (v == MI355_VARIANT_PINGPONG) {
     rows = cols = 256;

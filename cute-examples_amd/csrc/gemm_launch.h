@@ -77,6 +77,7 @@ int launch_quantize_mxfp8(const void* x, int in_dtype, int64_t rows, int64_t K, 
                           uint8_t* scales, bool shuffled, hipStream_t stream);
 // Skinny (small-M) weight-streaming kernel.  stream_splits is a pure host function.
 int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx = false);  // mx: block scales ride along
+int stream_tile_cols(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx = false);  // rows of W per workgroup: 64 or 128
 int launch_stream_mx(const GemmArgs& g, int out_dtype, int splits, void* workspace, hipStream_t stream);
 int launch_stream(const GemmArgs& g, int in_dtype, int out_dtype, int splits, void* workspace, hipStream_t stream);
 // Per-tensor e4m3 quantisation (amax -> scale -> cast); scale_amax points to two floats.

@@ -26,6 +26,9 @@
 #include "ring_common.h"
 
 #include <type_traits>
+#ifdef MI355_EXPERIMENT
+#include <cstdlib>
+#endif
 
 namespace mi355 {
 namespace {
@@ -55,7 +58,6 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
   constexpr int kSliceChunks = G::kGroups * G::kCpl;   // 16-byte chunks of a row one MFMA consumes
   constexpr int kSlices = 8 / kSliceChunks;            // MFMAs per k-step and block pair
   constexpr int kTm = 16 * kMB * kWM, kTn = 16 * kNB * kWN;
-  static_assert(kTn == kTileN, "grid assumes 64-row W tiles");
   constexpr bool kMx = G::kMx;
   static_assert(!kMx || (kWM == 1 && kWN == 4 && kNB == 1), "block scales: one 64-row half group per operand");
   constexpr int kDataBytes = (kTm + kTn) * kRowBytes;
@@ -261,8 +263,8 @@ __global__ __launch_bounds__(256) void splitk_reduce(const float* partial, GemmA
 
 template <class T, class OutT, int kMB, int kNB, int kWM, int kWN, int kDepth>
 int launch_cfg(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
-  constexpr int kTm = 16 * kMB * kWM;
-  const int64_t tiles = ((g.M + kTm - 1) / kTm) * ((g.N + kTileN - 1) / kTileN);
+  constexpr int kTm = 16 * kMB * kWM, kTn = 16 * kNB * kWN;
+  const int64_t tiles = ((g.M + kTm - 1) / kTm) * ((g.N + kTn - 1) / kTn);
   float* partial = splits > 1 ? ws : nullptr;
   hipLaunchKernelGGL((gemm_tn_stream<T, OutT, kMB, kNB, kWM, kWN, kDepth>), dim3((unsigned)tiles, (unsigned)splits),
                      dim3(kThreads), 0, stream, g, partial, splits);
@@ -308,37 +310,14 @@ int launch_64(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
   else return launch_cfg<T, OutT, 2, 2, 2, 2, kDepth>(g, splits, ws, stream);
 }
 
-template <class T, class OutT>
-int launch_m(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
-  if (splits == 1 && unsplit_deep(g.M, g.N, std::is_same<T, MxE4M3>::value)) {
-    if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
-    if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
-    return launch_64<T, OutT, kDepthUnsplit>(g, splits, ws, stream);
-  }
-  if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, kDepth16>(g, splits, ws, stream);   //  16x64, 10 KiB/step
-  if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, kDepth32>(g, splits, ws, stream);   //  32x64, 12 KiB/step
-  if (g.M <= 64) return launch_64<T, OutT, kDepth64>(g, splits, ws, stream);                 //  64x64, 16 KiB/step
-  if constexpr (std::is_same<T, MxE4M3>::value) {
-    return -1;   // block scales: up to 64 rows (the host routes taller problems to the tile kernel)
-  } else {
-    if (g.M <= 128) return launch_cfg<T, OutT, 4, 2, 2, 2, kDepth128>(g, splits, ws, stream);  // 128x64, 24 KiB/step
-    return launch_cfg<T, OutT, 4, 4, 4, 1, kDepth256>(g, splits, ws, stream);                  // 256x64, 40 KiB/step
-  }
-}
-
-}  // namespace
-
-// K splits for a skinny problem: as many workgroups as can be resident at once (one wave of
-// workgroups, no tail), each with enough k-steps.
-int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
-  const int64_t tm = M <= 16 ? 16 : M <= 32 ? 32 : M <= 64 ? 64 : M <= 128 ? 128 : 256;
-  const int depth = M <= 16 ? 4 : M <= 32 ? 4 : M <= 64 ? 3 : M <= 128 ? 4 : 3;  // kDepth16 .. kDepth256
-  const int64_t ring_bytes = depth * ((tm + kTileN) * kRowBytes + (mx ? 512 : 0));
+// K splits for tiles of tm x tn in a ring of `depth` stages: as many workgroups as can be resident at
+// once (one wave of workgroups, no tail), each with enough k-steps.
+int splits_for(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx, int64_t tm, int64_t tn, int depth) {
+  const int64_t ring_bytes = depth * ((tm + tn) * kRowBytes + (mx ? 512 : 0));
   const int64_t per_cu = 163840 / ring_bytes < 8 ? 163840 / ring_bytes : 8;   // LDS-bound residency
   const int64_t slots = 256 * per_cu;  // MI355X has 256 CUs; a heuristic only, so no device query here
-  const int64_t tiles = ((M + tm - 1) / tm) * ((N + kTileN - 1) / kTileN);
+  const int64_t tiles = ((M + tm - 1) / tm) * ((N + tn - 1) / tn);
   const int64_t steps = (K * elem_bytes + kRowBytes - 1) / kRowBytes;
-  if (unsplit_deep(M, N, mx)) return 1;
   // The workgroups of a CU share its bandwidth, and one of them already keeps it busy, so what counts
   // is the CU with the most k-steps to stream: ceil(workgroups / 256) workgroups of ceil(steps / S)
   // k-steps, each paying about four more to fill and drain its ring; splits beyond that only add
@@ -357,6 +336,67 @@ int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
     }
   }
   return best;
+}
+
+int splits_narrow(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
+  if (unsplit_deep(M, N, mx)) return 1;
+  const int64_t tm = M <= 16 ? 16 : M <= 32 ? 32 : M <= 64 ? 64 : M <= 128 ? 128 : 256;
+  const int depth = M <= 16 ? kDepth16 : M <= 32 ? kDepth32 : M <= 64 ? kDepth64 : M <= 128 ? kDepth128 : kDepth256;
+  return splits_for(M, N, K, elem_bytes, mx, tm, kTileN, depth);
+}
+
+// 64 x 128 tiles for 33...64 rows: a quarter fewer cache lines requested per output than 64 x 64 (192
+// per 64 x 128 outputs and k-step against 2 x 128), paid for with half as many tiles to spread over the
+// CUs.  Measured against the 64 x 64 tiles on 112 bf16 problems (M = 48 and 64, N = 2048...32768,
+// K = 2048...14336, weights from HBM), each with its own best split: 3-16 % faster where 160-256 wide
+// tiles make one unsplit round (N = 20480...32768), 2-11 % at N = 8192...11008 from 64 k-steps on and
+// 4-13 % at N = 4096...6144 from 128 k-steps on; 3-20 % slower with fewer k-steps than that or fewer
+// columns (the split needed to occupy the CUs leaves each workgroup too few k-steps), within +-3 % at
+// N = 12288...16384, where the 64 x 64 tiles run unsplit on the deep ring.
+constexpr int kTileNWide = 128, kDepthWide = 3;
+bool wide_tiles(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
+#ifdef MI355_EXPERIMENT
+  if (getenv("MI355_STREAM_NOWIDE")) return false;
+  if (getenv("MI355_STREAM_ALLWIDE")) return !mx && M > 32 && M <= 64;
+#endif
+  if (mx || M <= 32 || M > 64) return false;
+  const int64_t tiles = (N + kTileNWide - 1) / kTileNWide;
+  const int64_t steps = (K * elem_bytes + kRowBytes - 1) / kRowBytes;
+  if (tiles >= 160) return tiles <= 256;
+  if (tiles >= 64) return tiles < 96 && steps >= 64;
+  return tiles >= 32 && steps >= 128;
+}
+
+template <class T, class OutT>
+int launch_m(const GemmArgs& g, int splits, float* ws, hipStream_t stream) {
+  if (wide_tiles(g.M, g.N, g.K, T::kBytes, std::is_same<T, MxE4M3>::value)) {
+    if constexpr (!std::is_same<T, MxE4M3>::value) return launch_cfg<T, OutT, 2, 4, 2, 2, kDepthWide>(g, splits, ws, stream);
+  }
+  if (splits == 1 && unsplit_deep(g.M, g.N, std::is_same<T, MxE4M3>::value)) {
+    if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
+    if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, kDepthUnsplit>(g, splits, ws, stream);
+    return launch_64<T, OutT, kDepthUnsplit>(g, splits, ws, stream);
+  }
+  if (g.M <= 16) return launch_cfg<T, OutT, 1, 1, 1, 4, kDepth16>(g, splits, ws, stream);   //  16x64, 10 KiB/step
+  if (g.M <= 32) return launch_cfg<T, OutT, 2, 1, 1, 4, kDepth32>(g, splits, ws, stream);   //  32x64, 12 KiB/step
+  if (g.M <= 64) return launch_64<T, OutT, kDepth64>(g, splits, ws, stream);                 //  64x64, 16 KiB/step
+  if constexpr (std::is_same<T, MxE4M3>::value) {
+    return -1;   // block scales: up to 64 rows (the host routes taller problems to the tile kernel)
+  } else {
+    if (g.M <= 128) return launch_cfg<T, OutT, 4, 2, 2, 2, kDepth128>(g, splits, ws, stream);  // 128x64, 24 KiB/step
+    return launch_cfg<T, OutT, 4, 4, 4, 1, kDepth256>(g, splits, ws, stream);                  // 256x64, 40 KiB/step
+  }
+}
+
+}  // namespace
+
+int stream_tile_cols(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
+  return wide_tiles(M, N, K, elem_bytes, mx) ? kTileNWide : kTileN;
+}
+
+int stream_splits(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
+  if (wide_tiles(M, N, K, elem_bytes, mx)) return splits_for(M, N, K, elem_bytes, mx, 64, kTileNWide, kDepthWide);
+  return splits_narrow(M, N, K, elem_bytes, mx);
 }
 
 int launch_splitk_reduce(const float* partial, const GemmArgs& g, int out_dtype, hipStream_t stream) {

@@ -224,7 +224,7 @@ size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K,
 /* What mi355_gemm_tn would launch for this problem: the resolved variant (return value, or a
  * negative mi355_status), and for the tiled variants the tile (rows of A x rows of B per
  * workgroup), the uniform K split and the tail split (tiles of the last round cut along K;
- * 0 tiles / 1 split when there is none).  For the skinny variant tile_rows x 64 and its K split.
+ * 0 tiles / 1 split when there is none).  For the skinny variant its tile (rows of A x 64 or 128 rows of B) and its K split.
  * Any output pointer may be NULL.  Pure host function.  Counterpart in the reference: the
  * compile-time DefaultConfig (kernels/gemm_kernels/sm90a/gemm.cuh:420-451). */
 int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant,

@@ -660,6 +660,21 @@ def test_skinny_kernel_every_tile_height_and_split(abi, dt, M, N, K):
     assert oracle.rel_frobenius(C, oracle.c_gemm_tn_f32(A, B, 0.25)) <= TOL[dt]
 
 
+@pytest.mark.parametrize("dt,M,N,K", [(torch.bfloat16, 64, 8192, 4096), (torch.float16, 33, 8200, 4104), (torch.bfloat16, 50, 4100, 8200),
+                                      (torch.float16, 64, 20484, 520), (torch.float8_e4m3fn, 48, 8192, 8192),
+                                      (torch.float8_e4m3fn, 64, 4100, 16400), (torch.bfloat16, 40, 32768, 256)])
+def test_skinny_kernel_on_128_wide_tiles(abi, dt, M, N, K):
+    """33...64 rows against enough columns and k-steps: 64 x 128 tiles, split and unsplit, ragged M, N and K."""
+    plan = ac.plan(abi, M, N, K, ac.torch_code(dt), ac.SKINNY)
+    assert plan[:3] == (ac.SKINNY, 64, 128), plan
+    A = rand((M, K), M, torch.float32).clamp_(-50, 50).to(dt)
+    B = rand((N, K), N, torch.float32).clamp_(-50, 50).to(dt)
+    C = run_abi(abi, A, B, ac.SKINNY, 0.25)
+    check(C, A, B, 0.25)
+    assert oracle.rel_frobenius(C, oracle.c_gemm_tn_f32(A, B, 0.25)) <= TOL[dt]
+    assert torch.equal(run_abi(abi, A, B, ac.SKINNY, 0.25).view(torch.int16), C.view(torch.int16))
+
+
 @pytest.mark.parametrize("dt,M,N,K", [(torch.bfloat16, 16, 4096, 5696), (torch.bfloat16, 48, 4100, 11016),
                                       (torch.float8_e4m3fn, 64, 2048, 13584), (torch.float16, 200, 1024, 5768)])
 def test_skinny_k_split_that_does_not_divide_the_k_steps(abi, dt, M, N, K):
