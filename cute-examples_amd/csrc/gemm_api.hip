@@ -224,6 +224,7 @@ int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant, 
   if (v == MI355_VARIANT_SKINNY) {
     rows = M <= 16 ? 16 : M <= 32 ? 32 : M <= 64 ? 64 : M <= 128 ? 128 : 256;
     cols = mi355::stream_tile_cols(M, N, K, es);
+    if (cols == 128) rows = 64;   // the wide tile exists with 64 rows only
     splits = mi355::stream_splits(M, N, K, es);
   } else if (v == MI355_VARIANT_PINGPONG) {
     rows = cols = 256;

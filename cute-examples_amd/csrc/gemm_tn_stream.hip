@@ -26,9 +26,6 @@
 #include "ring_common.h"
 
 #include <type_traits>
-#ifdef MI355_EXPERIMENT
-#include <cstdlib>
-#endif
 
 namespace mi355 {
 namespace {
@@ -345,7 +342,7 @@ int splits_narrow(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
   return splits_for(M, N, K, elem_bytes, mx, tm, kTileN, depth);
 }
 
-// 64 x 128 tiles for 33...64 rows: a quarter fewer cache lines requested per output than 64 x 64 (192
+// 64 x 128 tiles, made for 33...64 rows: a quarter fewer cache lines requested per output than 64 x 64 (192
 // per 64 x 128 outputs and k-step against 2 x 128), paid for with half as many tiles to spread over the
 // CUs.  Measured against the 64 x 64 tiles on 112 bf16 problems (M = 48 and 64, N = 2048...32768,
 // K = 2048...14336, weights from HBM), each with its own best split: 3-16 % faster where 160-256 wide
@@ -355,13 +352,13 @@ int splits_narrow(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
 // N = 12288...16384, where the 64 x 64 tiles run unsplit on the deep ring.
 constexpr int kTileNWide = 128, kDepthWide = 3;
 bool wide_tiles(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
-#ifdef MI355_EXPERIMENT
-  if (getenv("MI355_STREAM_NOWIDE")) return false;
-  if (getenv("MI355_STREAM_ALLWIDE")) return !mx && M > 32 && M <= 64;
-#endif
-  if (mx || M <= 32 || M > 64) return false;
+  if (mx || M > 64) return false;
   const int64_t tiles = (N + kTileNWide - 1) / kTileNWide;
   const int64_t steps = (K * elem_bytes + kRowBytes - 1) / kRowBytes;
+  // Up to 32 rows the same tile (its lower half idle) wins only just above what the 64-column tiles
+  // cover in one round: N = 20480 and 24576 at M = 16...32 and K = 2048...8192 2-14 % faster, N = 28672
+  // the same, N = 32768 and N = 16384 0-4 % and 7-20 % slower.
+  if (M <= 32) return tiles >= 160 && tiles < 208;
   if (tiles >= 160) return tiles <= 256;
   if (tiles >= 64) return tiles < 96 && steps >= 64;
   return tiles >= 32 && steps >= 128;

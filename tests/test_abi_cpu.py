@@ -188,7 +188,8 @@ def test_plan(abi):
     assert ac.plan(abi, 64, 8192, 2048, ac.BF16)[1:3] == (64, 64)     # 32 k-steps: too few
     assert ac.plan(abi, 64, 8192, 4096, ac.E4M3)[1:3] == (64, 64)     # the same in fp8
     assert ac.plan(abi, 64, 8192, 8192, ac.E4M3)[1:3] == (64, 128)
-    assert ac.plan(abi, 32, 28672, 4096, ac.BF16)[1:3] == (32, 64)    # only the 64-row tile has a wide form
+    assert ac.plan(abi, 32, 28672, 4096, ac.BF16)[1:3] == (32, 64)
+    assert ac.plan(abi, 16, 24576, 4096, ac.BF16) == (ac.SKINNY, 64, 128, 1, 0, 1)   # the wide tile has 64 rows only
     assert ac.plan(abi, 100, 30, 77, ac.BF16)[0] == ac.SIMPLE
     assert ac.plan(abi, 256, 256, 68, ac.BF16, ac.BASIC)[0] == ac.ERR_SHAPE
     assert ac.plan(abi, 256, 256, 64, 7)[0] == ac.ERR_DTYPE
