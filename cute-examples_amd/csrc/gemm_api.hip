@@ -50,8 +50,11 @@ constexpr int64_t kSkinnyAutoMaxM = 64;
 // streaming weights (M*K*elem_bytes <= 2.2 MB): measured on 72 bf16 and fp8 problems with M = 96 and
 // 128 (N = 2048...16384), -6 % in the geometric mean where the rule applies, from -22 % to +10 %;
 // with more tiles the tile kernel is 14-20 % faster, with more bytes of A up to 40 % faster.
+// Of those, 16-bit problems with enough columns and k-steps go to the tile kernel's nine-slot ring
+// instead (ring_one_row_deep).
 bool auto_streams(int64_t M, int64_t N, int64_t K, int64_t es) {
   if (M <= kSkinnyAutoMaxM) return true;
+  if (mi355::ring_one_row_deep(M, N, K, (int)es)) return false;
   return M <= 128 && (N + 63) / 64 <= 256 && M * K * es <= 2200000;
 }
 bool skinny_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int in_dtype) {

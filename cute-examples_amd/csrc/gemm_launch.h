@@ -51,6 +51,9 @@ int launch_tile256_pingpong(const GemmArgs& g, int in_dtype, int out_dtype, hipS
 constexpr int kRingTile256x128 = 384;
 // 128 x 128 tile on the nine-slot ring (four k-steps of copies in flight, one workgroup per CU).
 constexpr int kRingTile128Deep = 129;
+// One row of 128 x 128 tiles that the tile kernel runs on the nine-slot ring, also where the streaming kernel could
+// take the problem (pure host function).
+bool ring_one_row_deep(int64_t M, int64_t N, int64_t K, int elem_bytes);
 inline int ring_tile_rows(int tile) { return tile == 128 || tile == kRingTile128Deep ? 128 : 256; }
 inline int ring_tile_cols(int tile) { return tile == 256 ? 256 : 128; }
 int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes);

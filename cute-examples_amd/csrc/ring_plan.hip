@@ -105,6 +105,22 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
 
 }  // namespace
 
+// One row of 128 x 128 tiles (M <= 128) of 16-bit operands on the nine-slot ring, K split as
+// uniform_splits says: every workgroup streams its own rows of B from HBM, and the ring that keeps
+// four k-steps in flight does that faster than the five-slot ring and than the streaming kernel's
+// 64-column tiles, which fetch the rows of A twice as often.  Measured, bf16, M = 72...128, weights
+// from HBM, against what the planner took before (the streaming kernel up to about 2 MB of A, else
+// the tile kernel's estimate): N = 4096...28672 x K = 1024...14336, 75 problems, 66 faster by 5-26 %
+// (128 x 8192 x 4096 26.9 -> 22.9 us, 96 x 11008 x 8192 64.9 -> 49.0 us, 80 x 14336 x 4096
+// 37.5 -> 30.1 us), 4 slower by 2-8 % (N = 11008 with K = 14336 or 2048); with 16...31 tiles from
+// 128 k-steps on 0-11 % faster; with fewer tiles or fewer k-steps than that the streaming kernel's
+// finer split wins by 6-23 %, and so it does at M <= 64 (0-21 %).
+bool ring_one_row_deep(int64_t M, int64_t N, int64_t K, int elem_bytes) {
+  if (elem_bytes != 2 || M > 128) return false;
+  const int64_t tiles = tiles_of(M, N, 128), steps = k_steps_of(K, elem_bytes);
+  return tiles <= kCuSlots && (tiles >= 32 || (tiles >= 16 && steps >= 128));
+}
+
 // Tile the single-group kernel should use (256, 128 or kRingTile256x128): the shortest estimate,
 // except that 256x256 is preferred over 256x128 within 5 % (it moves fewer bytes) and that a small
 // problem (at most two 128x128 tiles per CU) stays on 128x128 tiles unless a larger tile beats them
@@ -119,6 +135,7 @@ int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes) {
   // (256, 11008...14336, 2048...4096) and
   // (192, 14336, 4096): 3-10 % less time; with longer rows of K (from 5120 elements), more tiles than
   // CUs or fewer than two thirds of them it loses by 1-60 %.
+  if (ring_one_row_deep(M, N, K, elem_bytes)) return kRingTile128Deep;
   const int64_t small_tiles = tiles_of(M, N, 128);
   if (elem_bytes == 2 && M <= 256 && small_tiles >= 170 && small_tiles <= kCuSlots && k_steps_of(K, elem_bytes) >= 16 &&
       k_steps_of(K, elem_bytes) <= 64)

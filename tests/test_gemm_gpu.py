@@ -644,6 +644,20 @@ def test_one_or_two_tile_rows_on_the_nine_slot_ring(abi, dt, M, N, K):
     assert oracle.rel_frobenius(C[:, :2048], small) < 2e-3
 
 
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K", [(128, 8192, 4096), (100, 4100, 8200), (72, 2052, 8200), (65, 28672, 520), (90, 6144, 4096)])
+def test_one_tile_row_with_k_splits_on_the_nine_slot_ring(abi, dt, M, N, K):
+    """65...128 rows: AUTO takes the tile kernel's 128x128 tiles on the nine-slot ring, K split evenly or not
+    (129 k-steps in 7 and in 8 parts, the last k-step ragged), ragged M and N, and unsplit."""
+    v, rows, cols, splits, _, _ = ac.plan(abi, M, N, K, ac.torch_code(dt))
+    assert (v, rows, cols) == (ac.BASIC, 128, 128) and (splits > 1) == (N < 28672), (v, rows, cols, splits)
+    A, B = rand((M, K), M, dt), rand((N, K), N + 1, dt, 0.05)
+    C = run_abi(abi, A, B, ac.AUTO, 0.5)
+    check(C, A, B, 0.5)
+    assert oracle.rel_frobenius(C, oracle.c_gemm_tn_f32(A, B, 0.5)) <= TOL[dt]
+    assert torch.equal(run_abi(abi, A, B, ac.AUTO, 0.5).view(torch.int16), C.view(torch.int16))
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 512, 128), (16, 128, 8), (48, 260, 1096), (256, 64, 4104), (10, 260, 256), (17, 64, 1024), (33, 512, 4096),
                                    (64, 1024, 2048), (100, 640, 1024), (129, 72, 512), (256, 768, 2048)])
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
@@ -692,7 +706,7 @@ def test_skinny_k_split_that_does_not_divide_the_k_steps(abi, dt, M, N, K):
     assert torch.equal(run_abi(abi, A, B, ac.SKINNY, 0.25).view(torch.int16), C.view(torch.int16))
 
 
-@pytest.mark.parametrize("M,N,K", [(16, 4096, 14336), (90, 6144, 4096)])
+@pytest.mark.parametrize("M,N,K", [(16, 4096, 14336), (90, 2048, 4096)])
 def test_auto_without_a_workspace_takes_the_tile_kernel_for_few_rows(abi, M, N, K):
     """The streaming kernel's K split needs a workspace; MI355_VARIANT_AUTO called without one still
     succeeds (on the tile kernel, unsplit), an explicit MI355_VARIANT_SKINNY does not."""
