@@ -50,8 +50,8 @@ constexpr int64_t kSkinnyAutoMaxM = 64;
 // streaming weights (M*K*elem_bytes <= 2.2 MB): measured on 72 bf16 and fp8 problems with M = 96 and
 // 128 (N = 2048...16384), -6 % in the geometric mean where the rule applies, from -22 % to +10 %;
 // with more tiles the tile kernel is 14-20 % faster, with more bytes of A up to 40 % faster.
-// Of those, 16-bit problems with enough columns and k-steps go to the tile kernel's nine-slot ring
-// instead (ring_one_row_deep).
+// Of those, problems with enough columns and k-steps go to the tile kernel's nine-slot ring instead
+// (ring_one_row_deep).
 bool auto_streams(int64_t M, int64_t N, int64_t K, int64_t es) {
   if (M <= kSkinnyAutoMaxM) return true;
   if (mi355::ring_one_row_deep(M, N, K, (int)es)) return false;
@@ -327,8 +327,8 @@ int mx_stream_splits(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, 
 }
 
 size_t mx_partial_bytes(int64_t M, int64_t N, int64_t K, int* splits, int* tail_tiles, int* tail_splits) {
-  int s = mi355::ring_splits(M, N, K, 1), tt = 0, ts = 1;
-  size_t bytes = s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : mi355::ring_tail(M, N, K, 1, &tt, &ts);
+  int s = mi355::ring_splits(M, N, K, 1, true), tt = 0, ts = 1;
+  size_t bytes = s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : mi355::ring_tail(M, N, K, 1, &tt, &ts, true);
   if (splits) *splits = s;
   if (tail_tiles) *tail_tiles = tt;
   if (tail_splits) *tail_splits = ts;
@@ -406,7 +406,7 @@ int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, in
     g.tail_tiles = tail_tiles;
     g.tail_splits = tail_splits;
   }
-  const int tile = mi355::ring_tile_edge(M, N, K, 1);
+  const int tile = mi355::ring_tile_edge(M, N, K, 1, true);
   g.tiles_m = (M + mi355::ring_tile_rows(tile) - 1) / mi355::ring_tile_rows(tile);
   g.tiles_n = (N + mi355::ring_tile_cols(tile) - 1) / mi355::ring_tile_cols(tile);
   return mi355::launch_tile_ring_mx(g, out_dtype, tile, s) == 0 ? MI355_OK : MI355_ERR_LAUNCH;

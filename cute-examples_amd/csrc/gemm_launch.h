@@ -56,14 +56,15 @@ constexpr int kRingTile128Deep = 129;
 bool ring_one_row_deep(int64_t M, int64_t N, int64_t K, int elem_bytes);
 inline int ring_tile_rows(int tile) { return tile == 128 || tile == kRingTile128Deep ? 128 : 256; }
 inline int ring_tile_cols(int tile) { return tile == 256 ? 256 : 128; }
-int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes);
-int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes);
+// block_scaled: for the kernel with block scales, which exists on the five-slot ring only.
+int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_scaled = false);
+int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_scaled = false);
 // C = rne(scale * sum_s partial[s]) for partial laid out [splits][M][N] in fp32.
 int launch_splitk_reduce(const float* partial, const GemmArgs& g, int out_dtype, hipStream_t stream);
 int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, hipStream_t stream);
 // Tail split the single-group kernel would use for this problem (pure host heuristic): returns the
 // workspace bytes it needs (0 = no tail split) and sets *tail_tiles, *tail_splits.
-size_t ring_tail(int64_t M, int64_t N, int64_t K, int elem_bytes, int* tail_tiles, int* tail_splits);
+size_t ring_tail(int64_t M, int64_t N, int64_t K, int elem_bytes, int* tail_tiles, int* tail_splits, bool block_scaled = false);
 int launch_tile_ring_mx(const GemmArgs& g, int out_dtype, int tile, hipStream_t stream);
 // Per-input-type halves of launch_tile_ring (one translation unit each).
 int launch_tile_ring_bf16(const GemmArgs& g, int out_dtype, int tile, hipStream_t stream);

@@ -619,8 +619,8 @@ int launch_tile(const GemmArgs& g, hipStream_t stream) {
 template <class T, class OutT>
 int launch(const GemmArgs& g, int tile, hipStream_t stream) {
   if (tile == kRingTile256x128) return launch_tile<T, OutT, 256, 128>(g, stream);
-  if (tile == kRingTile128Deep) {   // the planner picks it for 16-bit inputs only
-    if constexpr (T::kBytes == 2) return launch_tile<T, OutT, 128, 128, 4>(g, stream);
+  if (tile == kRingTile128Deep) {   // the planner does not pick it with block scales (their registers are timed for five slots)
+    if constexpr (!std::is_same<T, MxE4M3>::value) return launch_tile<T, OutT, 128, 128, 4>(g, stream);
     else return -1;
   }
   return tile == 128 ? launch_tile<T, OutT, 128>(g, stream) : launch_tile<T, OutT, 256>(g, stream);

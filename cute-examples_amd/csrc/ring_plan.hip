@@ -105,7 +105,7 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
 
 }  // namespace
 
-// One row of 128 x 128 tiles (M <= 128) of 16-bit operands on the nine-slot ring, K split as
+// One row of 128 x 128 tiles (M <= 128) on the nine-slot ring, K split as
 // uniform_splits says: every workgroup streams its own rows of B from HBM, and the ring that keeps
 // four k-steps in flight does that faster than the five-slot ring and than the streaming kernel's
 // 64-column tiles, which fetch the rows of A twice as often.  Measured, bf16, M = 72...128, weights
@@ -114,11 +114,13 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
 // (128 x 8192 x 4096 26.9 -> 22.9 us, 96 x 11008 x 8192 64.9 -> 49.0 us, 80 x 14336 x 4096
 // 37.5 -> 30.1 us), 4 slower by 2-8 % (N = 11008 with K = 14336 or 2048); with 16...31 tiles from
 // 128 k-steps on 0-11 % faster; with fewer tiles or fewer k-steps than that the streaming kernel's
-// finer split wins by 6-23 %, and so it does at M <= 64 (0-21 %).
+// finer split wins by 6-23 %, and so it does at M <= 64 (0-21 %).  e4m3, M = 72...128, N = 4096...28672,
+// K = 4096...16384: 41 of 45 problems 5-24 % faster, the rest (32 k-steps, 32 tiles) within 3 %.
 bool ring_one_row_deep(int64_t M, int64_t N, int64_t K, int elem_bytes) {
-  if (elem_bytes != 2 || M > 128) return false;
+  if (M > 128) return false;
   const int64_t tiles = tiles_of(M, N, 128), steps = k_steps_of(K, elem_bytes);
-  return tiles <= kCuSlots && (tiles >= 32 || (tiles >= 16 && steps >= 128));
+  if (tiles > kCuSlots || tiles * uniform_splits(tiles, steps) < 96) return false;   // under 96 items: no gain, or 1-3 % slower
+  return tiles >= 32 || (tiles >= 16 && steps >= 128);
 }
 
 // Tile the single-group kernel should use (256, 128 or kRingTile256x128): the shortest estimate,
@@ -127,7 +129,7 @@ bool ring_one_row_deep(int64_t M, int64_t N, int64_t K, int elem_bytes) {
 // by 10 %, a larger one unless beaten by 6 %.  (With 10 % for all sizes the small tile was
 // picked on large problems where 256x256 measured 20-40 % faster; with no margin on mid-sized fp8
 // problems where the small tile measured 7-15 % faster.  Mean regret over 124 measured problems: 0.9 %.)
-int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes) {
+int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_scaled) {
   // One or two rows of 128 x 128 tiles that nearly fill the CUs in one round, and a short K: every
   // workgroup streams its own rows of B from HBM, which the nine-slot ring keeps further ahead of the
   // MFMAs than the five-slot one can, and unsplit tiles spare the partial planes of a K split.
@@ -135,7 +137,7 @@ int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes) {
   // (256, 11008...14336, 2048...4096) and
   // (192, 14336, 4096): 3-10 % less time; with longer rows of K (from 5120 elements), more tiles than
   // CUs or fewer than two thirds of them it loses by 1-60 %.
-  if (ring_one_row_deep(M, N, K, elem_bytes)) return kRingTile128Deep;
+  if (!block_scaled && ring_one_row_deep(M, N, K, elem_bytes)) return kRingTile128Deep;   // scales: five-slot ring only
   const int64_t small_tiles = tiles_of(M, N, 128);
   if (elem_bytes == 2 && M <= 256 && small_tiles >= 170 && small_tiles <= kCuSlots && k_steps_of(K, elem_bytes) >= 16 &&
       k_steps_of(K, elem_bytes) <= 64)
@@ -150,16 +152,16 @@ int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes) {
 }
 
 // K splits for the single-group kernel on the tile ring_tile_edge picks.
-int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes) {
-  return uniform_splits(tiles_of(M, N, ring_tile_edge(M, N, K, elem_bytes)), k_steps_of(K, elem_bytes));
+int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_scaled) {
+  return uniform_splits(tiles_of(M, N, ring_tile_edge(M, N, K, elem_bytes, block_scaled)), k_steps_of(K, elem_bytes));
 }
 
 // The tail split (tail_plan) of this problem, if it runs on 256x256 tiles without a uniform K
 // split: returns the workspace bytes of its partial tiles.
-size_t ring_tail(int64_t M, int64_t N, int64_t K, int elem_bytes, int* tail_tiles, int* tail_splits) {
+size_t ring_tail(int64_t M, int64_t N, int64_t K, int elem_bytes, int* tail_tiles, int* tail_splits, bool block_scaled) {
   *tail_tiles = 0;
   *tail_splits = 1;
-  if (M <= 0 || N <= 0 || K <= 0 || ring_tile_edge(M, N, K, elem_bytes) != 256) return 0;
+  if (M <= 0 || N <= 0 || K <= 0 || ring_tile_edge(M, N, K, elem_bytes, block_scaled) != 256) return 0;
   tail_plan(tiles_of(M, N, 256), k_steps_of(K, elem_bytes), tail_tiles, tail_splits);
   return (size_t)*tail_tiles * (size_t)*tail_splits * 256 * 256 * sizeof(float);
 }

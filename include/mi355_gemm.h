@@ -172,7 +172,8 @@ int mi355_quantize_e4m3(const void *x, int x_dtype, int64_t n, void *x_q,
  * N % 4 == 0, ldc % 4 == 0, C 8-byte aligned; the size limits of the tiled variants.  Runs the
  * weight-streaming kernel (MI355_VARIANT_SKINNY) for M <= 64 and otherwise the tiled kernel
  * (MI355_VARIANT_BASIC) with the tile and splits mi355_gemm_plan reports for MI355_E4M3 operands
- * of this shape and that variant.
+ * of this shape and that variant (except with 65...128 rows, where plain operands may get a ring
+ * that the block-scaled kernel does not have and this call keeps the planner's other choice).
  * Counterpart in the reference: none (it has no fp8 path); same launcher contract as
  * mi355_gemm_tn (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92), block format per the OCP
  * Microscaling Formats (MX) specification v1.0.

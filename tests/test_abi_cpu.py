@@ -190,11 +190,12 @@ def test_plan(abi):
     assert ac.plan(abi, 64, 8192, 8192, ac.E4M3)[1:3] == (64, 128)
     assert ac.plan(abi, 32, 28672, 4096, ac.BF16)[1:3] == (32, 64)
     assert ac.plan(abi, 16, 24576, 4096, ac.BF16) == (ac.SKINNY, 64, 128, 1, 0, 1)   # the wide tile has 64 rows only
-    # 65...128 rows of 16-bit operands against 4096...32768 columns: the tile kernel, one row of 128x128 tiles, K split
+    # 65...128 rows against 4096...32768 columns: the tile kernel, one row of 128x128 tiles, K split
     assert ac.plan(abi, 128, 8192, 4096, ac.BF16) == (ac.BASIC, 128, 128, 4, 0, 1)
     assert ac.plan(abi, 100, 4100, 8200, ac.F16) == (ac.BASIC, 128, 128, 7, 0, 1)      # 33 tiles, 129 k-steps
     assert ac.plan(abi, 96, 2048, 4096, ac.BF16)[0] == ac.SKINNY                        # 16 tiles, 64 k-steps: streams
-    assert ac.plan(abi, 96, 8192, 8192, ac.E4M3)[0] == ac.SKINNY                        # fp8 keeps streaming
+    assert ac.plan(abi, 96, 8192, 8192, ac.E4M3) == (ac.BASIC, 128, 128, 4, 0, 1)       # 64 tiles of 64 k-steps, in four parts
+    assert ac.plan(abi, 96, 4096, 4096, ac.E4M3)[0] == ac.SKINNY                        # 32 tiles x 2 parts: too few items
     assert ac.plan(abi, 100, 30, 77, ac.BF16)[0] == ac.SIMPLE
     assert ac.plan(abi, 256, 256, 68, ac.BF16, ac.BASIC)[0] == ac.ERR_SHAPE
     assert ac.plan(abi, 256, 256, 64, 7)[0] == ac.ERR_DTYPE
@@ -305,8 +306,9 @@ def test_plan_invariants_over_random_shapes(abi):
             v, rows, cols, splits, tail_tiles, tail_splits = ac.plan(abi, M, N, K, dt)
             steps = -(-K * es // 128)
             assert v in (ac.BASIC, ac.SKINNY), (M, N, K, v)
-            one_row = -(-N // 128)      # 65...128 rows of 16-bit operands: one row of 128x128 tiles on the nine-slot ring
-            deep = es == 2 and M <= 128 and one_row <= 256 and (one_row >= 32 or (one_row >= 16 and steps >= 128))
+            one_row = -(-N // 128)      # 65...128 rows: one row of 128x128 tiles on the nine-slot ring
+            parts = max([1] + [p for p in range(2, 17) if one_row * p <= 256 and steps // p >= 16])
+            deep = M <= 128 and one_row <= 256 and one_row * parts >= 96 and (one_row >= 32 or (one_row >= 16 and steps >= 128))
             assert (v == ac.SKINNY) == (M <= 64 or (not deep and M <= 128 and -(-N // 64) <= 256 and M * K * es <= 2200000))
             if deep and M > 64:
                 assert (v, rows, cols) == (ac.BASIC, 128, 128), (M, N, K)

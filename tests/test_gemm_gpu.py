@@ -644,14 +644,20 @@ def test_one_or_two_tile_rows_on_the_nine_slot_ring(abi, dt, M, N, K):
     assert oracle.rel_frobenius(C[:, :2048], small) < 2e-3
 
 
-@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,N,K", [(128, 8192, 4096), (100, 4100, 8200), (72, 2052, 8200), (65, 28672, 520), (90, 6144, 4096)])
+@pytest.mark.parametrize("dt,M,N,K", [(dt, M, N, K) for dt in (torch.bfloat16, torch.float16) for M, N, K in
+                                      [(128, 8192, 4096), (100, 4100, 8200), (72, 2052, 8200), (65, 28672, 520), (90, 6144, 4096)]] +
+                         [(torch.float8_e4m3fn, 128, 8192, 4096), (torch.float8_e4m3fn, 100, 4100, 8208),
+                          (torch.float8_e4m3fn, 72, 2052, 16400), (torch.float8_e4m3fn, 65, 28672, 528)])
 def test_one_tile_row_with_k_splits_on_the_nine_slot_ring(abi, dt, M, N, K):
     """65...128 rows: AUTO takes the tile kernel's 128x128 tiles on the nine-slot ring, K split evenly or not
     (129 k-steps in 7 and in 8 parts, the last k-step ragged), ragged M and N, and unsplit."""
     v, rows, cols, splits, _, _ = ac.plan(abi, M, N, K, ac.torch_code(dt))
     assert (v, rows, cols) == (ac.BASIC, 128, 128) and (splits > 1) == (N < 28672), (v, rows, cols, splits)
-    A, B = rand((M, K), M, dt), rand((N, K), N + 1, dt, 0.05)
+    if dt == torch.float8_e4m3fn:
+        A = rand((M, K), M, torch.float32).clamp_(-50, 50).to(dt)
+        B = rand((N, K), N + 1, torch.float32, 0.05).to(dt)
+    else:
+        A, B = rand((M, K), M, dt), rand((N, K), N + 1, dt, 0.05)
     C = run_abi(abi, A, B, ac.AUTO, 0.5)
     check(C, A, B, 0.5)
     assert oracle.rel_frobenius(C, oracle.c_gemm_tn_f32(A, B, 0.5)) <= TOL[dt]
