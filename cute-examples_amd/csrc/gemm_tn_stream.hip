@@ -3,10 +3,11 @@
 // C[M,N] = scale * X[M,K] · W[N,K]^T with M <= 256 is bound by reading W once from HBM, so the
 // kernel is built around keeping many bytes of W in flight per CU rather than around MFMA issue:
 //
-//   * output tile TM x 64 with TM = 16/32/64/128/256 >= M; the grid is (N/64 tiles) x (K splits),
-//     several workgroups resident per CU (the LDS ring of one workgroup is 30-120 KiB), or, when
-//     the tiles alone occupy most CUs, no K split and a deeper ring (see unsplit_deep);
-//   * per k-step (128 B of K per row) the TM rows of X and 64 rows of W go global -> LDS with
+//   * output tile TM x 64 with TM = 16/32/64/128/256 >= M, or 64 x 128 (see wide_tiles); the grid
+//     is (tiles along N) x (K splits), several workgroups resident per CU (the LDS ring of one
+//     workgroup is 30-120 KiB), or, when the tiles alone occupy most CUs, no K split and a deeper
+//     ring (see unsplit_deep);
+//   * per k-step (128 B of K per row) the TM rows of X and the 64 or 128 rows of W go global -> LDS with
 //     full-cache-line direct-to-LDS loads into a ring of kDepth stages, kDepth-1 k-steps ahead;
 //   * the four waves read MFMA fragments from LDS (same 16-byte-chunk swizzle as the big-tile
 //     kernels) and run v_mfma_f32_16x16x32 (two per k-step and block pair) or, for fp8,
