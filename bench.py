@@ -45,14 +45,15 @@ PEAK_HBM_GBS = 8000.0
 # reads for the 1 GiB copy: x2.000 and x1.000).  Workloads without a counter run report null.
 MEASURED_TRAFFIC_BYTES = {"bf16_8192": 1.746e9, "fp8_8192": 0.970e9, "mxfp8_8192": 0.965e9, "bf16_4096": 2.352e8,
                           "skinny_16_14336_4096": 1.190e8, "skinny_64_14336_4096": 1.236e8, "skinny_64_4096_14336": 1.900e8,
-                          "skinny_256_14336_4096": 1.546e8, "skinny_256_6144_4096": 1.209e8}
+                          "skinny_256_14336_4096": 1.546e8, "skinny_256_6144_4096": 1.209e8, "skinny_128_8192_4096": 1.130e8}
 TRAFFIC_PROFILE = {"bf16_8192": "profiles/gemm_tn_tile_ring__bf16_8192.md", "fp8_8192": "profiles/gemm_tn_tile_ring__fp8_8192.md",
                    "mxfp8_8192": "profiles/gemm_tn_tile_ring__mxfp8_8192.md", "bf16_4096": "profiles/gemm_tn_tile_ring__bf16_4096.md",
                    "skinny_16_14336_4096": "profiles/gemm_tn_stream__skinny_16_14336_4096.md",
                    "skinny_64_14336_4096": "profiles/gemm_tn_stream__skinny_64_14336_4096.md",
                    "skinny_64_4096_14336": "profiles/gemm_tn_stream__skinny_64_4096_14336.md",
                    "skinny_256_14336_4096": "profiles/gemm_tn_tile_ring__skinny_256_14336_4096.md",
-                   "skinny_256_6144_4096": "profiles/gemm_tn_tile_ring__skinny_256_6144_4096.md"}
+                   "skinny_256_6144_4096": "profiles/gemm_tn_tile_ring__skinny_256_6144_4096.md",
+                   "skinny_128_8192_4096": "profiles/gemm_tn_tile_ring__skinny_128_8192_4096.md"}
 SETTLE_MIN_MS, SETTLE_MAX_MS, SETTLE_BATCH_MS = 150.0, 2000.0, 10.0
 
 
@@ -400,7 +401,7 @@ def main():
     if not a.no_extras:
         names = ["bf16_8192", "fp8_8192", "mxfp8_8192", "bf16_4096", "fp16_512"] + \
                 ["skinny_%d_%d_%d" % (m, n, k) for (n, k) in ((14336, 4096), (4096, 14336), (6144, 4096))
-                 for m in (16, 64, 256)] + ["skinnyfp8_16_14336_4096", "skinnymx_16_14336_4096"]
+                 for m in (16, 64, 256)] + ["skinny_128_8192_4096", "skinnyfp8_16_14336_4096", "skinnymx_16_14336_4096"]
         for n in names:
             if n == a.workload or (n == "fp8_8192" and fp8_block):
                 continue
