@@ -105,7 +105,7 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
 
 }  // namespace
 
-// One row of 128 x 128 tiles (M <= 128) on the nine-slot ring, K split as
+// One row (M <= 128) or one column (N <= 128) of 128 x 128 tiles on the nine-slot ring, K split as
 // uniform_splits says: every workgroup streams its own rows of B from HBM, and the ring that keeps
 // four k-steps in flight does that faster than the five-slot ring and than the streaming kernel's
 // 64-column tiles, which fetch the rows of A twice as often.  Measured, bf16, M = 72...128, weights
@@ -117,9 +117,15 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
 // finer split wins by 6-23 %, and so it does at M <= 64 (0-21 %).  e4m3, M = 72...128, N = 4096...28672,
 // K = 4096...16384: 41 of 45 problems 5-24 % faster, the rest (32 k-steps, 32 tiles) within 3 %.
 bool ring_one_row_deep(int64_t M, int64_t N, int64_t K, int elem_bytes) {
-  if (M > 128) return false;
+  if (M > 128 && N > 128) return false;
   const int64_t tiles = tiles_of(M, N, 128), steps = k_steps_of(K, elem_bytes);
   if (tiles > kCuSlots || tiles * uniform_splits(tiles, steps) < 96) return false;   // under 96 items: no gain, or 1-3 % slower
+  // One column of tiles (N <= 128 under many rows: router and adapter projections) is the same picture
+  // with the operands' roles exchanged.  bf16, N = 64 and 128, K = 2048...7168 against the estimate's
+  // choice (mostly 256 x 128 tiles): M = 8192...32768 19 of 24 problems 3-41 % faster (32768 x 128 x 4096
+  // 76 -> 45 us), the rest within 4 %; M = 4096 (32 tiles) from 5 % faster to 10 % slower, so from 64 tiles on;
+  // e4m3 on seven such problems 1-31 % faster.
+  if (M > 128) return tiles >= 64 && steps >= 16;   // (e4m3 24576 x 128 x 1024, 8 k-steps: 11 % slower)
   return tiles >= 32 || (tiles >= 16 && steps >= 128);
 }
 

@@ -196,6 +196,9 @@ def test_plan(abi):
     assert ac.plan(abi, 96, 2048, 4096, ac.BF16)[0] == ac.SKINNY                        # 16 tiles, 64 k-steps: streams
     assert ac.plan(abi, 96, 8192, 8192, ac.E4M3) == (ac.BASIC, 128, 128, 4, 0, 1)       # 64 tiles of 64 k-steps, in four parts
     assert ac.plan(abi, 96, 4096, 4096, ac.E4M3)[0] == ac.SKINNY                        # 32 tiles x 2 parts: too few items
+    # one column of 128x128 tiles under many rows: the same ring
+    assert ac.plan(abi, 32768, 128, 4096, ac.BF16) == (ac.BASIC, 128, 128, 1, 0, 1)
+    assert ac.plan(abi, 8192, 96, 8192, ac.E4M3) == (ac.BASIC, 128, 128, 4, 0, 1)
     assert ac.plan(abi, 100, 30, 77, ac.BF16)[0] == ac.SIMPLE
     assert ac.plan(abi, 256, 256, 68, ac.BF16, ac.BASIC)[0] == ac.ERR_SHAPE
     assert ac.plan(abi, 256, 256, 64, 7)[0] == ac.ERR_DTYPE

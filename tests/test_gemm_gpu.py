@@ -664,6 +664,22 @@ def test_one_tile_row_with_k_splits_on_the_nine_slot_ring(abi, dt, M, N, K):
     assert torch.equal(run_abi(abi, A, B, ac.AUTO, 0.5).view(torch.int16), C.view(torch.int16))
 
 
+@pytest.mark.parametrize("dt,M,N,K", [(torch.bfloat16, 8200, 128, 4096), (torch.float16, 12289, 100, 2056), (torch.float8_e4m3fn, 8192, 96, 8208),
+                                      (torch.bfloat16, 32768, 64, 1024)])
+def test_one_tile_column_on_the_nine_slot_ring(abi, dt, M, N, K):
+    """Many rows against at most 128 columns: one column of 128x128 tiles on the nine-slot ring, with and without a K split."""
+    v, rows, cols, splits, _, _ = ac.plan(abi, M, N, K, ac.torch_code(dt))
+    assert (v, rows, cols) == (ac.BASIC, 128, 128), (v, rows, cols, splits)
+    if dt == torch.float8_e4m3fn:
+        A = rand((M, K), M, torch.float32).clamp_(-50, 50).to(dt)
+        B = rand((N, K), N + 1, torch.float32, 0.05).to(dt)
+    else:
+        A, B = rand((M, K), M, dt), rand((N, K), N + 1, dt, 0.05)
+    C = run_abi(abi, A, B, ac.AUTO, 0.5)
+    check(C, A, B, 0.5)
+    assert torch.equal(run_abi(abi, A, B, ac.AUTO, 0.5).view(torch.int16), C.view(torch.int16))
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 64, 128), (16, 512, 128), (16, 128, 8), (48, 260, 1096), (256, 64, 4104), (10, 260, 256), (17, 64, 1024), (33, 512, 4096),
                                    (64, 1024, 2048), (100, 640, 1024), (129, 72, 512), (256, 768, 2048)])
 @pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16, torch.float8_e4m3fn])
