@@ -11,7 +11,6 @@ namespace mi355 {
 namespace {
 
 constexpr int64_t kCuSlots = 256;  // one work item per CU of an MI355X; heuristics only, so no device query
-constexpr int64_t kSmallProblemTiles = 2 * kCuSlots;  // 128x128 tiles that are resident all at once
 
 int64_t k_steps_of(int64_t K, int elem_bytes) { return (K * elem_bytes + kRowBytes - 1) / kRowBytes; }
 
@@ -59,48 +58,69 @@ void tail_plan(int64_t tiles, int64_t steps, int* tail_tiles, int* tail_splits) 
   *tail_splits = best;
 }
 
-// Estimated duration, in microseconds, of the problem on tile shape `tile`, fitted to timings of
-// 124 bf16 and fp8 problems of 1-400 GFLOP per tile shape:
-//   rounds x (k-steps per item x time of a k-step + start-up and store of a tile) + reduce
+// Estimated duration, in microseconds, of the problem on tile shape `tile`: linear models.  For the two
+// large tiles, of which a CU holds one,
+//   rounds x k-steps per item x (step + step_busy x occupancy + few_rows / tile rows + few_cols / tile columns)
+//   + rounds x fixed + (reduce_mb x MB of partial sums + reduce, if K is split),
+// rounds = ceil(items / 256), occupancy = items / (rounds x 256) -- a k-step of a busy chip takes longer
+// (lower clock, shared memory system) -- and the two sharing terms for operands that few tiles share and
+// that therefore come from HBM rather than from an XCD's L2 (few tile rows: the rows of B; few tile
+// columns: the rows of A).  Of the 128 x 128 tiles a CU holds two, which hide each other's waits: a round
+// of up to 512 items in which some CU has two costs `pair` per k-step (less `pair_slack` x the unused
+// share of the 512 places), a last round of at most 256 items `single + single_busy x occupancy`.
 // A k-step is 128 bytes of K per row for every input type and takes the same time for all of them.
-//   256x256  1.45 us when (nearly) all CUs are busy, 1.2 us otherwise (higher clock), also in a last
-//            round that is not nearly full; a last round that gets a tail split counts 1/S of a
-//            round plus 0.2
-//   256x128  0.85 us: half the MFMA work of a 256x256 tile, three quarters of its copies
-//   128x128  0.45 us + 1/800 us per k-step of the item (a quarter of the work, half of the copies; 0.49 us
-//            measured at 32 k-steps, 0.61 at 128: long items run at a lower clock), 0.75 us when either
-//            dimension has fewer than 16 tiles (measured; such problems re-read one operand from far away)
-//   reduce   the partial planes are read back at about 5 TB/s, plus a launch
+// Coefficients: weighted least squares (relative error) over 200 bf16 problems drawn log-uniformly from
+// M, N = 256...32768, K = 1024...16384 (1-800 GFLOP), each timed on all three tiles with the rows of B
+// rotating through 600 MB so that they come from memory as weights do; residuals 7-9 % rms.  Picking the
+// shortest estimate costs 0.4 % of the best tile's time on average over those problems (0.45 % and 0.5 %
+// when fitted on one part of them and scored on the other), against 3.6 % for the model this replaces,
+// whose constants came from squarer problems and cache-resident operands (its worst choices, 25-45 %
+// slower than the best tile, were 256 x 256 tiles on problems with a few tile rows and thousands of
+// columns, or the reverse).
+struct TileCost {
+  double step, step_busy, few_rows, few_cols, fixed, reduce_mb, reduce;
+};
+constexpr TileCost kCost256x128 = {0.380, 0.449, 0.163, 0.098, 8.02, 0.191, 2.07};
+constexpr TileCost kCost256 = {0.580, 0.878, 0.220, 0.0, 15.72, 0.093, 2.64};
+struct SmallTileCost {
+  double pair, pair_slack, single, single_busy, few_rows, fixed, reduce_mb, reduce;
+};
+constexpr SmallTileCost kCost128 = {0.990, 0.498, 0.244, 0.352, 0.519, 5.53, 0.101, 1.71};
+
 double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
   const int64_t rows = ring_tile_rows(tile), cols = ring_tile_cols(tile);
   const int64_t tm = (M + rows - 1) / rows, tn = (N + cols - 1) / cols, tiles = tm * tn;
   const int64_t steps = k_steps_of(K, elem_bytes);
   const int s = uniform_splits(tiles, steps);
   const int64_t items = tiles * s;
+  const double item_steps = (double)steps / s;
+  double partial_mb = s > 1 ? (double)s * (double)M * (double)N * 4.0e-6 : 0.0;
+  if (tile != 256 && tile != kRingTile256x128) {
+    const SmallTileCost& c = kCost128;
+    const int64_t full = items / (2 * kCuSlots), rest = items - full * 2 * kCuSlots;
+    const bool pair = rest > kCuSlots, single = rest > 0 && !pair;
+    const double pair_rounds = (double)(full + (pair ? 1 : 0));
+    const double slack = pair ? 1.0 - (double)rest / (double)(2 * kCuSlots) : 0.0;
+    const double rounds = pair_rounds + (single ? 1.0 : 0.0);
+    const double step_sum = c.pair * pair_rounds - c.pair_slack * slack +
+                            (single ? c.single + c.single_busy * (double)rest / (double)kCuSlots : 0.0) +
+                            c.few_rows * rounds / (double)tm;
+    return item_steps * step_sum + c.fixed * rounds + (partial_mb > 0.0 ? c.reduce_mb * partial_mb + c.reduce : 0.0);
+  }
+  const TileCost& c = tile == 256 ? kCost256 : kCost256x128;
   double rounds = (double)((items + kCuSlots - 1) / kCuSlots);
-  double step_us, fixed_us;
-  if (tile == 256) {
-    step_us = items >= 224 ? 1.45 : 1.2;
-    fixed_us = 6.0;
+  double occupancy = (double)items / (rounds * (double)kCuSlots);
+  if (tile == 256 && s == 1) {
     int tail_tiles, tail_splits;
     tail_plan(tiles, steps, &tail_tiles, &tail_splits);
-    if (tail_tiles) {
-      rounds = (double)(tiles / kCuSlots) + 1.0 / tail_splits + 0.2;
-    } else if (s == 1 && items > kCuSlots) {
-      // full rounds, then a last round that runs at the higher clock unless it is (nearly) full too
-      const int64_t rest = items % kCuSlots;
-      const double last = rest == 0 ? 0.0 : (double)steps * (rest >= 224 ? 1.45 : 1.2) + fixed_us;
-      return (double)(items / kCuSlots) * ((double)steps * 1.45 + fixed_us) + last;
+    if (tail_tiles) {   // the last round takes 1/S of a round
+      rounds = (double)(tiles / kCuSlots) + 1.0 / tail_splits;
+      occupancy = 1.0;
+      partial_mb = (double)tail_tiles * tail_splits * 256.0 * 256.0 * 4.0e-6;
     }
-  } else if (tile == kRingTile256x128) {
-    step_us = 0.85;
-    fixed_us = 6.0;
-  } else {
-    step_us = (tm < tn ? tm : tn) >= 16 ? 0.45 + 0.00125 * (double)(steps / s) : 0.75;
-    fixed_us = 4.0;
   }
-  const double reduce_us = s > 1 ? (double)s * (double)M * (double)N * 4.0 / 5.0e6 + 2.0 : 0.0;
-  return rounds * ((double)steps / s * step_us + fixed_us) + reduce_us;
+  const double step_us = c.step + c.step_busy * occupancy + c.few_rows / (double)tm + c.few_cols / (double)tn;
+  return rounds * (item_steps * step_us + c.fixed) + (partial_mb > 0.0 ? c.reduce_mb * partial_mb + c.reduce : 0.0);
 }
 
 }  // namespace
@@ -129,12 +149,9 @@ bool ring_one_row_deep(int64_t M, int64_t N, int64_t K, int elem_bytes) {
   return tiles >= 32 || (tiles >= 16 && steps >= 128);
 }
 
-// Tile the single-group kernel should use (256, 128 or kRingTile256x128): the shortest estimate,
-// except that 256x256 is preferred over 256x128 within 5 % (it moves fewer bytes) and that a small
-// problem (at most two 128x128 tiles per CU) stays on 128x128 tiles unless a larger tile beats them
-// by 10 %, a larger one unless beaten by 6 %.  (With 10 % for all sizes the small tile was
-// picked on large problems where 256x256 measured 20-40 % faster; with no margin on mid-sized fp8
-// problems where the small tile measured 7-15 % faster.  Mean regret over 124 measured problems: 0.9 %.)
+// Tile the single-group kernel should use (256, 128, kRingTile256x128 or kRingTile128Deep): the rules for
+// one row or column of tiles and for two rows first, then the shortest estimate, a larger tile being
+// preferred within 2 % (it moves fewer bytes).
 int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_scaled) {
   // One or two rows of 128 x 128 tiles that nearly fill the CUs in one round, and a short K: every
   // workgroup streams its own rows of B from HBM, which the nine-slot ring keeps further ahead of the
@@ -151,10 +168,12 @@ int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_s
   const double e256 = estimate_us(256, M, N, K, elem_bytes);
   const double e128 = estimate_us(128, M, N, K, elem_bytes);
   const double e2 = estimate_us(kRingTile256x128, M, N, K, elem_bytes);
-  const double best_large = e256 <= 1.05 * e2 ? e256 : e2;
-  const double margin = tiles_of(M, N, 128) <= kSmallProblemTiles ? 1.1 : 1.06;
-  if (e128 <= margin * best_large) return 128;
-  return e256 <= 1.05 * e2 ? 256 : kRingTile256x128;
+  // Under 16 k-steps, fewer than any fitted problem had, the estimates of the small tiles run low (e4m3,
+  // 14 k-steps, 1264 x 3240 and 11664 x 328: 128 x 128 tiles estimated 2 % ahead of 256 x 128, measured 8 and 15 %
+  // behind): a larger tile is preferred within 10 % there.
+  const double margin = k_steps_of(K, elem_bytes) < 16 ? 1.10 : 1.02;
+  const double best = margin * (e256 < e128 ? (e256 < e2 ? e256 : e2) : (e128 < e2 ? e128 : e2));
+  return e256 <= best ? 256 : e2 <= best ? kRingTile256x128 : 128;
 }
 
 // K splits for the single-group kernel on the tile ring_tile_edge picks.

@@ -300,7 +300,7 @@ def test_basic_kernel_with_128_tiles_and_k_splits(abi, dt, M, N, K):
     (torch.float8_e4m3fn, 4096, 6144, 8192),
     (torch.float16, 4000, 6100, 4200),         # ragged M, N and last k-step: 384 tiles of 256, 66 k-steps cut in two
     (torch.bfloat16, 5746, 5832, 5648),        # 529 tiles: 17 cut in five, 89 k-steps (the last ragged): items of 17 and 18
-    (torch.bfloat16, 4096, 4352, 3008),        # 272 tiles: 16 cut in two, 47 k-steps: 23 + 24
+    (torch.bfloat16, 4352, 4608, 3008),        # 306 tiles: 50 cut in two, 47 k-steps: 23 + 24
     (torch.float8_e4m3fn, 4352, 4352, 6784),   # 33 tiles cut in three, 53 k-steps: 17 + 18 + 18
 ])
 def test_tail_split(abi, dt, M, N, K):
@@ -338,7 +338,7 @@ def test_tail_split(abi, dt, M, N, K):
 @pytest.mark.parametrize("dt,M,N,K,tile,splits", [
     (torch.bfloat16, 512, 6144, 5696, (256, 256), 5),        # 48 tiles, 89 k-steps: 17 + 18 + 18 + 18 + 18
     (torch.bfloat16, 500, 6100, 5648, (256, 256), 5),        # the same with ragged rows, columns and last k-step
-    (torch.float8_e4m3fn, 256, 4096, 13568, (128, 128), 4),  # 64 small tiles, 106 k-steps cut in four
+    (torch.float8_e4m3fn, 256, 4096, 8320, (128, 128), 4),   # 64 small tiles, 65 k-steps cut in four
     (torch.float16, 200, 2048, 4160, (128, 128), 4),         # 32 small tiles, 65 k-steps: 16 + 16 + 16 + 17
 ])
 def test_k_split_that_does_not_divide_the_k_steps(abi, dt, M, N, K, tile, splits):
