@@ -51,10 +51,12 @@ int launch_tile256_pingpong(const GemmArgs& g, int in_dtype, int out_dtype, hipS
 constexpr int kRingTile256x128 = 384;
 // 128 x 128 tile on the nine-slot ring (four k-steps of copies in flight, one workgroup per CU).
 constexpr int kRingTile128Deep = 129;
+// The same ring without the staggered start of the k-steps: for tiles that share rows of A and B through the L2.
+constexpr int kRingTile128DeepPlain = 130;
 // One row of 128 x 128 tiles that the tile kernel runs on the nine-slot ring, also where the streaming kernel could
 // take the problem (pure host function).
 bool ring_one_row_deep(int64_t M, int64_t N, int64_t K, int elem_bytes);
-inline int ring_tile_rows(int tile) { return tile == 128 || tile == kRingTile128Deep ? 128 : 256; }
+inline int ring_tile_rows(int tile) { return tile == 128 || tile == kRingTile128Deep || tile == kRingTile128DeepPlain ? 128 : 256; }
 inline int ring_tile_cols(int tile) { return tile == 256 ? 256 : 128; }
 // block_scaled: for the kernel with block scales, which exists on the five-slot ring only.
 int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_scaled = false);

@@ -90,7 +90,8 @@ constexpr uint32_t kMxUnitBytes = 512;
 // come from HBM, not from the L2: with d = 2 an operand-step has about one k-step of flight time
 // before the barrier that waits for it (a third of a microsecond on the small tile), with d = 4
 // about three.
-template <class T, class OutT, bool kRaggedK, int kTileT, int kWavesN = 2, int kTileNT = kTileT, int kAhead = 2>
+template <class T, class OutT, bool kRaggedK, int kTileT, int kWavesN = 2, int kTileNT = kTileT, int kAhead = 2,
+          bool kRotateT = (kAhead > 2)>
 __global__ __launch_bounds__(threads_of(kWavesN), (kTileT == 256 || kAhead > 2) ? 1 : 2) void gemm_tn_tile_ring(GemmArgs g) {
   constexpr int kSlots = 2 * kAhead + 1;          // shadows the five of ring_common.h
   constexpr int kTile = kTileT;                   // rows of A per workgroup
@@ -251,12 +252,15 @@ __global__ __launch_bounds__(threads_of(kWavesN), (kTileT == 256 || kAhead > 2) 
     copy_rows(rsrc, jc, slotc, soff, voff_b, tail_b, b_step, dma_wave_b);
   };
   // Byte offset of k-step kt of the item that starts at global k-step step0, clamped to its last.
-  // kRotate (the deep ring, i.e. problems of one or two tile rows whose workgroups all read
+  // kRotate (the deep ring on problems of one or two tile rows, whose workgroups all read
   // different rows of B): an item walks its k-steps from its own starting point `rot` and wraps
   // around, so that the workgroups running side by side do not all read the same 128-byte column
   // of rows that lie a power of two apart, i.e. the same few memory channels, at the same time.
   // Only the order of the fp32 additions of a tile depends on it, and that order is fixed per item.
-  constexpr bool kRotate = kAhead > 2;
+  // Where tiles share rows of A and of B through an XCD's L2 (several tile rows and columns) the
+  // deep ring runs without it: items at different k-steps would not find each other's panels there
+  // (bf16 1184 x 2640 x 7168 on 210 tiles: 79.5 us with, 60.3 us without).
+  constexpr bool kRotate = kRotateT;
   uint32_t rot = 0;
   auto soff_of = [&](uint32_t step0, uint32_t kt) __attribute__((always_inline)) -> uint32_t {
     uint32_t at = kt < steps ? kt : steps - 1;
@@ -592,7 +596,7 @@ __global__ __launch_bounds__(256) void tail_reduce(GemmArgs g) {
   *(u32x2*)((uint16_t*)g.C + m * g.ldc + n) = Pack4<OutT>::run(sum[0] * scale, sum[1] * scale, sum[2] * scale, sum[3] * scale);
 }
 
-template <class T, class OutT, int kTileT, int kTileNT = kTileT, int kAhead = 2, int kWavesN = 2>
+template <class T, class OutT, int kTileT, int kTileNT = kTileT, int kAhead = 2, int kWavesN = 2, bool kRotateT = (kAhead > 2)>
 int launch_tile(const GemmArgs& g, hipStream_t stream) {
   const int64_t items = g.tail_tiles ? g.tiles_m * g.tiles_n + (int64_t)g.tail_tiles * (g.tail_splits - 1)
                                      : g.tiles_m * g.tiles_n * g.splits;
@@ -600,10 +604,10 @@ int launch_tile(const GemmArgs& g, hipStream_t stream) {
   const int64_t slots = (int64_t)compute_units() * ((kTileT == 256 || kAhead > 2) ? 1 : 2);  // resident workgroups (LDS-bound)
   const int64_t blocks = items < slots ? items : slots;
   if ((g.K * T::kBytes) % kRowBytes == 0) {
-    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, false, kTileT, kWavesN, kTileNT, kAhead>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
+    hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, false, kTileT, kWavesN, kTileNT, kAhead, kRotateT>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
   } else {
     if constexpr (std::is_same<T, MxE4M3>::value) return -1;  // block scales need whole k-steps (host check)
-    else hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, true, kTileT, kWavesN, kTileNT, kAhead>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
+    else hipLaunchKernelGGL((gemm_tn_tile_ring<T, OutT, true, kTileT, kWavesN, kTileNT, kAhead, kRotateT>), dim3((unsigned)blocks), dim3(threads_of(kWavesN)), 0, stream, g);
   }
   if (hipGetLastError() != hipSuccess) return -1;
   if (g.splits > 1)
@@ -619,9 +623,11 @@ int launch_tile(const GemmArgs& g, hipStream_t stream) {
 template <class T, class OutT>
 int launch(const GemmArgs& g, int tile, hipStream_t stream) {
   if (tile == kRingTile256x128) return launch_tile<T, OutT, 256, 128>(g, stream);
-  if (tile == kRingTile128Deep) {   // the planner does not pick it with block scales (their registers are timed for five slots)
-    if constexpr (!std::is_same<T, MxE4M3>::value) return launch_tile<T, OutT, 128, 128, 4>(g, stream);
-    else return -1;
+  if (tile == kRingTile128Deep || tile == kRingTile128DeepPlain) {
+    // the planner does not pick these with block scales (their registers are timed for five slots)
+    if constexpr (std::is_same<T, MxE4M3>::value) return -1;
+    else if (tile == kRingTile128Deep) return launch_tile<T, OutT, 128, 128, 4>(g, stream);
+    else return launch_tile<T, OutT, 128, 128, 4, 2, false>(g, stream);
   }
   return tile == 128 ? launch_tile<T, OutT, 128>(g, stream) : launch_tile<T, OutT, 256>(g, stream);
 }

@@ -166,14 +166,21 @@ int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_s
       k_steps_of(K, elem_bytes) <= 64)
     return kRingTile128Deep;
   const double e256 = estimate_us(256, M, N, K, elem_bytes);
-  const double e128 = estimate_us(128, M, N, K, elem_bytes);
+  double e128 = estimate_us(128, M, N, K, elem_bytes);
+  // 128 x 128 tiles that make a single round (at most one per CU) have nobody to hide their waits: there the
+  // nine-slot ring, without the staggered start, takes about an eighth less time than the five-slot one (bf16, eleven
+  // problems of 2 x 33...22 x 8 tile rows and columns and 29...245 k-steps, weights from memory: 4-27 % less, mean 14 %;
+  // with more tiles than CUs, where a CU holds two five-slot workgroups, it takes 3-8 % more).
+  const int64_t tiles128 = tiles_of(M, N, 128);
+  const bool single_round = !block_scaled && tiles128 * uniform_splits(tiles128, k_steps_of(K, elem_bytes)) <= kCuSlots;
+  if (single_round) e128 *= 0.87;
   const double e2 = estimate_us(kRingTile256x128, M, N, K, elem_bytes);
   // Under 16 k-steps, fewer than any fitted problem had, the estimates of the small tiles run low (e4m3,
   // 14 k-steps, 1264 x 3240 and 11664 x 328: 128 x 128 tiles estimated 2 % ahead of 256 x 128, measured 8 and 15 %
   // behind): a larger tile is preferred within 10 % there.
   const double margin = k_steps_of(K, elem_bytes) < 16 ? 1.10 : 1.02;
   const double best = margin * (e256 < e128 ? (e256 < e2 ? e256 : e2) : (e128 < e2 ? e128 : e2));
-  return e256 <= best ? 256 : e2 <= best ? kRingTile256x128 : 128;
+  return e256 <= best ? 256 : e2 <= best ? kRingTile256x128 : single_round ? kRingTile128DeepPlain : 128;
 }
 
 // K splits for the single-group kernel on the tile ring_tile_edge picks.

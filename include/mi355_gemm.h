@@ -171,9 +171,10 @@ int mi355_quantize_e4m3(const void *x, int x_dtype, int64_t n, void *x_q,
  * Constraints: K % 128 == 0; A, B 16-byte aligned with row strides that are multiples of 16;
  * N % 4 == 0, ldc % 4 == 0, C 8-byte aligned; the size limits of the tiled variants.  Runs the
  * weight-streaming kernel (MI355_VARIANT_SKINNY) for M <= 64 and otherwise the tiled kernel
- * (MI355_VARIANT_BASIC) with the tile and splits mi355_gemm_plan reports for MI355_E4M3 operands
- * of this shape and that variant (except with 65...128 rows, where plain operands may get a ring
- * that the block-scaled kernel does not have and this call keeps the planner's other choice).
+ * (MI355_VARIANT_BASIC) with the planner's choice of tile and splits among the tiles this kernel
+ * has: what mi355_gemm_plan reports for MI355_E4M3 operands of this shape and that variant,
+ * except where plain operands get the nine-slot ring of 128 x 128 tiles (one row or column of
+ * tiles, or tiles that make a single round), which the block-scaled kernel does not have.
  * Counterpart in the reference: none (it has no fp8 path); same launcher contract as
  * mi355_gemm_tn (kernels/gemm_kernels/sm90a/gemm_test.cu:12-92), block format per the OCP
  * Microscaling Formats (MX) specification v1.0.

@@ -293,6 +293,27 @@ def test_basic_kernel_with_128_tiles_and_k_splits(abi, dt, M, N, K):
     assert torch.equal(C.view(torch.int16), C2.view(torch.int16))   # fixed summation order
 
 
+@pytest.mark.parametrize("dt,M,N,K", [(torch.bfloat16, 3491, 1364, 288), (torch.float16, 2062, 3316, 488), (torch.float8_e4m3fn, 2589, 3220, 976),
+                                      (torch.bfloat16, 1024, 3072, 4096), (torch.float16, 1030, 3076, 4104), (torch.float8_e4m3fn, 296, 8768, 5136)])
+def test_small_tiles_two_per_cu_and_single_round(abi, dt, M, N, K):
+    """128x128 tiles: more of them than CUs (the five-slot ring, two workgroups per CU) and a single round (the nine-slot
+    ring without the staggered start), ragged edges and last k-steps; element by element against the generic kernel."""
+    plan = ac.plan(abi, M, N, K, ac.torch_code(dt), ac.BASIC)
+    assert plan[1:3] == (128, 128), plan
+    A = rand((M, K), M, torch.float32).clamp_(-50, 50).to(dt)
+    B = rand((N, K), N, torch.float32).clamp_(-50, 50).to(dt)
+    scale = 2.0 ** -4
+    C = run_abi(abi, A, B, ac.BASIC, scale)
+    check(C, A, B, scale)
+    S = torch.empty((M, N), dtype=out_dtype_of(dt), device="cuda")
+    assert ac.gemm_tn(abi, A.cuda(), B.cuda(), S, scale, ac.SIMPLE) == 0
+    torch.cuda.synchronize()
+    d = (C.float() - S.cpu().float()).abs()
+    bad = d > 2e-2 * S.cpu().float().abs() + 2e-2 * (K ** 0.5) * scale
+    assert int(bad.sum()) == 0, (int(bad.sum()), float(d.max()))
+    assert torch.equal(run_abi(abi, A, B, ac.AUTO, scale).view(torch.int16), C.view(torch.int16))
+
+
 @pytest.mark.parametrize("dt,M,N,K", [
     (torch.bfloat16, 4096, 6144, 4096),        # 384 tiles of 256: one full round + 128 tiles cut in two
     (torch.bfloat16, 6144, 6144, 6144),        # two full rounds + 64 tiles cut in four
@@ -369,8 +390,8 @@ def test_k_split_that_does_not_divide_the_k_steps(abi, dt, M, N, K, tile, splits
     (torch.float16, 256, 4096, 14336),         # 32 tiles, K split 8 ways
     (torch.float8_e4m3fn, 1024, 6144, 4096),
     (torch.float8_e4m3fn, 1000, 6100, 4112),   # ragged; 4112 fp8 bytes = 32 k-steps + 16 bytes
-    (torch.float8_e4m3fn, 256, 4096, 14336),   # K split 7 ways
-    (torch.bfloat16, 500, 2000, 8200),         # 2 x 16 tiles, 129 k-steps (the last ragged) cut in eight
+    (torch.float8_e4m3fn, 256, 6144, 14336),   # 48 tiles, 112 k-steps cut in five: 22 + 22 + 23 + 22 + 23
+    (torch.bfloat16, 500, 3000, 16400),        # 2 x 24 tiles, 257 k-steps (the last ragged) cut in five
 ])
 def test_rectangular_tile(abi, dt, M, N, K):
     """Problems the planner gives the 256x128 tile: against the oracle and, element by element,
