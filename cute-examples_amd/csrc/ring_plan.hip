@@ -171,8 +171,15 @@ int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_s
   // nine-slot ring, without the staggered start, takes about an eighth less time than the five-slot one (bf16, eleven
   // problems of 2 x 33...22 x 8 tile rows and columns and 29...245 k-steps, weights from memory: 4-27 % less, mean 14 %;
   // with more tiles than CUs, where a CU holds two five-slot workgroups, it takes 3-8 % more).
-  const int64_t tiles128 = tiles_of(M, N, 128);
-  const bool single_round = !block_scaled && tiles128 * uniform_splits(tiles128, k_steps_of(K, elem_bytes)) <= kCuSlots;
+  // Items of fewer than 16 k-steps stay on five slots: the longer prologue of the deeper ring shows (fp16 512^3, 16 tiles
+  // of 8 k-steps: 6.5 us on five slots, 7.2 on nine).
+  const int64_t tiles128 = tiles_of(M, N, 128), steps128 = k_steps_of(K, elem_bytes);
+  const int splits128 = uniform_splits(tiles128, steps128);
+  // Nor is there anything to wait for when both operands sit in the L2 from the previous call (back-to-back launches of
+  // bf16 1024^3, 768^2 x 2048, 2048^2 x 1024, 4-8 MB of operands: five slots 5-8 % faster; with the operands coming from
+  // memory the nine slots win at those sizes too, by 1-12 %): from 8 MB of operands on.
+  const bool single_round = !block_scaled && tiles128 * splits128 <= kCuSlots && steps128 / splits128 >= 16 &&
+                            (M + N) * K * elem_bytes >= (int64_t)8 << 20;
   if (single_round) e128 *= 0.87;
   const double e2 = estimate_us(kRingTile256x128, M, N, K, elem_bytes);
   // Under 16 k-steps, fewer than any fitted problem had, the estimates of the small tiles run low (e4m3,
