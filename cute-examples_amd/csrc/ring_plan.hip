@@ -87,7 +87,8 @@ struct SmallTileCost {
 };
 constexpr SmallTileCost kCost128 = {0.990, 0.498, 0.244, 0.352, 0.519, 5.53, 0.101, 1.71};
 
-double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
+// k_loop_factor scales the k-step part of the small tile's estimate (not the fixed and reduction parts): see ring_tile_edge.
+double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes, double k_loop_factor = 1.0) {
   const int64_t rows = ring_tile_rows(tile), cols = ring_tile_cols(tile);
   const int64_t tm = (M + rows - 1) / rows, tn = (N + cols - 1) / cols, tiles = tm * tn;
   const int64_t steps = k_steps_of(K, elem_bytes);
@@ -105,7 +106,7 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes) {
     const double step_sum = c.pair * pair_rounds - c.pair_slack * slack +
                             (single ? c.single + c.single_busy * (double)rest / (double)kCuSlots : 0.0) +
                             c.few_rows * rounds / (double)tm;
-    return item_steps * step_sum + c.fixed * rounds + (partial_mb > 0.0 ? c.reduce_mb * partial_mb + c.reduce : 0.0);
+    return k_loop_factor * item_steps * step_sum + c.fixed * rounds + (partial_mb > 0.0 ? c.reduce_mb * partial_mb + c.reduce : 0.0);
   }
   const TileCost& c = tile == 256 ? kCost256 : kCost256x128;
   double rounds = (double)((items + kCuSlots - 1) / kCuSlots);
@@ -166,21 +167,22 @@ int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_s
       k_steps_of(K, elem_bytes) <= 64)
     return kRingTile128Deep;
   const double e256 = estimate_us(256, M, N, K, elem_bytes);
-  double e128 = estimate_us(128, M, N, K, elem_bytes);
   // 128 x 128 tiles that make a single round (at most one per CU) have nobody to hide their waits: there the
-  // nine-slot ring, without the staggered start, takes about an eighth less time than the five-slot one (bf16, eleven
+  // nine-slot ring, without the staggered start, takes a sixth less time per k-step than the five-slot one (bf16, eleven
   // problems of 2 x 33...22 x 8 tile rows and columns and 29...245 k-steps, weights from memory: 4-27 % less, mean 14 %;
   // with more tiles than CUs, where a CU holds two five-slot workgroups, it takes 3-8 % more).
   // Items of fewer than 16 k-steps stay on five slots: the longer prologue of the deeper ring shows (fp16 512^3, 16 tiles
   // of 8 k-steps: 6.5 us on five slots, 7.2 on nine).
   const int64_t tiles128 = tiles_of(M, N, 128), steps128 = k_steps_of(K, elem_bytes);
   const int splits128 = uniform_splits(tiles128, steps128);
-  // Nor is there anything to wait for when both operands sit in the L2 from the previous call (back-to-back launches of
-  // bf16 1024^3, 768^2 x 2048, 2048^2 x 1024, 4-8 MB of operands: five slots 5-8 % faster; with the operands coming from
-  // memory the nine slots win at those sizes too, by 1-12 %): from 8 MB of operands on.
-  const bool single_round = !block_scaled && tiles128 * splits128 <= kCuSlots && steps128 / splits128 >= 16 &&
-                            (M + N) * K * elem_bytes >= (int64_t)8 << 20;
-  if (single_round) e128 *= 0.87;
+  // (When both operands still sit in the L2 from the previous call -- back-to-back launches of bf16 1024^3,
+  // 768^2 x 2048, 2048^2 x 1024, 4-8 MB of operands -- there is nothing to wait for and five slots are 5-8 % faster;
+  // with the rows of B coming from memory, as weights do, nine slots win at those sizes too, by 6-16 %.)
+  const bool single_round = !block_scaled && tiles128 * splits128 <= kCuSlots && steps128 / splits128 >= 16;
+  // The factor on the k-step part of the estimate: 0.82 (on 60 further problems timed on all four forms 0.78...0.80 leave a
+  // regret of 0.2 %, 0.82 one of 0.4 %, 0.86 0.8 %, 0.76 0.55 %, no candidate 1.5 %; 0.82 keeps bf16 256 x 6144 x 4096 on
+  // 256 x 128 tiles, 28.1 us against 29.5).
+  const double e128 = estimate_us(128, M, N, K, elem_bytes, single_round ? 0.82 : 1.0);
   const double e2 = estimate_us(kRingTile256x128, M, N, K, elem_bytes);
   // Under 16 k-steps, fewer than any fitted problem had, the estimates of the small tiles run low (e4m3,
   // 14 k-steps, 1264 x 3240 and 11664 x 328: 128 x 128 tiles estimated 2 % ahead of 256 x 128, measured 8 and 15 %

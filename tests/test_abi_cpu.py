@@ -176,7 +176,8 @@ def test_plan(abi):
     assert ac.plan(abi, 4096, 6144, 4096, ac.BF16) == (ac.BASIC, 256, 256, 1, 128, 2)       # tail split
     assert ac.plan(abi, 512, 14336, 4096, ac.BF16) == (ac.BASIC, 256, 128, 1, 0, 1)         # 224 rectangular tiles
     assert ac.plan(abi, 2048, 2048, 2048, ac.F16) == (ac.BASIC, 128, 128, 1, 0, 1)          # 256 small tiles
-    assert ac.plan(abi, 512, 6144, 4096, ac.BF16) == (ac.BASIC, 256, 128, 2, 0, 1)          # 96 tiles cut in two
+    assert ac.plan(abi, 512, 6144, 4096, ac.BF16) == (ac.BASIC, 128, 128, 1, 0, 1)          # 192 small tiles in one round
+    assert ac.plan(abi, 256, 6144, 4096, ac.BF16) == (ac.BASIC, 256, 128, 4, 0, 1)          # 48 tiles cut in four
     v, rows, cols, splits, _, _ = ac.plan(abi, 16, 6144, 4096, ac.BF16)
     assert (v, rows, cols) == (ac.SKINNY, 16, 64) and splits >= 2
     # 224 tiles of 64 columns: (nearly) one per CU, so no K split (the kernel then runs a deeper ring)
