@@ -116,7 +116,18 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
   // The tiles' starting points are spread evenly over the k-steps (neighbouring tiles one n-th of the
   // way apart: of four spacings tried this was the best, 16x14336x4096 bf16 25.1 -> 21.9 us against
   // a stride of seven k-steps).
-  const uint32_t rot = __builtin_amdgcn_readfirstlane((blockIdx.x * steps / gridDim.x + blockIdx.y * 3u) % steps);
+  // Tiles of 64 rows of X differ: a third to a half of what such a workgroup reads is its slice of X, which
+  // all tiles of its K split read too.  Spread evenly, the four or eight of them that share an XCD's L2 pass
+  // a given k-step so far apart in time that the rows of W streaming through have evicted it in between
+  // (bf16 64x4096x14336: 164 MiB fetched by the L2s for 113 MiB of operands).  So there the XCDs start an
+  // eighth of the k-steps apart and an XCD's tiles two k-steps apart: 31.5 -> 27.4 us on that problem,
+  // 64x8192x28672 103 -> 91 us, 56x5120x13824 34.6 -> 31.9 us.  With many tiles per XCD (evenly spread
+  // neighbours under three k-steps apart) and on the shorter tiles, where X is a small share, the even
+  // spread stays: clustered, bf16 16x14336x4096 took 23.7 us against 21.4 and 64x14336x4096 28.0 against 26.3.
+  uint32_t first = blockIdx.x * steps / gridDim.x;
+  if (kTm == 64 && 8u * steps >= 3u * gridDim.x)
+    first = ((blockIdx.x + gridDim.x * blockIdx.y) & 7u) * steps / 8u + (blockIdx.x >> 3) * 2u;
+  const uint32_t rot = __builtin_amdgcn_readfirstlane((first + blockIdx.y * 3u) % steps);
   auto issue_step = [&](uint32_t stage, uint32_t kt) __attribute__((always_inline)) {
     uint32_t at = (kt < steps ? kt : steps - 1) + rot;   // steps past the end repeat the last one
     at = at >= steps ? at - steps : at;
