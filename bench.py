@@ -44,7 +44,7 @@ PEAK_HBM_GBS = 8000.0
 # (FETCH_SIZE, then WRITE_SIZE, each with --copy-calibration and scaled by what the same counter
 # reads for the 1 GiB copy: x2.000 and x1.000).  Workloads without a counter run report null.
 MEASURED_TRAFFIC_BYTES = {"bf16_8192": 1.746e9, "fp8_8192": 0.944e9, "mxfp8_8192": 0.965e9, "bf16_4096": 2.352e8,
-                          "skinny_16_14336_4096": 1.190e8, "skinny_64_14336_4096": 1.236e8, "skinny_64_4096_14336": 1.897e8,
+                          "skinny_16_14336_4096": 1.190e8, "skinny_64_14336_4096": 1.236e8, "skinny_64_4096_14336": 1.527e8,
                           "skinny_256_14336_4096": 1.561e8, "skinny_256_6144_4096": 1.209e8, "skinny_128_8192_4096": 1.130e8}
 TRAFFIC_PROFILE = {"bf16_8192": "profiles/gemm_tn_tile_ring__bf16_8192.md", "fp8_8192": "profiles/gemm_tn_tile_ring__fp8_8192.md",
                    "mxfp8_8192": "profiles/gemm_tn_tile_ring__mxfp8_8192.md", "bf16_4096": "profiles/gemm_tn_tile_ring__bf16_4096.md",
