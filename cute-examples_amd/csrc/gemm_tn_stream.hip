@@ -356,24 +356,28 @@ int splits_narrow(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
 
 // 64 x 128 tiles, made for 33...64 rows: a quarter fewer cache lines requested per output than 64 x 64 (192
 // per 64 x 128 outputs and k-step against 2 x 128), paid for with half as many tiles to spread over the
-// CUs.  Measured against the 64 x 64 tiles on 112 bf16 problems (M = 48 and 64, N = 2048...32768,
-// K = 2048...14336, weights from HBM), each with its own best split: 3-16 % faster where 160-256 wide
-// tiles make one unsplit round (N = 20480...32768), 2-11 % at N = 8192...11008 from 64 k-steps on and
-// 4-13 % at N = 4096...6144 from 128 k-steps on; 3-20 % slower with fewer k-steps than that or fewer
-// columns (the split needed to occupy the CUs leaves each workgroup too few k-steps), within +-3 % at
-// N = 12288...16384, where the 64 x 64 tiles run unsplit on the deep ring.
+// CUs.  Measured against the 64 x 64 tiles (M = 40...64, bf16, weights from HBM, each form with its own best
+// split, the k-steps started as the kernel's `rot` says): 3-30 % faster with 129-256 wide tiles (the narrow
+// ones no longer fit one round; N = 16896...32768, 16...448 k-steps), 2-17 % with 40-95 from 64 k-steps on
+// and 2-28 % with 24-39 from 128 k-steps on; with fewer k-steps or fewer columns than that 1-17 % slower (the
+// split that occupies the CUs leaves a workgroup too few k-steps); with 96-128 wide tiles, where the narrow
+// ones make one unsplit round on the deep ring and the wide ones need a split, from 8 % faster to 21 %
+// slower (K = 16384 at N = 13824 and 16384), so not there.  60 random problems inside the rule against the
+// narrower one before it (160-256 tiles, 64-95 from 64 k-steps, 32-63 from 128): geometric mean -9 %,
+// none more than 1 % slower; e4m3 on six -4...-13 %.
 constexpr int kTileNWide = 128, kDepthWide = 3;
 bool wide_tiles(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
   if (mx || M > 64) return false;
   const int64_t tiles = (N + kTileNWide - 1) / kTileNWide;
   const int64_t steps = (K * elem_bytes + kRowBytes - 1) / kRowBytes;
   // Up to 32 rows the same tile (its lower half idle) wins only just above what the 64-column tiles
-  // cover in one round: N = 20480 and 24576 at M = 16...32 and K = 2048...8192 2-14 % faster, N = 28672
+  // cover in one round: N = 17408...24576 at M = 16...32 and K = 2048...8192 2-18 % faster, N = 28672
   // the same, N = 32768 and N = 16384 0-4 % and 7-20 % slower.
-  if (M <= 32) return tiles >= 160 && tiles < 208;
-  if (tiles >= 160) return tiles <= 256;
-  if (tiles >= 64) return tiles < 96 && steps >= 64;
-  return tiles >= 32 && steps >= 128;
+  if (M <= 32) return tiles > 128 && tiles < 208;
+  if (tiles > 128) return tiles <= 256;
+  if (tiles >= 96) return false;
+  if (tiles >= 40) return steps >= 64;
+  return tiles >= 24 && steps >= 128;
 }
 
 template <class T, class OutT>

@@ -190,6 +190,12 @@ def test_plan(abi):
     assert ac.plan(abi, 64, 8192, 2048, ac.BF16)[1:3] == (64, 64)     # 32 k-steps: too few
     assert ac.plan(abi, 64, 8192, 4096, ac.E4M3)[1:3] == (64, 64)     # the same in fp8
     assert ac.plan(abi, 64, 8192, 8192, ac.E4M3)[1:3] == (64, 128)
+    assert ac.plan(abi, 64, 18432, 2048, ac.BF16)[1:3] == (64, 128)   # 288 narrow tiles would not fit one round
+    assert ac.plan(abi, 64, 6144, 4096, ac.BF16)[1:3] == (64, 128)    # 48 wide tiles of 64 k-steps
+    assert ac.plan(abi, 64, 3072, 8192, ac.BF16)[1:3] == (64, 128)    # 24 of 128 k-steps
+    assert ac.plan(abi, 64, 3072, 4096, ac.BF16)[1:3] == (64, 64)
+    assert ac.plan(abi, 64, 14336, 4096, ac.BF16)[1:3] == (64, 64)    # 224 narrow tiles: one unsplit round
+    assert ac.plan(abi, 16, 17408, 4096, ac.BF16)[1:3] == (64, 128)
     assert ac.plan(abi, 32, 28672, 4096, ac.BF16)[1:3] == (32, 64)
     assert ac.plan(abi, 16, 24576, 4096, ac.BF16) == (ac.SKINNY, 64, 128, 1, 0, 1)   # the wide tile has 64 rows only
     # 65...128 rows against 4096...32768 columns: the tile kernel, one row of 128x128 tiles, K split
