@@ -123,9 +123,13 @@ __global__ __launch_bounds__(kThreads) void gemm_tn_stream(GemmArgs g, float* pa
   // eighth of the k-steps apart and an XCD's tiles two k-steps apart: 31.5 -> 27.4 us on that problem,
   // 64x8192x28672 103 -> 91 us, 56x5120x13824 34.6 -> 31.9 us.  With many tiles per XCD (evenly spread
   // neighbours under three k-steps apart) and on the shorter tiles, where X is a small share, the even
-  // spread stays: clustered, bf16 16x14336x4096 took 23.7 us against 21.4 and 64x14336x4096 28.0 against 26.3.
+  // spread stays: clustered, bf16 16x14336x4096 took 23.7 us against 21.4 and 64x14336x4096 28.0 against 26.3,
+  // and 23x24388x8264 on the 64 x 128 tile (its lower rows out of range) 100.0 against 95.3.  Beyond 96 tile
+  // columns it takes eight k-steps between neighbours for the cluster to pay: 64x20480x28672 (22 apart)
+  // 239 -> 220 us, 64x18432x16384 (14) 127 -> 121 us, but 64x24388x8264 (5.4), 64x28672x8192 (4.6) and
+  // 64x16384x7168 (3.5) 2-3 % slower.
   uint32_t first = blockIdx.x * steps / gridDim.x;
-  if (kTm == 64 && 8u * steps >= 3u * gridDim.x)
+  if (kTm == 64 && rows_x > 32 && 8u * steps >= (gridDim.x > 96u ? 8u : 3u) * gridDim.x)
     first = ((blockIdx.x + gridDim.x * blockIdx.y) & 7u) * steps / 8u + (blockIdx.x >> 3) * 2u;
   const uint32_t rot = __builtin_amdgcn_readfirstlane((first + blockIdx.y * 3u) % steps);
   auto issue_step = [&](uint32_t stage, uint32_t kt) __attribute__((always_inline)) {
