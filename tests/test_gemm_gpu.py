@@ -720,10 +720,13 @@ def test_skinny_kernel_every_tile_height_and_split(abi, dt, M, N, K):
 @pytest.mark.parametrize("dt,M,N,K", [(torch.bfloat16, 64, 8192, 4096), (torch.float16, 33, 8200, 4104), (torch.bfloat16, 50, 4100, 8200),
                                       (torch.float16, 64, 20484, 520), (torch.float8_e4m3fn, 48, 8192, 8192),
                                       (torch.float8_e4m3fn, 64, 4100, 16400), (torch.bfloat16, 40, 32768, 256),
-                                      (torch.float16, 9, 20484, 264), (torch.float8_e4m3fn, 32, 24576, 1040)])
+                                      (torch.float16, 9, 20484, 264), (torch.float8_e4m3fn, 32, 24576, 1040),
+                                      (torch.bfloat16, 40, 16640, 8448), (torch.bfloat16, 64, 3072, 8192),
+                                      (torch.float16, 20, 17412, 1032)])
 def test_skinny_kernel_on_128_wide_tiles(abi, dt, M, N, K):
-    """33...64 rows against enough columns and k-steps, fewer rows against 20480...26496 columns: 64 x 128
-    tiles, split and unsplit, ragged M, N and K."""
+    """33...64 rows against enough columns and k-steps, fewer rows against 16512...26496 columns: 64 x 128
+    tiles, split and unsplit, ragged M, N and K; k-steps started evenly spread (few rows, or many tile columns
+    with few k-steps) and clustered by XCD (more than 32 rows: 33 tile columns split along K, 130 unsplit)."""
     plan = ac.plan(abi, M, N, K, ac.torch_code(dt), ac.SKINNY)
     assert plan[:3] == (ac.SKINNY, 64, 128), plan
     A = rand((M, K), M, torch.float32).clamp_(-50, 50).to(dt)
