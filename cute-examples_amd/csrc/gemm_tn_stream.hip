@@ -33,6 +33,7 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kTileN = 64;
+constexpr int kTileNWide = 128, kDepthWide = 3;   // the 64 x 128 tile of wide_tiles and its ring depth
 
 // kMB x kNB 16x16 blocks per wave, kWM x kWN waves (kWM * kWN == 4).
 // Geometry per input type: 16x16 blocks for all of them (fp8 on the 16x16x128 shape).
@@ -342,7 +343,12 @@ int splits_for(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx, int64_t
   for (int s = 1; s <= 32; ++s) {
     if (tiles * s > slots) break;
     if (s > 1 && steps / s < 8) break;
-    const double cost = (double)((tiles * s + 255) / 256) * (double)((steps + s - 1) / s + 4) + 0.5 * s;
+    // On the 128-column tiles, which also serve thousands of columns, the partial planes count too: S x M x N
+    // floats written and read back, priced in k-steps of a CU (3e-6 each; fifteen problems with every S forced:
+    // all at their best S with 2e-6...4.4e-6; without the term 48x18432x2048 was cut in three, 23.1 us
+    // against 21.5 unsplit).
+    const double planes = tn == kTileNWide && s > 1 ? 3e-6 * (double)s * (double)M * (double)N : 0.0;
+    const double cost = (double)((tiles * s + 255) / 256) * (double)((steps + s - 1) / s + 4) + 0.5 * s + planes;
     if (s == 1 || cost < best_cost) {
       best = s;
       best_cost = cost;
@@ -369,7 +375,6 @@ int splits_narrow(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
 // slower (K = 16384 at N = 13824 and 16384), so not there.  60 random problems inside the rule against the
 // narrower one before it (160-256 tiles, 64-95 from 64 k-steps, 32-63 from 128): geometric mean -9 %,
 // none more than 1 % slower; e4m3 on six -4...-13 %.
-constexpr int kTileNWide = 128, kDepthWide = 3;
 bool wide_tiles(int64_t M, int64_t N, int64_t K, int elem_bytes, bool mx) {
   if (mx || M > 64) return false;
   const int64_t tiles = (N + kTileNWide - 1) / kTileNWide;
