@@ -55,6 +55,15 @@ TRAFFIC_PROFILE = {"bf16_8192": "profiles/gemm_tn_tile_ring__bf16_8192.md", "fp8
                    "skinny_256_6144_4096": "profiles/gemm_tn_tile_ring__skinny_256_6144_4096.md",
                    "skinny_128_8192_4096": "profiles/gemm_tn_tile_ring__skinny_128_8192_4096.md"}
 SETTLE_MIN_MS, SETTLE_MAX_MS, SETTLE_BATCH_MS = 150.0, 2000.0, 10.0
+# Counter readings of the committed rocprofv3 profiles of this script (not re-measured in a plain
+# run): the share of SIMD cycles with an MFMA in flight and the shader clock during the kernel
+# (busy CU cycles / CUs / traced duration).
+PROFILED = {
+    "bf16_8192": {"mfma_busy": 0.884, "shader_clock_ghz": 1.74, "lds_bank_conflict_cycles": 0,
+                  "source": "profiles/gemm_tn_tile_ring__bf16_8192.md"},
+    "fp8_8192": {"mfma_busy": 0.872, "shader_clock_ghz": 1.77, "lds_bank_conflict_cycles": 0,
+                 "source": "profiles/gemm_tn_tile_ring__fp8_8192.md"},
+}
 
 
 def parse():
@@ -71,6 +80,7 @@ def parse():
     p.add_argument("--no-fp8", action="store_true", help="skip the fp8 8192^3 block of the metric")
     p.add_argument("--calibrate", action="store_true", help="(default) measure the MFMA-only and plain-read ceilings")
     p.add_argument("--no-calibrate", action="store_true")
+    p.add_argument("--no-vendor", action="store_true", help="skip torch.mm / torch._scaled_mm on the same operands")
     p.add_argument("--no-settle", action="store_true", help="skip the clock-settle phase in front of every measurement")
     p.add_argument("--copy-calibration", action="store_true",
                    help="also run three 1 GiB device-to-device copies (known traffic: 1 GiB read + 1 GiB "
@@ -247,54 +257,92 @@ def roofline_of(row, workload, variant, sets, flops, nbytes):
     return roof
 
 
-def calibrate(A, B, do_settle=True):
+MFMA_SHAPES = {"bf16": ("16x16x32", "32x32x16"), "f16": ("16x16x32", "32x32x16"), "e4m3": ("16x16x128", "32x32x64")}
+
+
+def calibrate(A, B, do_settle=True, read=True):
     """The library's two ceiling kernels through its C ABI: matrix cores only, on the workload's own
-    operands (dtype of A), and a plain read of 1 GiB.  Returns the two roofline entries."""
+    operands (dtype of A) -- on the MFMA shape the kernels use and on the 32-wide shape they do not --
+    and a plain read of 1 GiB.  Returns the two roofline entries (the second None without `read`)."""
     import ctypes
     import torch
     lib = ctypes.CDLL(os.path.join(ROOT, "cute-examples_amd", "gemm_kernels", "libmi355gemm.so"))
     vp, sz, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
     lib.mi355_calibrate_sink_bytes.restype = sz
-    lib.mi355_calibrate_mfma.argtypes = [ci, vp, sz, vp, sz, ci, vp, ctypes.POINTER(ctypes.c_double), vp]
+    lib.mi355_calibrate_mfma_shape.argtypes = [ci, ci, vp, sz, vp, sz, ci, vp, ctypes.POINTER(ctypes.c_double), vp]
     lib.mi355_calibrate_read.argtypes = [vp, sz, vp, vp]
     code = {torch.bfloat16: 0, torch.float16: 1, torch.float8_e4m3fn: 2}[A.dtype]
+    tag = {0: "bf16", 1: "f16", 2: "e4m3"}[code]
     sink = torch.empty(lib.mi355_calibrate_sink_bytes(), dtype=torch.uint8, device=A.device)
     flops = ctypes.c_double()
     iters = 4000   # ~2 ms per launch
     stream = torch.cuda.current_stream().cuda_stream
 
-    def mfma():
-        rc = lib.mi355_calibrate_mfma(code, A.data_ptr(), A.numel() * A.element_size(), B.data_ptr(),
-                                      B.numel() * B.element_size(), iters, sink.data_ptr(), ctypes.byref(flops), stream)
-        assert rc == 0, rc
-    ms, _, n_settle, settle_ms = time_calls(mfma, 40, 5, do_settle)
+    def mfma_on(a, b, wide):
+        def run():
+            rc = lib.mi355_calibrate_mfma_shape(code, wide, a.data_ptr(), a.numel() * a.element_size(), b.data_ptr(),
+                                                b.numel() * b.element_size(), iters, sink.data_ptr(), ctypes.byref(flops), stream)
+            assert rc == 0, rc
+        return run
+    ms, _, n_settle, settle_ms = time_calls(mfma_on(A, B, 0), 40, 5, do_settle)
     mfma_entry = {"value": round(flops.value / ms / 1e9, 1), "unit": "TFLOP/s", "ms_per_launch": round(ms, 4),
-                  "settle_launches": n_settle, "settle_ms": round(settle_ms, 1),
-                  "what": "mi355_calibrate_mfma: 4 waves per CU, the tile kernel's MFMA pattern on fragments of this "
+                  "settle_launches": n_settle, "settle_ms": round(settle_ms, 1), "mfma_shape": MFMA_SHAPES[tag][0],
+                  "what": "mi355_calibrate_mfma_shape: 4 waves per CU, the tile kernel's MFMA pattern on fragments of this "
                           "workload's operands held in registers; no LDS, no copies, no barriers"}
-    # The same loop on all-zero operands: no data toggling, so the board power limit does not bind
+    # The same loop on the 32-wide MFMA shape, which the kernels do not use: what the choice of shape
+    # is worth on this GPU and this data.
+    ms_wide, _, _, _ = time_calls(mfma_on(A, B, 1), 40, 5, do_settle)
+    mfma_entry["by_shape"] = {MFMA_SHAPES[tag][0]: mfma_entry["value"],
+                              MFMA_SHAPES[tag][1]: round(flops.value / ms_wide / 1e9, 1)}
+    # The kernels' shape on all-zero operands: no data toggling, so the board power limit does not bind
     # and the clock stays near nominal.  The gap to the figure above is what the data costs in clock.
     zeros = torch.zeros(1 << 20, dtype=torch.uint8, device=A.device)
-
-    def mfma_zero():
-        rc = lib.mi355_calibrate_mfma(code, zeros.data_ptr(), zeros.numel(), zeros.data_ptr(), zeros.numel(), iters,
-                                      sink.data_ptr(), ctypes.byref(flops), stream)
-        assert rc == 0, rc
-    ms0, _, _, _ = time_calls(mfma_zero, 40, 5, do_settle)
+    ms0, _, _, _ = time_calls(mfma_on(zeros, zeros, 0), 40, 5, do_settle)
     mfma_entry["value_zero_operands"] = round(flops.value / ms0 / 1e9, 1)
-    src = torch.empty(1 << 30, dtype=torch.uint8, device=A.device)
-    src.view(torch.int32).random_()
+    read_entry = None
+    if read:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=A.device)
+        src.view(torch.int32).random_()
 
-    def read():
-        rc = lib.mi355_calibrate_read(src.data_ptr(), src.numel(), sink.data_ptr(), stream)
-        assert rc == 0, rc
-    ms, _, n_settle, settle_ms = time_calls(read, 100, 10, do_settle)
-    read_entry = {"value": round(src.numel() / ms / 1e6, 1), "unit": "GB/s", "ms_per_launch": round(ms, 4),
-                  "settle_launches": n_settle, "settle_ms": round(settle_ms, 1),
-                  "what": "mi355_calibrate_read: 16-byte loads over 1 GiB (four times the Infinity Cache), nothing else"}
-    del src, sink
+        def read_all():
+            rc = lib.mi355_calibrate_read(src.data_ptr(), src.numel(), sink.data_ptr(), stream)
+            assert rc == 0, rc
+        ms, _, n_settle, settle_ms = time_calls(read_all, 100, 10, do_settle)
+        read_entry = {"value": round(src.numel() / ms / 1e6, 1), "unit": "GB/s", "ms_per_launch": round(ms, 4),
+                      "settle_launches": n_settle, "settle_ms": round(settle_ms, 1),
+                      "what": "mi355_calibrate_read: 16-byte loads over 1 GiB (four times the Infinity Cache), nothing else"}
+        del src
+    del sink
     torch.cuda.empty_cache()
     return mfma_entry, read_entry
+
+
+def vendor_same_run(sets, C, fp8, flops, steps, warmup, do_settle):
+    """The vendor library on the same operands, same protocol (settle, W warm-up, K timed launches):
+    torch.mm (hipBLASLt) for the 16-bit types, torch._scaled_mm for e4m3 with per-tensor scales.
+    A yardstick of what this GPU gives a tuned kernel today; None with the reason if torch refuses."""
+    import torch
+    A, B = sets[0][:2]
+    Bt = B.t()
+    try:
+        if fp8:
+            sa = torch.tensor(float(fp8[0]), dtype=torch.float32, device=A.device)
+            sb = torch.tensor(float(fp8[1]), dtype=torch.float32, device=A.device)
+
+            def call():
+                torch._scaled_mm(A, Bt, scale_a=sa, scale_b=sb, out_dtype=torch.bfloat16, out=C)
+            what = "torch._scaled_mm(A_q, B_q.T, scale_a, scale_b, out_dtype=bf16) on the same operands"
+        else:
+            def call():
+                torch.mm(A, Bt, out=C)
+            what = "torch.mm(A, B.T) (hipBLASLt) on the same operands"
+        call()
+        torch.cuda.synchronize()
+        ms, _, n_settle, settle_ms = time_calls(call, steps, warmup, do_settle)
+    except Exception as e:   # noqa: BLE001  (a yardstick, not the product: report and go on)
+        return {"value": None, "unit": "TFLOP/s", "what": "not available: %s: %s" % (type(e).__name__, str(e)[:160])}
+    return {"value": round(flops / ms / 1e9, 2), "unit": "TFLOP/s", "ms_per_launch": round(ms, 5), "steps": steps,
+            "warmup": warmup, "settle_launches": n_settle, "settle_ms": round(settle_ms, 1), "what": what}
 
 
 def cpu_baseline(A, B, total_rows, scale=1.0, budget_s=12.0, native_budget_s=5.0):
@@ -340,6 +388,29 @@ def cpu_baseline(A, B, total_rows, scale=1.0, budget_s=12.0, native_budget_s=5.0
                       % (kind, rows, N, K, done, el, os.cpu_count())}
 
 
+def other_configs(extras, mfma_ceiling, hbm_read):
+    """The other configurations the baseline names (the nine small-M projection shapes, bf16 4096^3,
+    fp16 512^3) in brief: time per launch, achieved rate, fraction of the published peak and of the
+    ceiling measured in this run (MFMA-only loop on the headline's operands / plain read)."""
+    wanted = ["bf16_4096", "fp16_512"] + ["skinny_%d_%d_%d" % (m, n, k) for (n, k) in ((14336, 4096), (4096, 14336), (6144, 4096))
+                                          for m in (16, 64, 256)]
+    out = {}
+    for row in extras:
+        name = row["workload"]
+        if name not in wanted or "variant" in row:
+            continue
+        if name.startswith("skinny"):
+            e = {"ms": row["ms"], "achieved": row["gbs"], "unit": "GB/s", "bound": "hbm",
+                 "frac": round(row["gbs"] / PEAK_HBM_GBS, 4),
+                 "frac_of_measured_ceiling": round(row["gbs"] / hbm_read["value"], 4) if hbm_read else None}
+        else:
+            e = {"ms": row["ms"], "achieved": row["tflops"], "unit": "TFLOP/s", "bound": "mfma",
+                 "frac": round(row["tflops"] / PEAK_TFLOPS[row["dtype"]], 4),
+                 "frac_of_measured_ceiling": round(row["tflops"] / mfma_ceiling["value"], 4) if mfma_ceiling else None}
+        out[name] = e
+    return out
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -370,6 +441,12 @@ def main():
             roof["frac_of_measured_ceiling"] = round(head["tflops"] / roof["measured_mfma_ceiling"]["value"], 4)
         else:
             roof["frac_of_measured_ceiling"] = round(head["gbs"] / roof["measured_hbm_read"]["value"], 4)
+    if roof["bound"] == "mfma" and not a.no_vendor:
+        roof["torch_mm_same_run"] = vendor_same_run(sets, C, fp8, flops, a.steps, a.warmup, do_settle)
+        if roof["torch_mm_same_run"]["value"]:
+            roof["vs_torch_mm_same_run"] = round(head["tflops"] / roof["torch_mm_same_run"]["value"], 4)
+    if a.workload in PROFILED:
+        roof["profiled"] = PROFILED[a.workload]
 
     head_scale = float(fp8[0]) * float(fp8[1]) if fp8 and isinstance(fp8[0], float) else 1.0
     cpu_operands = (sets[0][0][:1024].cpu(), sets[0][1].cpu(), sets[0][0].shape[0], head_scale) if not a.no_cpu else None
@@ -383,8 +460,13 @@ def main():
         sets8, C8, sc8, flops8, nbytes8 = keep
         roof8 = roofline_of(row, "fp8_8192", a.variant, sets8, flops8, nbytes8)
         if not a.no_calibrate:
-            roof8["measured_mfma_ceiling"], _ = calibrate(sets8[0][0], sets8[0][1], do_settle)
+            roof8["measured_mfma_ceiling"], _ = calibrate(sets8[0][0], sets8[0][1], do_settle, read=False)
             roof8["frac_of_measured_ceiling"] = round(row["tflops"] / roof8["measured_mfma_ceiling"]["value"], 4)
+        if not a.no_vendor:
+            roof8["torch_mm_same_run"] = vendor_same_run(sets8, C8, sc8, flops8, a.steps, a.warmup, do_settle)
+            if roof8["torch_mm_same_run"]["value"]:
+                roof8["vs_torch_mm_same_run"] = round(row["tflops"] / roof8["torch_mm_same_run"]["value"], 4)
+        roof8["profiled"] = PROFILED["fp8_8192"]
         fp8_block = {"value": row["tflops"], "unit": "TFLOP/s", "ms_per_step": row["ms"], "steps": a.steps,
                      "warmup": a.warmup, "settle_launches": row["settle_launches"], "settle_ms": row["settle_ms"],
                      "dtype": "e4m3", "pct_of_dense_mfma_peak": row["pct_mfma_peak"],
@@ -429,8 +511,15 @@ def main():
         roof["fp8_8192"] = {"value": fp8_block["value"], "unit": "TFLOP/s", "ms_per_step": fp8_block["ms_per_step"],
                             "peak": r8["peak"], "frac": r8["frac"], "traffic": r8["traffic"],
                             "measured_mfma_ceiling": (r8.get("measured_mfma_ceiling") or {}).get("value"),
+                            "mfma_ceiling_by_shape": (r8.get("measured_mfma_ceiling") or {}).get("by_shape"),
+                            "frac_of_measured_ceiling": r8.get("frac_of_measured_ceiling"),
+                            "torch_mm_same_run": (r8.get("torch_mm_same_run") or {}).get("value"),
+                            "vs_torch_mm_same_run": r8.get("vs_torch_mm_same_run"),
+                            "profiled": r8.get("profiled"),
                             "cpu_baseline_value": (fp8_block["cpu_baseline"] or {}).get("value"),
                             "see": "the top-level \"fp8\" object of this line"}
+    if extras:
+        roof["other_configs"] = other_configs(extras, roof.get("measured_mfma_ceiling"), roof.get("measured_hbm_read"))
     out = {
         "metric": METRIC, "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "settle_launches": head["settle_launches"], "settle_ms": head["settle_ms"],
@@ -438,7 +527,12 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic",
         "config": {"workload": "%s: M=%d N=%d K=%d, A (M,K) and B (N,K) K-contiguous, fp32 accumulate"
                                % (a.workload, head["M"], head["N"], head["K"]),
-                   "variant": roof["kernel"], "parallelism": "single GPU"},
+                   "variant": roof["kernel"], "parallelism": "single GPU",
+                   "protocol": ("no settle phase; " if a.no_settle else
+                                "a clock-settle phase (the same launch for >= %d ms, until three ~%d ms batches agree "
+                                "within 1 %%; settle_launches / settle_ms) precedes the W warm-up launches; "
+                                % (SETTLE_MIN_MS, SETTLE_BATCH_MS)) +
+                               "then W warm-up and K timed launches back to back, HIP events on the launch stream"},
         "pct_of_dense_mfma_peak": head["pct_mfma_peak"],
         "roofline": roof, "cpu_baseline": cpu, "extras": extras, "fp8": fp8_block,
     }

@@ -8,7 +8,10 @@
 //                  caller's A and B) and runs the tile kernel's MFMA pattern on them -- 64
 //                  accumulator blocks, acc[i][j] += a[i] * b[j], the same instruction and the same
 //                  dependency distance as a k-step of gemm_tn_tile_ring -- with no LDS traffic, no
-//                  copies, no barriers.  One workgroup of four waves per CU.
+//                  copies, no barriers.  One workgroup of four waves per CU.  The same loop also
+//                  exists on the 32-wide MFMA shapes the kernels do not use (4 + 4 fragments, 16
+//                  blocks: the same 128 x 128 outputs per wave), so that a benchmark can show what
+//                  the choice of shape is worth on the GPU and the data at hand.
 //   read_ceiling   16-byte loads, grid-stride over the buffer, xor-reduced so nothing is elided.
 //
 // Counterpart in the reference: none (its benchmark takes the peak from a table,
@@ -20,12 +23,32 @@
 namespace mi355 {
 namespace {
 
+// v_mfma_f32_32x32x16 for the 16-bit types: the shape the tile kernels do NOT run on (measured
+// here so that the choice is visible); fp8 on 32x32x64 is Geo<E4M3> of ring_common.h.
+template <class T> struct Geo32;
+template <> struct Geo32<BF16> {
+  static constexpr int kBlk = 32;
+  typedef i32x4 Frag;
+  typedef f32x16 Acc;
+  static __device__ __forceinline__ void mfma_inplace(Frag x, Frag y, Acc& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));
+  }
+};
+template <> struct Geo32<F16> {
+  static constexpr int kBlk = 32;
+  typedef i32x4 Frag;
+  typedef f32x16 Acc;
+  static __device__ __forceinline__ void mfma_inplace(Frag x, Frag y, Acc& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(x), "v"(y));
+  }
+};
+
 template <class G>
 __global__ __launch_bounds__(256, 1) void mfma_ceiling(const uint8_t* a, const uint8_t* b, size_t a_bytes,
                                                        size_t b_bytes, int iters, float* sink) {
   typedef typename G::Frag Frag;
   typedef typename G::Acc Acc;
-  constexpr int kN = 8;
+  constexpr int kN = 128 / G::kBlk;   // blocks per side of the wave's 128 x 128 outputs
   Frag fa[kN], fb[kN];
   Acc acc[kN][kN];
   // Fragment i of this lane: sizeof(Frag) bytes of the operand, a different place for every lane,
@@ -77,11 +100,12 @@ extern "C" {
 
 size_t mi355_calibrate_sink_bytes(void) { return (size_t)4096 * 256 * 4; }
 
-int mi355_calibrate_mfma(int in_dtype, const void* a, size_t a_bytes, const void* b, size_t b_bytes, int iters,
-                         void* sink, double* flops, void* stream) {
+int mi355_calibrate_mfma_shape(int in_dtype, int wide_blocks, const void* a, size_t a_bytes, const void* b, size_t b_bytes,
+                               int iters, void* sink, double* flops, void* stream) {
   using namespace mi355;
   if (!a || !b || !sink || !flops) return MI355_ERR_NULL;
   if (in_dtype != MI355_BF16 && in_dtype != MI355_F16 && in_dtype != MI355_E4M3) return MI355_ERR_DTYPE;
+  if (wide_blocks != 0 && wide_blocks != 1) return MI355_ERR_VARIANT;
   if (iters <= 0 || a_bytes < 4096 || b_bytes < 4096) return MI355_ERR_SHAPE;
   if ((uintptr_t)a % 32 != 0 || (uintptr_t)b % 32 != 0 || (uintptr_t)sink % 4 != 0) return MI355_ERR_ALIGN;
   const int cus = compute_units();
@@ -89,16 +113,27 @@ int mi355_calibrate_mfma(int in_dtype, const void* a, size_t a_bytes, const void
   hipStream_t s = (hipStream_t)stream;
   const uint8_t* pa = (const uint8_t*)a;
   const uint8_t* pb = (const uint8_t*)b;
-  // flop per MFMA: 2 * 16 * 16 * K, K = 32 (16-bit) or 128 (fp8)
-  const double per_mfma = in_dtype == MI355_E4M3 ? 2.0 * 16 * 16 * 128 : 2.0 * 16 * 16 * 32;
-  *flops = per_mfma * 64.0 * (double)iters * 4.0 * (double)cus;
-  if (in_dtype == MI355_BF16)
-    hipLaunchKernelGGL(mfma_ceiling<Geo<BF16>>, dim3(cus), dim3(256), 0, s, pa, pb, a_bytes, b_bytes, iters, (float*)sink);
-  else if (in_dtype == MI355_F16)
-    hipLaunchKernelGGL(mfma_ceiling<Geo<F16>>, dim3(cus), dim3(256), 0, s, pa, pb, a_bytes, b_bytes, iters, (float*)sink);
-  else
-    hipLaunchKernelGGL(mfma_ceiling<GeoE4M3Rows>, dim3(cus), dim3(256), 0, s, pa, pb, a_bytes, b_bytes, iters, (float*)sink);
+  // Every shape covers the wave's 128 x 128 outputs once per pass over its blocks, with a K extent
+  // of 32 or 16 elements (16-bit, 16- or 32-wide blocks) or 128 or 64 elements (fp8).
+  const double k_extent = in_dtype == MI355_E4M3 ? (wide_blocks ? 64.0 : 128.0) : (wide_blocks ? 16.0 : 32.0);
+  *flops = 2.0 * 128.0 * 128.0 * k_extent * (double)iters * 4.0 * (double)cus;
+  const dim3 grid(cus), block(256);
+  float* out = (float*)sink;
+  if (!wide_blocks) {
+    if (in_dtype == MI355_BF16) hipLaunchKernelGGL(mfma_ceiling<Geo<BF16>>, grid, block, 0, s, pa, pb, a_bytes, b_bytes, iters, out);
+    else if (in_dtype == MI355_F16) hipLaunchKernelGGL(mfma_ceiling<Geo<F16>>, grid, block, 0, s, pa, pb, a_bytes, b_bytes, iters, out);
+    else hipLaunchKernelGGL(mfma_ceiling<GeoE4M3Rows>, grid, block, 0, s, pa, pb, a_bytes, b_bytes, iters, out);
+  } else {
+    if (in_dtype == MI355_BF16) hipLaunchKernelGGL(mfma_ceiling<Geo32<BF16>>, grid, block, 0, s, pa, pb, a_bytes, b_bytes, iters, out);
+    else if (in_dtype == MI355_F16) hipLaunchKernelGGL(mfma_ceiling<Geo32<F16>>, grid, block, 0, s, pa, pb, a_bytes, b_bytes, iters, out);
+    else hipLaunchKernelGGL(mfma_ceiling<Geo<E4M3>>, grid, block, 0, s, pa, pb, a_bytes, b_bytes, iters, out);
+  }
   return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ERR_LAUNCH;
+}
+
+int mi355_calibrate_mfma(int in_dtype, const void* a, size_t a_bytes, const void* b, size_t b_bytes, int iters,
+                         void* sink, double* flops, void* stream) {
+  return mi355_calibrate_mfma_shape(in_dtype, 0, a, a_bytes, b, b_bytes, iters, sink, flops, stream);
 }
 
 int mi355_calibrate_read(const void* src, size_t bytes, void* sink, void* stream) {

@@ -264,6 +264,10 @@ int mi355_gemm_tile_coord(int64_t block, int64_t tiles_m, int64_t tiles_n,
  * device data of that type, e.g. the operands of the GEMM being measured: the sustained clock
  * depends on the data; at least 4096 bytes each, 32-byte aligned).  *flops receives the flop count
  * of the launch; the caller times it.  `sink` is device memory of mi355_calibrate_sink_bytes().
+ * mi355_calibrate_mfma_shape is the same with the choice of MFMA shape: wide_blocks == 0 is the
+ * above, wide_blocks == 1 runs the loop on the 32-wide shapes the kernels do not use
+ * (v_mfma_f32_32x32x16 for the 16-bit types, v_mfma_f32_32x32x64_f8f6f4 for MI355_E4M3; 16
+ * accumulator blocks, the same 128 x 128 outputs per wave), so that a benchmark can report both.
  *
  * mi355_calibrate_read enqueues one launch that reads `bytes` bytes at `src` (16-byte aligned)
  * with plain 16-byte loads and nothing else.
@@ -271,6 +275,9 @@ int mi355_gemm_tile_coord(int64_t block, int64_t tiles_m, int64_t tiles_n,
 size_t mi355_calibrate_sink_bytes(void);
 int mi355_calibrate_mfma(int in_dtype, const void *a, size_t a_bytes, const void *b, size_t b_bytes,
                          int iters, void *sink, double *flops, void *stream);
+int mi355_calibrate_mfma_shape(int in_dtype, int wide_blocks, const void *a, size_t a_bytes,
+                               const void *b, size_t b_bytes, int iters, void *sink, double *flops,
+                               void *stream);
 int mi355_calibrate_read(const void *src, size_t bytes, void *sink, void *stream);
 
 /* Human-readable text for a status code; never NULL.  Replaces the TORCH_CHECK messages of

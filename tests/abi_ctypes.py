@@ -62,6 +62,8 @@ def load():
     L.mi355_calibrate_sink_bytes.restype = sz
     L.mi355_calibrate_mfma.argtypes = [ci, vp, sz, vp, sz, ci, vp, ctypes.POINTER(ctypes.c_double), vp]
     L.mi355_calibrate_mfma.restype = ci
+    L.mi355_calibrate_mfma_shape.argtypes = [ci, ci, vp, sz, vp, sz, ci, vp, ctypes.POINTER(ctypes.c_double), vp]
+    L.mi355_calibrate_mfma_shape.restype = ci
     L.mi355_calibrate_read.argtypes = [vp, sz, vp, vp]
     L.mi355_calibrate_read.restype = ci
     L.mi355_gemm_strerror.argtypes = [ci]

@@ -43,20 +43,31 @@ def test_calibration_kernels_run_and_report_plausible_ceilings(abi):
     stream = torch.cuda.current_stream().cuda_stream
     flops = ctypes.c_double()
     assert abi.mi355_calibrate_mfma(ac.BF16, None, 4096, None, 4096, 10, sink.data_ptr(), ctypes.byref(flops), stream) == ac.ERR_NULL
-    for code, dt, peak in ((ac.BF16, torch.bfloat16, 2500.0), (ac.E4M3, torch.float8_e4m3fn, 5000.0)):
+    assert abi.mi355_calibrate_mfma_shape(ac.BF16, 2, sink.data_ptr(), 4096, sink.data_ptr(), 4096, 10, sink.data_ptr(),
+                                          ctypes.byref(flops), stream) == ac.ERR_VARIANT
+    for code, dt, peak in ((ac.BF16, torch.bfloat16, 2500.0), (ac.F16, torch.float16, 2500.0), (ac.E4M3, torch.float8_e4m3fn, 5000.0)):
         A = torch.randn(1024, 1024, device="cuda").to(dt)
         B = torch.randn(1024, 1024, device="cuda").to(dt)
         nbytes = A.numel() * A.element_size()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        for timed in (False, True):
-            e0.record()
-            rc = abi.mi355_calibrate_mfma(code, A.data_ptr(), nbytes, B.data_ptr(), nbytes, 2000, sink.data_ptr(),
-                                          ctypes.byref(flops), stream)
-            e1.record()
-            assert rc == ac.OK
-            torch.cuda.synchronize()
-        tflops = flops.value / e0.elapsed_time(e1) / 1e9
-        assert 100.0 < tflops <= 1.02 * peak, tflops
+        flop_counts = []
+        for wide in (None, 0, 1):      # the plain entry point, then both MFMA shapes by name
+            for timed in (False, True):
+                e0.record()
+                if wide is None:
+                    rc = abi.mi355_calibrate_mfma(code, A.data_ptr(), nbytes, B.data_ptr(), nbytes, 2000, sink.data_ptr(),
+                                                  ctypes.byref(flops), stream)
+                else:
+                    rc = abi.mi355_calibrate_mfma_shape(code, wide, A.data_ptr(), nbytes, B.data_ptr(), nbytes, 2000,
+                                                        sink.data_ptr(), ctypes.byref(flops), stream)
+                e1.record()
+                assert rc == ac.OK
+                torch.cuda.synchronize()
+            tflops = flops.value / e0.elapsed_time(e1) / 1e9
+            assert 100.0 < tflops <= 1.02 * peak, (code, wide, tflops)
+            flop_counts.append(flops.value)
+        # 2000 passes over 128 x 128 outputs per wave: the narrow shapes span twice the K of the wide ones
+        assert flop_counts[0] == flop_counts[1] == 2 * flop_counts[2]
     src = torch.empty(1 << 28, dtype=torch.uint8, device="cuda")
     src.view(torch.int32).random_()
     for timed in (False, True):

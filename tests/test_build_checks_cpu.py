@@ -6,7 +6,8 @@ import sys
 
 import pytest
 
-sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "cute-examples_amd"))
+PKG = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "cute-examples_amd")
+sys.path.insert(0, PKG)
 import check_async_loads  # noqa: E402
 
 HEAD = "_ZN5mi35512_GLOBAL__N_117gemm_tn_tile_ringINS_6MxE4M3ENS_4BF16ELb0ELi256ELi2EEEvNS_8GemmArgsE: ; @kernel\n"
@@ -234,3 +235,37 @@ def test_scratch_use_is_rejected(tmp_path):
     f.write_text(meta % (0, 0) + meta % (1420, 1756))
     with pytest.raises(RuntimeError, match="uses scratch memory"):
         check_async_loads.check_no_scratch(str(f))
+
+
+def test_fallback_build_of_the_block_scaled_kernel_passes_the_hazard_checks(tmp_path):
+    """The block-scaled kernel's fallback build (MI355_MX_SYNC_SCALES: scale loads that wait for
+    themselves, what build.py switches to when a compiler copies a scale register) compiles for
+    gfx950 here, without a GPU, and its generated assembly passes the checks every build applies:
+    store-data and MFMA-result distances, the copies' LDS base, no scratch.  In that object every
+    scale load is followed by a wait for all outstanding vector-memory instructions."""
+    import glob
+    import importlib.util
+    import shutil
+    import subprocess
+    spec = importlib.util.spec_from_file_location("_mi355_build_for_test", os.path.join(PKG, "build.py"))
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    if not (os.path.exists(hipcc) or shutil.which(hipcc)):
+        pytest.skip("hipcc not found")
+    src = build.CHECKED_SOURCE
+    cmd = [hipcc] + build.HIPCC_FLAGS + ["-c", "-save-temps=obj", "-DMI355_MX_SYNC_SCALES", "-o",
+                                         str(tmp_path / "mx_sync.o"), os.path.join(build.CSRC, src)]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert proc.returncode == 0, proc.stdout[-2000:]
+    asm = glob.glob(str(tmp_path / "*-hip-amdgcn-*gfx950.s"))
+    assert len(asm) == 1, asm
+    stores, mfmas = check_async_loads.check_hazard_distances(asm[0])
+    assert stores > 100 and mfmas > 1000
+    assert check_async_loads.check_lds_base(asm[0]) > 100
+    check_async_loads.check_no_scratch(asm[0])
+    text = open(asm[0]).read().split("\n")
+    loads = [i for i, l in enumerate(text) if l.strip().startswith("buffer_load_dwordx2")]
+    assert len(loads) > 100
+    for i in loads:
+        assert text[i + 1].strip().startswith("s_waitcnt vmcnt(0)"), text[i:i + 2]
