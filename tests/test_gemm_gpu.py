@@ -685,6 +685,28 @@ def test_one_tile_row_with_k_splits_on_the_nine_slot_ring(abi, dt, M, N, K):
     assert torch.equal(run_abi(abi, A, B, ac.AUTO, 0.5).view(torch.int16), C.view(torch.int16))
 
 
+@pytest.mark.parametrize("dt,M,N,K,steps", [(torch.bfloat16, 100, 16384, 64, 1), (torch.bfloat16, 100, 16388, 72, 2),
+                                            (torch.float16, 128, 20000, 200, 4), (torch.float8_e4m3fn, 90, 12288, 512, 4),
+                                            (torch.bfloat16, 128, 12288, 320, 5), (torch.float8_e4m3fn, 70, 32768, 1008, 8)])
+def test_one_tile_row_with_fewer_k_steps_than_the_nine_slot_ring_keeps_in_flight(abi, dt, M, N, K, steps):
+    """One row of 128x128 tiles, unsplit, with 1...8 k-steps: fewer than the nine-slot ring's five
+    opening operand-steps (or than its nine slots), so its copies are clamped to the last k-step and
+    the rotated starting points wrap inside a handful of steps; ragged K, M and N among them."""
+    es = 1 if dt == torch.float8_e4m3fn else 2
+    assert -(-K * es // 128) == steps
+    v, rows, cols, splits, _, _ = ac.plan(abi, M, N, K, ac.torch_code(dt))
+    assert (v, rows, cols, splits) == (ac.BASIC, 128, 128, 1), (v, rows, cols, splits)
+    if dt == torch.float8_e4m3fn:
+        A = rand((M, K), M, torch.float32).clamp_(-50, 50).to(dt)
+        B = rand((N, K), N + 1, torch.float32, 0.05).to(dt)
+    else:
+        A, B = rand((M, K), M, dt), rand((N, K), N + 1, dt, 0.05)
+    C = run_abi(abi, A, B, ac.AUTO, 0.5)
+    check(C, A, B, 0.5)
+    assert oracle.rel_frobenius(C, oracle.c_gemm_tn_f32(A, B, 0.5)) <= TOL[dt]
+    assert torch.equal(run_abi(abi, A, B, ac.AUTO, 0.5).view(torch.int16), C.view(torch.int16))
+
+
 @pytest.mark.parametrize("dt,M,N,K", [(torch.bfloat16, 8200, 128, 4096), (torch.float16, 12289, 100, 2056), (torch.float8_e4m3fn, 8192, 96, 8208),
                                       (torch.bfloat16, 32768, 64, 1024)])
 def test_one_tile_column_on_the_nine_slot_ring(abi, dt, M, N, K):

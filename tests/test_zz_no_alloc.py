@@ -113,3 +113,44 @@ def test_noalloc_refuses_what_does_not_fit(abi):
     assert ac.gemm_tn_noalloc(abi, A, B, C) == ac.ERR_SCRATCH
     torch.cuda.synchronize()
     assert torch.isnan(C.float()).all()
+
+
+def test_noalloc_under_graph_capture_replays(abi):
+    """What the entry point is for: one warm call outside any capture (the per-GPU scratch address is
+    looked up on the first call), then two calls captured into one graph on one stream -- a K-split
+    problem followed by a smaller one whose partial planes overlap the first one's in the shared
+    buffer -- replayed with new operand contents, eager work in between, every replay bit for bit
+    what mi355_gemm_tn gives.  A replay finds the previous replay's partial planes in the buffer."""
+    shapes = [(64, 4096, 14336), (16, 6144, 4096)]
+    for M, N, K in shapes:
+        assert abi.mi355_gemm_workspace_bytes(M, N, K, ac.BF16, ac.AUTO) > 0
+    ops = [(torch.empty(M, K, dtype=torch.bfloat16, device="cuda").normal_(),
+            torch.empty(N, K, dtype=torch.bfloat16, device="cuda").normal_(),
+            torch.full((M, N), float("nan"), dtype=torch.bfloat16, device="cuda")) for M, N, K in shapes]
+
+    def both_calls():
+        for A, B, C in ops:
+            assert ac.gemm_tn_noalloc(abi, A, B, C) == ac.OK
+
+    print("noalloc graph capture", flush=True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        both_calls()                              # the warm call, outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        both_calls()
+    for replay in range(3):
+        for A, B, C in ops:
+            A.normal_()
+            B.normal_()
+            C.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for A, B, C in ops:
+            want = torch.full_like(C, float("nan"))
+            assert ac.gemm_tn(abi, A, B, want) == ac.OK     # eager work between the replays
+            torch.cuda.synchronize()
+            assert same_bits(C, want), (replay, tuple(C.shape))
