@@ -174,6 +174,13 @@ def build_case(name, variant, device="cuda", seed=0):
         A, sa, B, sb = w.mxfp8_8192(seed, device)
         # weights-style call: the block scales are re-laid once, outside the timed launches
         sets, tag, fp8 = [(A, B)], "e4m3", ("mx", gemm_kernels.shuffle_mx_scales(sa), gemm_kernels.shuffle_mx_scales(sb))
+    elif name.startswith("bf16_shape_") or name.startswith("fp16_shape_"):
+        # any shape: bf16_shape_M_N_K / fp16_shape_M_N_K, Normal(0,1) operands
+        M, N, K = (int(x) for x in name.split("_")[2:])
+        dt = torch.bfloat16 if name.startswith("bf16") else torch.float16
+        gen = torch.Generator(device=device).manual_seed(seed)
+        sets = [(torch.randn(M, K, device=device, generator=gen).to(dt), torch.randn(N, K, device=device, generator=gen).to(dt))]
+        tag, fp8 = ("bf16" if dt == torch.bfloat16 else "f16"), None
     elif name.startswith("skinny_"):
         M, N, K = (int(x) for x in name.split("_")[1:])
         # rotate operand sets so weights come from HBM, not the Infinity Cache (256 MB)

@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "gemm_kernels")
 LIB = os.path.join(OUT, "libmi355gemm.so")
 
-HIP_SOURCES = ["gemm_api.hip", "gemm_tn_simple.hip", "gemm_tn_ring_bf16.hip", "gemm_tn_ring_f16.hip", "gemm_tn_ring_e4m3.hip", "gemm_tn_ring_mx.hip", "ring_plan.hip", "gemm_tn_pingpong.hip", "gemm_tn_stream.hip", "quantize_e4m3.hip", "mx_scales.hip", "calibrate.hip"]
+HIP_SOURCES = ["gemm_api.hip", "gemm_tn_simple.hip", "gemm_tn_ring_bf16.hip", "gemm_tn_ring_f16.hip", "gemm_tn_ring_e4m3.hip", "gemm_tn_ring_mx.hip", "ring_plan.hip", "gemm_tn_pingpong.hip", "gemm_tn_alternate.hip", "gemm_tn_stream.hip", "quantize_e4m3.hip", "mx_scales.hip", "calibrate.hip"]
 
 # Sources whose device assembly is verified after compilation (check_async_loads.py): the copies'
 # LDS base in all of them, the asynchronous scale loads in the block-scaled one.
@@ -25,7 +25,7 @@ CHECKED_SOURCES = ["gemm_tn_ring_bf16.hip", "gemm_tn_ring_f16.hip", "gemm_tn_rin
 CHECKED_SOURCE = "gemm_tn_ring_mx.hip"
 # Sources whose kernels must keep the hardware's distances the compiler does not enforce (wide
 # stores and their data registers, inline-assembly MFMAs and their results): every GEMM kernel.
-HAZARD_SOURCES = CHECKED_SOURCES + ["gemm_tn_pingpong.hip", "gemm_tn_stream.hip", "calibrate.hip"]
+HAZARD_SOURCES = CHECKED_SOURCES + ["gemm_tn_pingpong.hip", "gemm_tn_alternate.hip", "gemm_tn_stream.hip", "calibrate.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",

@@ -57,6 +57,19 @@ bool auto_streams(int64_t M, int64_t N, int64_t K, int64_t es) {
   if (mi355::ring_one_row_deep(M, N, K, (int)es)) return false;
   return M <= 128 && (N + 63) / 64 <= 256 && M * K * es <= 2200000;
 }
+// Two workgroups per CU on 256 x 128 tiles, one storing while the other computes: where a tile is
+// nearly all epilogue.  The kernel copies 1.5 times the bytes per flop of the 256 x 256 tile and a CU
+// takes in no more than about 44 bytes per cycle, so its k loop is 13-17 % slower than the single
+// group's (bf16 8192^3: 1392 against 1625 TFLOP/s); what it hides is the store phase.  bf16, against
+// the rest of the planner: K = 256 at 16384^2 / 8192 x 16384 / 4096 x 8192 / 8192^2 / 6144^2 14 / 12 /
+// 10 / 7 / 1-5 % faster, K = 128 at 16384^2 / 8192^2 10 / 3 %; K = 320 and 384 (five and six k-steps)
+// 2 % slower, K = 512 from 2 % faster (8192^2) to 7 % slower (16384 x 8192).  So: 16-bit inputs (the
+// kernel has no fp8 form), at most four k-steps, at least two tiles per resident workgroup.
+bool auto_alternates(int64_t M, int64_t N, int64_t K, int in_dtype) {
+  if (in_dtype == MI355_E4M3) return false;
+  const int64_t k_steps = (K * 2 + 127) / 128, tiles = ((M + 255) / 256) * ((N + 127) / 128);
+  return k_steps >= 1 && k_steps <= 4 && tiles >= 1024;
+}
 bool skinny_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int in_dtype) {
   if (M > 256) return false;
   return tile256_ok(M, N, K, lda, ldb, ldc, in_dtype);
@@ -65,7 +78,7 @@ bool skinny_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_
 int check_common(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc,
                  int in_dtype, int out_dtype, int variant) {
   if (!valid_in(in_dtype) || !valid_out(out_dtype)) return MI355_ERR_DTYPE;
-  if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_SIMPLE) return MI355_ERR_VARIANT;
+  if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_ALTERNATE) return MI355_ERR_VARIANT;
   if (M < 0 || N < 0 || K < 0) return MI355_ERR_SHAPE;
   if (lda < K || ldb < K || ldc < N) return MI355_ERR_SHAPE;
   if (!extents_ok(M, N, K, lda, ldb, ldc)) return MI355_ERR_SHAPE;
@@ -78,12 +91,17 @@ int resolve(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t l
     if (!tile256_ok(M, N, K, lda, ldb, ldc, in_dtype)) return MI355_VARIANT_SIMPLE;
     // A few rows of activations against a large weight matrix: stream the weights.
     if (auto_streams(M, N, K, elem_bytes(in_dtype)) && skinny_ok(M, N, K, lda, ldb, ldc, in_dtype)) return MI355_VARIANT_SKINNY;
+    if (auto_alternates(M, N, K, in_dtype)) return MI355_VARIANT_ALTERNATE;
     return MI355_VARIANT_BASIC;
   }
   if (variant == MI355_VARIANT_BASIC || variant == MI355_VARIANT_PINGPONG)
     return tile256_ok(M, N, K, lda, ldb, ldc, in_dtype) ? variant : MI355_ERR_SHAPE;
   if (variant == MI355_VARIANT_SKINNY)
     return skinny_ok(M, N, K, lda, ldb, ldc, in_dtype) ? variant : MI355_ERR_SHAPE;
+  if (variant == MI355_VARIANT_ALTERNATE) {
+    if (in_dtype == MI355_E4M3) return MI355_ERR_VARIANT;   // 16-bit inputs only
+    return tile256_ok(M, N, K, lda, ldb, ldc, in_dtype) ? variant : MI355_ERR_SHAPE;
+  }
   return variant;
 }
 
@@ -218,7 +236,7 @@ int mi355_gemm_select_variant(int64_t M, int64_t N, int64_t K, int in_dtype) {
 int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant, int* tile_rows, int* tile_cols,
                     int* k_splits, int* tail_tiles, int* tail_splits) {
   if (!valid_in(in_dtype)) return MI355_ERR_DTYPE;
-  if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_SIMPLE) return MI355_ERR_VARIANT;
+  if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_ALTERNATE) return MI355_ERR_VARIANT;
   if (M < 0 || N < 0 || K < 0 || !extents_ok(M, N, K, K, K, N)) return MI355_ERR_SHAPE;
   const int v = resolve(M, N, K, K, K, N, in_dtype, variant);
   if (v < 0) return v;
@@ -231,6 +249,9 @@ int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant, 
     splits = mi355::stream_splits(M, N, K, es);
   } else if (v == MI355_VARIANT_PINGPONG) {
     rows = cols = 256;
+  } else if (v == MI355_VARIANT_ALTERNATE) {
+    rows = 256;
+    cols = 128;
   } else if (v == MI355_VARIANT_BASIC) {
     const int tile = mi355::ring_tile_edge(M, N, K, es);
     rows = mi355::ring_tile_rows(tile);
@@ -248,7 +269,7 @@ int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant, 
 
 size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int in_dtype, int variant) {
   if (!valid_in(in_dtype) || M <= 0 || N <= 0 || K <= 0) return 0;
-  if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_SIMPLE) return 0;
+  if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_ALTERNATE) return 0;
   if (!extents_ok(M, N, K, K, K, N)) return 0;
   const int v = resolve(M, N, K, K, K, N, in_dtype, variant);
   if (v == MI355_VARIANT_SIMPLE && variant == MI355_VARIANT_AUTO) {
@@ -472,7 +493,7 @@ int run_gemm(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_
   g.mx_a = g.mx_b = nullptr;
   hipStream_t s = (hipStream_t)stream;
 
-  if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG || v == MI355_VARIANT_SKINNY) {
+  if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG || v == MI355_VARIANT_SKINNY || v == MI355_VARIANT_ALTERNATE) {
     const bool aligned = ((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) && ((uintptr_t)C % 8 == 0);
     if (!aligned) {
       if (variant != MI355_VARIANT_AUTO) return MI355_ERR_ALIGN;
@@ -555,6 +576,11 @@ int run_gemm(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_
     g.tiles_n = (N + mi355::ring_tile_cols(tile) - 1) / mi355::ring_tile_cols(tile);
     rc = v == MI355_VARIANT_PINGPONG ? mi355::launch_tile256_pingpong(g, in_dtype, out_dtype, s)
                                      : mi355::launch_tile_ring(g, in_dtype, out_dtype, tile, s);
+  } else if (v == MI355_VARIANT_ALTERNATE) {
+    if (dry) return MI355_OK;
+    g.tiles_m = (M + 255) / 256;
+    g.tiles_n = (N + 127) / 128;
+    rc = mi355::launch_tile_alternate(g, in_dtype, out_dtype, s);
   } else {
     if (dry) return MI355_OK;
     g.tiles_m = g.tiles_n = 0;

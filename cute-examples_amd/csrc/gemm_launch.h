@@ -46,6 +46,8 @@ __device__ __forceinline__ float output_scale(const GemmArgs& g) {
 // Each returns 0 after a successful enqueue, non-zero if the runtime rejected the launch.
 // in_dtype / out_dtype use the numbering of enum mi355_dtype.
 int launch_tile256_pingpong(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
+// Two workgroups per CU on 256x128 tiles (g.tiles_n counts 128-column tiles); bf16 / fp16 inputs only.
+int launch_tile_alternate(const GemmArgs& g, int in_dtype, int out_dtype, hipStream_t stream);
 // Single-wave-group ring kernel.  `tile` is 256 or 128 (square tiles) or kRingTile256x128 (256 rows
 // of A by 128 rows of B); ring_tile_edge, ring_splits and ring_tail are pure host heuristics.
 constexpr int kRingTile256x128 = 384;

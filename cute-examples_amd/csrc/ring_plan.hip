@@ -4,6 +4,8 @@
 // compile-time tile choice of DefaultConfig (kernels/gemm_kernels/sm90a/gemm.cuh:420-451) and the
 // Scheduler's round structure (gemm.cuh:168-212).
 #include "gemm_launch.h"
+
+#include <cstdlib>
 #include "ring_common.h"
 
 namespace mi355 {
@@ -154,6 +156,14 @@ bool ring_one_row_deep(int64_t M, int64_t N, int64_t K, int elem_bytes) {
 // one row or column of tiles and for two rows first, then the shortest estimate, a larger tile being
 // preferred within 2 % (it moves fewer bytes).
 int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_scaled) {
+  // For measurements: MI355_RING_TILE = 256, 128, 384 (256 x 128), 129 (128 x 128 on nine slots, staggered
+  // start) or 130 (nine slots, plain) overrides the choice below, so that a profiler can be pointed at a
+  // form the planner would not take (the nine-slot forms exist without block scales only).
+  if (const char* force = std::getenv("MI355_RING_TILE")) {
+    const int t = std::atoi(force);
+    if (t == 256 || t == 128 || t == kRingTile256x128 || (!block_scaled && (t == kRingTile128Deep || t == kRingTile128DeepPlain)))
+      return t;
+  }
   // One or two rows of 128 x 128 tiles that nearly fill the CUs in one round, and a short K: every
   // workgroup streams its own rows of B from HBM, which the nine-slot ring keeps further ahead of the
   // MFMAs than the five-slot one can, and unsplit tiles spare the partial planes of a K split.

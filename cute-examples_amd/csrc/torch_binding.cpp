@@ -33,7 +33,8 @@ int variant_code(const std::string& v) {
   if (v == "pingpong") return MI355_VARIANT_PINGPONG;
   if (v == "skinny") return MI355_VARIANT_SKINNY;
   if (v == "simple") return MI355_VARIANT_SIMPLE;
-  TORCH_CHECK(false, "unknown variant '", v, "' (expected auto, basic, pingpong, skinny or simple)");
+  if (v == "alternate") return MI355_VARIANT_ALTERNATE;
+  TORCH_CHECK(false, "unknown variant '", v, "' (expected auto, basic, pingpong, alternate, skinny or simple)");
 }
 
 const char* variant_name(int v) {
@@ -43,6 +44,7 @@ const char* variant_name(int v) {
     case MI355_VARIANT_PINGPONG: return "pingpong";
     case MI355_VARIANT_SKINNY: return "skinny";
     case MI355_VARIANT_SIMPLE: return "simple";
+    case MI355_VARIANT_ALTERNATE: return "alternate";
   }
   return "?";
 }

@@ -38,7 +38,9 @@ enum mi355_variant {
   MI355_VARIANT_BASIC = 1,    /* 256x256, 256x128 or 128x128 tile, one wave group, LDS ring   */
   MI355_VARIANT_PINGPONG = 2, /* same tile, two wave groups alternating MFMA and load phases   */
   MI355_VARIANT_SKINNY = 3,   /* small-M weight-streaming kernel with split-K                  */
-  MI355_VARIANT_SIMPLE = 4    /* one thread per output element; any shape; slow; self-check    */
+  MI355_VARIANT_SIMPLE = 4,   /* one thread per output element; any shape; slow; self-check    */
+  MI355_VARIANT_ALTERNATE = 5 /* 256x128 tiles, two workgroups per CU alternating whole tiles: one
+                                 workgroup's stores run under the other's MFMAs; bf16/fp16 inputs   */
 };
 
 /* Status codes (0 = success, negative = error; see mi355_gemm_strerror). */

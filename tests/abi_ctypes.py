@@ -9,7 +9,7 @@ LIB = os.path.join(ROOT, "cute-examples_amd", "gemm_kernels", "libmi355gemm.so")
 HEADER = os.path.join(ROOT, "include", "mi355_gemm.h")
 
 BF16, F16, E4M3, F32 = 0, 1, 2, 3
-AUTO, BASIC, PINGPONG, SKINNY, SIMPLE = 0, 1, 2, 3, 4
+AUTO, BASIC, PINGPONG, SKINNY, SIMPLE, ALTERNATE = 0, 1, 2, 3, 4, 5
 OK, ERR_NULL, ERR_DTYPE, ERR_SHAPE, ERR_VARIANT, ERR_WORKSPACE, ERR_LAUNCH, ERR_ALIGN, ERR_SCRATCH = 0, -1, -2, -3, -4, -5, -6, -7, -8
 NOALLOC_SCRATCH_BYTES = 64 << 20
 

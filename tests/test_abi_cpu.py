@@ -246,6 +246,30 @@ def test_select_variant(abi):
     assert abi.mi355_gemm_select_variant(8192, 8192, 8192, 9) == ac.ERR_DTYPE
 
 
+def test_alternate_variant_in_the_plan(abi):
+    """Two workgroups per CU on 256x128 tiles: AUTO takes it for 16-bit inputs with at most four
+    k-steps and at least 1024 tiles (tiles that are nearly all epilogue); explicitly it takes any
+    problem the tiled kernels take, except fp8; it never wants a workspace."""
+    sel = abi.mi355_gemm_select_variant
+    assert sel(8192, 8192, 256, ac.BF16) == ac.ALTERNATE
+    assert sel(16384, 16384, 128, ac.F16) == ac.ALTERNATE
+    assert sel(4096, 8192, 200, ac.BF16) == ac.ALTERNATE          # 16 x 64 tiles, four k-steps (the last ragged)
+    assert sel(8192, 8192, 320, ac.BF16) == ac.BASIC              # five k-steps
+    assert sel(4096, 4096, 256, ac.BF16) == ac.BASIC              # 512 tiles: one per workgroup
+    assert sel(8192, 8192, 256, ac.E4M3) == ac.BASIC              # fp8: two k-steps, but no such kernel
+    assert sel(64, 4096 * 128, 256, ac.BF16) == ac.SKINNY         # few rows: the streaming kernel comes first
+    assert ac.plan(abi, 8192, 8192, 256, ac.BF16) == (ac.ALTERNATE, 256, 128, 1, 0, 1)
+    assert ac.plan(abi, 1000, 1004, 4096, ac.F16, ac.ALTERNATE) == (ac.ALTERNATE, 256, 128, 1, 0, 1)
+    assert ac.plan(abi, 8192, 8192, 8192, ac.E4M3, ac.ALTERNATE)[0] == ac.ERR_VARIANT
+    assert abi.mi355_gemm_check(512, 512, 64, 64, 64, 512, ac.E4M3, ac.BF16, ac.ALTERNATE) == ac.ERR_VARIANT
+    assert abi.mi355_gemm_check(512, 512, 68, 68, 68, 512, ac.BF16, ac.BF16, ac.ALTERNATE) == ac.ERR_SHAPE   # K bytes % 16
+    assert abi.mi355_gemm_check(512, 512, 72, 72, 72, 512, ac.BF16, ac.F16, ac.ALTERNATE) == ac.OK
+    assert abi.mi355_gemm_check(512, 512, 72, 72, 72, 512, ac.BF16, ac.F16, 6) == ac.ERR_VARIANT
+    for M, N, K in [(8192, 8192, 256), (8192, 8192, 8192), (300, 200, 64)]:
+        assert abi.mi355_gemm_workspace_bytes(M, N, K, ac.BF16, ac.ALTERNATE) == 0
+    assert abi.mi355_gemm_workspace_bytes(8192, 8192, 256, ac.BF16, ac.AUTO) == 0
+
+
 @pytest.mark.parametrize("tm,tn", [(32, 32), (16, 16), (1, 1), (1, 56), (3, 5), (7, 9), (33, 31), (2, 24), (17, 1),
                                    (17, 17), (17, 16), (64, 64)])
 def test_tile_map_is_a_bijection(abi, tm, tn):
@@ -309,6 +333,7 @@ def test_plan_invariants_over_random_shapes(abi):
     import random
     rng = random.Random(7)
     seen = set()
+    seen_alternate = False
     for dt, es in ((ac.BF16, 2), (ac.F16, 2), (ac.E4M3, 1)):
         for _ in range(3000):
             M = rng.choice([rng.randint(1, 300), rng.randint(1, 5000), rng.randint(1, 20000)])
@@ -316,7 +341,14 @@ def test_plan_invariants_over_random_shapes(abi):
             K = (16 // es) * rng.choice([rng.randint(1, 64), rng.randint(1, 1024), rng.randint(1, 4096)])
             v, rows, cols, splits, tail_tiles, tail_splits = ac.plan(abi, M, N, K, dt)
             steps = -(-K * es // 128)
-            assert v in (ac.BASIC, ac.SKINNY), (M, N, K, v)
+            # two workgroups per CU: 16-bit inputs, at most four k-steps, at least 1024 tiles of 256x128
+            alternates = es == 2 and steps <= 4 and -(-M // 256) * -(-N // 128) >= 1024
+            if v == ac.ALTERNATE:
+                assert alternates and (rows, cols, splits, tail_tiles) == (256, 128, 1, 0), (M, N, K)
+                assert abi.mi355_gemm_workspace_bytes(M, N, K, dt, ac.AUTO) == 0
+                seen_alternate = True
+                continue
+            assert v in (ac.BASIC, ac.SKINNY) and (not alternates or v == ac.SKINNY), (M, N, K, v)
             one_row = -(-N // 128)      # 65...128 rows: one row of 128x128 tiles on the nine-slot ring
             parts = max([1] + [p for p in range(2, 17) if one_row * p <= 256 and steps // p >= 16])
             deep = M <= 128 and one_row <= 256 and one_row * parts >= 96 and (one_row >= 32 or (one_row >= 16 and steps >= 128))
@@ -340,7 +372,7 @@ def test_plan_invariants_over_random_shapes(abi):
                     want = tail_tiles * tail_splits * 256 * 256 * 4
                 seen.add((rows, cols, splits > 1, tail_tiles > 0))
             assert abi.mi355_gemm_workspace_bytes(M, N, K, dt, ac.AUTO) == want, (M, N, K)
-    assert len(seen) >= 7, seen
+    assert len(seen) >= 7 and seen_alternate, seen
 
 
 def test_noalloc_entry_point_decides_before_any_hip_call(abi):

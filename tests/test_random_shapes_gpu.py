@@ -42,7 +42,7 @@ def test_random_problems_against_fp32_matmul(abi, seed):
         N = 4 * rng.choice([rng.randint(1, 40), rng.randint(1, 400), rng.randint(1, 1500)])
         K = per16 * rng.choice([rng.randint(1, 16), rng.randint(1, 200), rng.randint(1, 1100)])
         lda, ldb, ldc = K + per16 * rng.choice([0, 0, 1, 5]), K + per16 * rng.choice([0, 0, 2, 7]), N + 4 * rng.choice([0, 0, 1, 9])
-        v = rng.choice([ac.AUTO, ac.BASIC, ac.PINGPONG] + ([ac.SKINNY] if M <= 256 else []))
+        v = rng.choice([ac.AUTO, ac.BASIC, ac.PINGPONG] + ([ac.ALTERNATE] if es == 2 else []) + ([ac.SKINNY] if M <= 256 else []))
         if v == ac.AUTO and rng.random() < 0.4:   # AUTO takes anything: the generic kernel, or repacking
             N, K = max(1, N - rng.randint(0, 3)), max(1, K - rng.randint(0, per16 - 1))
             lda, ldb, ldc = K + rng.choice([0, 0, 1, 5]), K + rng.choice([0, 0, 3]), N + rng.choice([0, 0, 1, 3])
