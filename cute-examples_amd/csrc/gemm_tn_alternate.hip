@@ -18,23 +18,26 @@
 //
 // LDS of a workgroup: 80 KiB = two 32 KiB slots of A (256 rows x 128 B, one k-step each) and ONE
 // 16 KiB slot of B (128 rows).  k-step t computes from A slot t%2 and the B slot while A(t+1) sits in
-// (or is on its way into) the other A slot.  The one B slot is refilled as soon as every wave holds
-// the k-step's B fragments in registers, and read again at the end of the k-step: B is the operand
-// with the short flight time, which the other workgroup's MFMAs cover.
+// (or is on its way into) the other A slot.  The one B slot is refilled early in the k-step, as soon
+// as every wave holds both K-halves of B(t) in registers, and must be back by the middle of it: B is
+// the operand with the short flight time (about half a k-step of the workgroup's own MFMAs, twice
+// that on the clock while the other workgroup takes its turns).
 //
-// Schedule of a k-step inside a wave (16-bit types; two slices = the two 64-byte halves of K; 32
-// MFMAs per slice, A-major: row block i of A against the four blocks of B):
+// Schedule of a k-step inside a wave (two slices = the two 64-byte halves of K; 32 MFMAs per slice,
+// A-major: row block i of A against the four blocks of B):
 //   slice 0   MFMAs on fa[0..7] (A(t) slice 0) and fb[0][..] (B(t) slice 0)
 //             reads: fb[1][..] <- B(t) slice 1 at the start; fa[i] <- A(t) slice 1, in place, one MFMA
 //             after the last MFMA of row i (a row is next used 32 MFMAs later)
+//             after row 1: lgkmcnt(1), s_barrier -- the B slot is free; copies B(t+1) -> B slot
 //   slice 1   MFMAs on fa (now slice 1) and fb[1]
-//             after row 0: lgkmcnt(0), vmcnt(0), s_barrier  -- every wave has read the k-step's slots,
-//             and A(t+1) has landed; then the copies B(t+1) -> B slot, A(t+2) -> the slot of A(t),
-//             spread over the rest of the slice
-//             reads: fa[i] <- A(t+1) slice 0, in place, two rows behind the MFMAs
-//   end       fa[6], fa[7] <- A(t+1); vmcnt(8) (B(t+1) landed, A(t+2) may fly), s_barrier,
-//             fb[0][..] <- B(t+1) slice 0
+//             after row 1: lgkmcnt(0), vmcnt(0), s_barrier -- every wave has read the slot of A(t);
+//             A(t+1) and B(t+1) have landed; then the copies A(t+2) -> the slot of A(t), spread over
+//             the rest of the slice
+//             reads: fb[0][..] <- B(t+1) slice 0 right after the barrier; fa[i] <- A(t+1) slice 0, in
+//             place, two rows behind the MFMAs
 // Two workgroup barriers per k-step; every wait in this list is time the other workgroup computes in.
+// (A first form refilled the B slot together with A's, after the second barrier, and waited for it
+// with a third barrier at the end of the k-step: 3-4 % slower from 16 k-steps on.)
 //
 // 16-bit input types only.
 #include "gemm_launch.h"
@@ -205,50 +208,50 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_tile_alternate(GemmArgs g) {
         const uint8_t* a_rows = lds + slot * kAltSlotA + a_lane;          // A(t)
         const uint8_t* a1_rows = lds + (slot ^ 1) * kAltSlotA + a_lane;   // A(t+1)
         const uint8_t* b_rows = lds + b_lane;
-        constexpr int kCopies = kCphB + kCphA;
-        // The k-step's sync point: every wave has read the slots of k-step t, A(t+1) has landed.
+        // Second sync point of the k-step: every wave has read the slot of A(t); A(t+1) and B(t+1) have landed.
         auto slots_free = [&]() __attribute__((always_inline)) {
           wait_lgkmcnt0();
           wait_vmcnt<0>();
           __builtin_amdgcn_s_barrier();
         };
-        // copy c of the k-step: B(t+1) first (it is needed first), then A(t+2) into the slot of A(t)
-        auto copy_c = [&](auto cc) __attribute__((always_inline)) {
-          constexpr int c = decltype(cc)::value;
-          if constexpr (c < kCphB) copy_b(rsrc_b, std::integral_constant<int, c>{}, soff_b);
-          else copy_a(rsrc_a, std::integral_constant<int, c - kCphB>{}, std::integral_constant<int, slot>{}, soff_a);
-        };
         {
           constexpr int kPerSlice = kNbA * kNbB;   // 32
           // ---- slice 0
+          constexpr int kSyncB = 2 * kNbB;                    // after row 1: the B slot is free
           static_for<kPerSlice>([&](auto uc) __attribute__((always_inline)) {
             constexpr int u = decltype(uc)::value, i = u / kNbB, j = u % kNbB;
             if constexpr (u < kNbB) fb[1][u] = load_frag(b_rows, u, 1);
             if constexpr (u >= kNbB && j == 1) fa[i - 1] = load_frag(a_rows, i - 1, 1);   // one MFMA after the row's last use
+            if constexpr (u == kSyncB) {
+              // Every wave holds both slices of B(t) in registers (fb[0] since the previous k-step, fb[1]
+              // from the loads above; the one younger LDS read is the first reload of A).
+              wait_lgkmcnt<1>();
+              __builtin_amdgcn_s_barrier();
+            }
+            if constexpr (u >= kSyncB && (u - kSyncB) % 2 == 0 && (u - kSyncB) / 2 < kCphB)
+              copy_b(rsrc_b, std::integral_constant<int, (u - kSyncB) / 2>{}, soff_b);           // B(t+1)
             G::mfma_inplace(fb[0][j], fa[i], acc[i][j]);
             MI355_FENCE();
           });
           // ---- slice 1 (the last row of A's slice 1 is loaded behind its first MFMA)
-          constexpr int kSync = kNbB;                         // after row 0
+          constexpr int kSync = 2 * kNbB;                   // after row 1: the slot of A(t) is free (its last read is 7 MFMAs old)
+          static_assert(kSync <= 2 * kNbB, "the first read of A(t+1) follows the sync");
           constexpr int kFirstCopy = kSync + 1, kSpan = kPerSlice - kFirstCopy;
           static_for<kPerSlice>([&](auto uc) __attribute__((always_inline)) {
             constexpr int u = decltype(uc)::value, i = u / kNbB, j = u % kNbB;
             if constexpr (u == 1) fa[kNbA - 1] = load_frag(a_rows, kNbA - 1, 1);
-            if constexpr (u == kSync) slots_free();
+            if constexpr (u == kSync) slots_free();           // ... and A(t+1), B(t+1) have landed
+            if constexpr (u > kSync && u <= kSync + kNbB) fb[0][u - kSync - 1] = load_frag(b_rows, u - kSync - 1, 0);   // B(t+1)
             if constexpr (u >= 2 * kNbB && j == 0) fa[i - 2] = load_frag(a1_rows, i - 2, 0);
-            static_for<kCopies>([&](auto cc) __attribute__((always_inline)) {
-              if constexpr (kFirstCopy + decltype(cc)::value * kSpan / kCopies == u) copy_c(cc);
+            static_for<kCphA>([&](auto cc) __attribute__((always_inline)) {
+              if constexpr (kFirstCopy + decltype(cc)::value * kSpan / kCphA == u)
+                copy_a(rsrc_a, cc, std::integral_constant<int, slot>{}, soff_a);                 // A(t+2)
             });
             G::mfma_inplace(fb[1][j], fa[i], acc[i][j]);
             MI355_FENCE();
           });
           fa[kNbA - 2] = load_frag(a1_rows, kNbA - 2, 0);
           fa[kNbA - 1] = load_frag(a1_rows, kNbA - 1, 0);
-          MI355_FENCE();
-          wait_vmcnt<kCphA>();             // B(t+1) has landed; the copies of A(t+2) are younger
-          __builtin_amdgcn_s_barrier();
-#pragma unroll
-          for (int j = 0; j < kNbB; ++j) fb[0][j] = load_frag(b_rows, j, 0);
           MI355_FENCE();
         }
         soff_b = soff_b + kRowBytes < soff_last ? soff_b + kRowBytes : soff_last;
