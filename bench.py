@@ -253,8 +253,7 @@ def roofline_of(row, workload, variant, sets, flops, nbytes):
         roof = {"bound": "hbm", "achieved": row["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(row["gbs"] / PEAK_HBM_GBS, 4), "traffic": traffic}
     # the counters are not read in this run: the figure is the one of the committed profile of this command
-    roof["traffic_source"] = (TRAFFIC_PROFILE[workload] + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this "
-                              "script, scaled by a 1 GiB copy; not re-measured in this run)") if traffic else None
+    roof["traffic_source"] = (TRAFFIC_PROFILE[workload] + " (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this script; not re-measured)") if traffic else None
     roof["kernel"] = gemm_kernels.select_variant(row["M"], row["N"], row["K"], sets[0][0].dtype) \
         if variant == "auto" else variant
     roof["flops_per_launch"] = flops
@@ -390,32 +389,55 @@ def cpu_baseline(A, B, total_rows, scale=1.0, budget_s=12.0, native_budget_s=5.0
     kind = "e4m3->fp32" if Ac.dtype == torch.float8_e4m3fn else "%s->fp32" % str(Ac.dtype).split(".")[-1]
     return {"value": round(tflops, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(),
             "kind": "port", "native_16bit_value": native,
-            "sample": "torch.matmul fp32 (incl. the %s casts) of %d-row blocks of A against all of B "
-                      "(N=%d, K=%d), %d rows in %.1f s; host has %d logical cpus"
-                      % (kind, rows, N, K, done, el, os.cpu_count())}
+            "sample": "%d rows in %.1f s: %d-row blocks of A x all of B (N=%d, K=%d), fp32 torch.matmul incl. %s casts; %d cpus"
+                      % (done, el, rows, N, K, kind, os.cpu_count())}
 
 
-def other_configs(extras, mfma_ceiling, hbm_read):
-    """The other configurations the baseline names (the nine small-M projection shapes, bf16 4096^3,
-    fp16 512^3) in brief: time per launch, achieved rate, fraction of the published peak and of the
-    ceiling measured in this run (MFMA-only loop on the headline's operands / plain read)."""
-    wanted = ["bf16_4096", "fp16_512"] + ["skinny_%d_%d_%d" % (m, n, k) for (n, k) in ((14336, 4096), (4096, 14336), (6144, 4096))
-                                          for m in (16, 64, 256)]
-    out = {}
-    for row in extras:
-        name = row["workload"]
-        if name not in wanted or "variant" in row:
-            continue
-        if name.startswith("skinny"):
-            e = {"ms": row["ms"], "achieved": row["gbs"], "unit": "GB/s", "bound": "hbm",
-                 "frac": round(row["gbs"] / PEAK_HBM_GBS, 4),
-                 "frac_of_measured_ceiling": round(row["gbs"] / hbm_read["value"], 4) if hbm_read else None}
-        else:
-            e = {"ms": row["ms"], "achieved": row["tflops"], "unit": "TFLOP/s", "bound": "mfma",
-                 "frac": round(row["tflops"] / PEAK_TFLOPS[row["dtype"]], 4),
-                 "frac_of_measured_ceiling": round(row["tflops"] / mfma_ceiling["value"], 4) if mfma_ceiling else None}
-        out[name] = e
-    return out
+def flatten_into(roof, fp8_block):
+    """The nested entries of the roofline object once more as scalar fields of it (plain numbers under
+    systematic names), for readers that keep only the scalar fields of this object."""
+    def tag(shape):
+        return shape.replace("x", "_")
+    ceil = roof.get("measured_mfma_ceiling")
+    if ceil:
+        roof["measured_mfma_ceiling_tflops"] = ceil["value"]
+        roof["mfma_ceiling_zero_operands_tflops"] = ceil.get("value_zero_operands")
+        for shape, v in (ceil.get("by_shape") or {}).items():
+            roof["mfma_ceiling_%s_tflops" % tag(shape)] = v
+    if roof.get("measured_hbm_read"):
+        roof["measured_hbm_read_gbs"] = roof["measured_hbm_read"]["value"]
+    if roof.get("torch_mm_same_run"):
+        roof["torch_mm_same_run_tflops"] = roof["torch_mm_same_run"]["value"]
+    prof = roof.get("profiled")
+    if prof:
+        roof["profiled_mfma_busy"], roof["profiled_shader_clock_ghz"] = prof["mfma_busy"], prof["shader_clock_ghz"]
+        roof["profiled_source"] = prof["source"]
+        if ceil:
+            # what the measured ceiling would give at the issue rate the counters show for this kernel
+            roof["measured_ceiling_times_profiled_busy_tflops"] = round(ceil["value"] * prof["mfma_busy"], 1)
+    if fp8_block:
+        r8 = fp8_block["roofline"]
+        roof["fp8_value_tflops"], roof["fp8_ms_per_step"], roof["fp8_frac"] = fp8_block["value"], fp8_block["ms_per_step"], r8["frac"]
+        c8 = r8.get("measured_mfma_ceiling")
+        if c8:
+            roof["fp8_measured_mfma_ceiling_tflops"] = c8["value"]
+            roof["fp8_frac_of_measured_ceiling"] = r8.get("frac_of_measured_ceiling")
+            for shape, v in (c8.get("by_shape") or {}).items():
+                roof["fp8_mfma_ceiling_%s_tflops" % tag(shape)] = v
+        if r8.get("torch_mm_same_run"):
+            roof["fp8_torch_scaled_mm_same_run_tflops"] = r8["torch_mm_same_run"]["value"]
+            roof["fp8_vs_torch_scaled_mm_same_run"] = r8.get("vs_torch_mm_same_run")
+        if r8.get("profiled"):
+            roof["fp8_profiled_mfma_busy"] = r8["profiled"]["mfma_busy"]
+            roof["fp8_profiled_shader_clock_ghz"] = r8["profiled"]["shader_clock_ghz"]
+        if fp8_block.get("cpu_baseline"):
+            roof["fp8_cpu_baseline_tflops"] = fp8_block["cpu_baseline"]["value"]
+    for name, e in (roof.get("other_configs") or {}).items():
+        unit = "tflops" if e["unit"] == "TFLOP/s" else "gbs"
+        roof["cfg_%s_ms" % name] = e["ms"]
+        roof["cfg_%s_%s" % (name, unit)] = e["achieved"]
+        roof["cfg_%s_frac" % name] = e["frac"]
+        roof["cfg_%s_frac_of_measured_ceiling" % name] = e["frac_of_measured_ceiling"]
 
 
 def main():
@@ -527,6 +549,7 @@ def main():
                             "see": "the top-level \"fp8\" object of this line"}
     if extras:
         roof["other_configs"] = other_configs(extras, roof.get("measured_mfma_ceiling"), roof.get("measured_hbm_read"))
+    flatten_into(roof, fp8_block)
     out = {
         "metric": METRIC, "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "settle_launches": head["settle_launches"], "settle_ms": head["settle_ms"],
@@ -535,11 +558,8 @@ def main():
         "config": {"workload": "%s: M=%d N=%d K=%d, A (M,K) and B (N,K) K-contiguous, fp32 accumulate"
                                % (a.workload, head["M"], head["N"], head["K"]),
                    "variant": roof["kernel"], "parallelism": "single GPU",
-                   "protocol": ("no settle phase; " if a.no_settle else
-                                "a clock-settle phase (the same launch for >= %d ms, until three ~%d ms batches agree "
-                                "within 1 %%; settle_launches / settle_ms) precedes the W warm-up launches; "
-                                % (SETTLE_MIN_MS, SETTLE_BATCH_MS)) +
-                               "then W warm-up and K timed launches back to back, HIP events on the launch stream"},
+                   "protocol": ("no settle; " if a.no_settle else "settle (>=%d ms, 3 batches within 1%%) precedes " % SETTLE_MIN_MS) +
+                               "W warm-up + K timed launches, HIP events on the launch stream"},
         "pct_of_dense_mfma_peak": head["pct_mfma_peak"],
         "roofline": roof, "cpu_baseline": cpu, "extras": extras, "fp8": fp8_block,
     }
