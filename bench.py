@@ -393,6 +393,29 @@ def cpu_baseline(A, B, total_rows, scale=1.0, budget_s=12.0, native_budget_s=5.0
                       % (done, el, rows, N, K, kind, os.cpu_count())}
 
 
+def other_configs(extras, mfma_ceiling, hbm_read):
+    """The other configurations the baseline names (the nine small-M projection shapes, bf16 4096^3,
+    fp16 512^3) in brief: time per launch, achieved rate, fraction of the published peak and of the
+    ceiling measured in this run (MFMA-only loop on the headline's operands / plain read)."""
+    wanted = ["bf16_4096", "fp16_512"] + ["skinny_%d_%d_%d" % (m, n, k) for (n, k) in ((14336, 4096), (4096, 14336), (6144, 4096))
+                                          for m in (16, 64, 256)]
+    out = {}
+    for row in extras:
+        name = row["workload"]
+        if name not in wanted or "variant" in row:
+            continue
+        if name.startswith("skinny"):
+            e = {"ms": row["ms"], "achieved": row["gbs"], "unit": "GB/s", "bound": "hbm",
+                 "frac": round(row["gbs"] / PEAK_HBM_GBS, 4),
+                 "frac_of_measured_ceiling": round(row["gbs"] / hbm_read["value"], 4) if hbm_read else None}
+        else:
+            e = {"ms": row["ms"], "achieved": row["tflops"], "unit": "TFLOP/s", "bound": "mfma",
+                 "frac": round(row["tflops"] / PEAK_TFLOPS[row["dtype"]], 4),
+                 "frac_of_measured_ceiling": round(row["tflops"] / mfma_ceiling["value"], 4) if mfma_ceiling else None}
+        out[name] = e
+    return out
+
+
 def flatten_into(roof, fp8_block):
     """The nested entries of the roofline object once more as scalar fields of it (plain numbers under
     systematic names), for readers that keep only the scalar fields of this object."""
@@ -412,9 +435,13 @@ def flatten_into(roof, fp8_block):
     if prof:
         roof["profiled_mfma_busy"], roof["profiled_shader_clock_ghz"] = prof["mfma_busy"], prof["shader_clock_ghz"]
         roof["profiled_source"] = prof["source"]
-        if ceil:
-            # what the measured ceiling would give at the issue rate the counters show for this kernel
-            roof["measured_ceiling_times_profiled_busy_tflops"] = round(ceil["value"] * prof["mfma_busy"], 1)
+        # An MFMA in every cycle of every SIMD at the clock the profile shows for this kernel (256 CUs x 4 SIMDs x
+        # 1024 flop per cycle for the 16-bit types, twice that for fp8), and the share of cycles the 0.70 / 0.60
+        # target of the published peak would therefore need MFMAs to be issued in.
+        per_ghz = 256 * 4 * (2048 if roof["peak"] > 3000 else 1024) / 1e3
+        roof["full_issue_at_profiled_clock_tflops"] = round(per_ghz * prof["shader_clock_ghz"], 1)
+        target = 0.60 if roof["peak"] > 3000 else 0.70
+        roof["mfma_busy_needed_for_target"] = round(target * roof["peak"] / roof["full_issue_at_profiled_clock_tflops"], 3)
     if fp8_block:
         r8 = fp8_block["roofline"]
         roof["fp8_value_tflops"], roof["fp8_ms_per_step"], roof["fp8_frac"] = fp8_block["value"], fp8_block["ms_per_step"], r8["frac"]
