@@ -120,11 +120,6 @@ __device__ __forceinline__ void wait_vmcnt_for(u32x2& a, u32x2& b) {
   asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(N) : "memory");
 }
 __device__ __forceinline__ void wait_lgkmcnt0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
-// LDS reads return in order: all but the N youngest LDS instructions of the wave are complete.
-template <int N>
-__device__ __forceinline__ void wait_lgkmcnt() {
-  asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
-}
 
 __device__ __forceinline__ uint32_t lds_address(const void* p) {
   return (uint32_t)(uintptr_t)p;

@@ -28,7 +28,7 @@
 //   slice 0   MFMAs on fa[0..7] (A(t) slice 0) and fb[0][..] (B(t) slice 0)
 //             reads: fb[1][..] <- B(t) slice 1 at the start; fa[i] <- A(t) slice 1, in place, one MFMA
 //             after the last MFMA of row i (a row is next used 32 MFMAs later)
-//             after row 1: lgkmcnt(1), s_barrier -- the B slot is free; copies B(t+1) -> B slot
+//             after row 1: lgkmcnt(0), s_barrier -- the B slot is free; copies B(t+1) -> B slot
 //   slice 1   MFMAs on fa (now slice 1) and fb[1]
 //             after row 1: lgkmcnt(0), vmcnt(0), s_barrier -- every wave has read the slot of A(t);
 //             A(t+1) and B(t+1) have landed; then the copies A(t+2) -> the slot of A(t), spread over
@@ -223,9 +223,10 @@ __global__ __launch_bounds__(256, 2) void gemm_tn_tile_alternate(GemmArgs g) {
             if constexpr (u < kNbB) fb[1][u] = load_frag(b_rows, u, 1);
             if constexpr (u >= kNbB && j == 1) fa[i - 1] = load_frag(a_rows, i - 1, 1);   // one MFMA after the row's last use
             if constexpr (u == kSyncB) {
-              // Every wave holds both slices of B(t) in registers (fb[0] since the previous k-step, fb[1]
-              // from the loads above; the one younger LDS read is the first reload of A).
-              wait_lgkmcnt<1>();
+              // Every wave holds both slices of B(t) in registers: fb[0] since the previous k-step, fb[1]
+              // from the loads above (issued at least four MFMAs ago; the wait also covers the first
+              // reload of A, three MFMAs old, so that no LDS wait in this kernel is counted by hand).
+              wait_lgkmcnt0();
               __builtin_amdgcn_s_barrier();
             }
             if constexpr (u >= kSyncB && (u - kSyncB) % 2 == 0 && (u - kSyncB) / 2 < kCphB)
