@@ -21,9 +21,9 @@
 //   slice 1: MFMAs on buffer 1 | ds_reads of slice 0 of k-step t+1 -> buffer 0
 //   from the barrier to the end of the k-step: the 16 direct-to-LDS loads of B(t+2), A(t+3),
 //            spread evenly between the MFMAs
-// One workgroup barrier and one scalar branch per k-step: a workgroup has one wave per SIMD, so
-// every branch is a bubble in its MFMA stream.  The k loop is unrolled over the five positions of
-// the ring, which makes every LDS offset an immediate; copies past the end of K re-read the last
+// One workgroup barrier per k-step and one scalar branch per turn of the ring: a workgroup has one
+// wave per SIMD, so every branch is a bubble in its MFMA stream.  The k loop is unrolled over the five
+// positions of the ring, which makes every LDS offset an immediate; copies past the end of K re-read the last
 // k-step into a slot nobody reads instead of being branched around.  The MFMAs are inline
 // assembly with the accumulator tied in place; fragment loads and everything else are compiled
 // code pinned between them with scheduling barriers.
@@ -436,9 +436,7 @@ __global__ __launch_bounds__(threads_of(kWavesN), (kTileT == 256 || kAhead > 2) 
     uint32_t mx_soff = mx_soff_of(2);
     uint32_t kt = 0;
     bool last = false;
-    for (;;) {
-    static_for<kSlots>([&](auto phase) __attribute__((always_inline)) {
-      if (last) return;
+    auto k_step = [&](auto phase) __attribute__((always_inline)) {
       constexpr uint32_t slot_a = (2 * decltype(phase)::value) % kSlots;
       constexpr uint32_t slot_b = (slot_a + 1) % kSlots, slot_a1 = (slot_a + 2) % kSlots, slot_b1 = (slot_a + 3) % kSlots;
       const uint8_t* a_rows = ring + slot_a * kSlotBytes + a_lane;
@@ -545,9 +543,18 @@ __global__ __launch_bounds__(threads_of(kWavesN), (kTileT == 256 || kAhead > 2) 
       if constexpr (kMx) mx_soff = mx_soff + kMxUnitBytes < mx_soff_last ? mx_soff + kMxUnitBytes : mx_soff_last;
       ++kt;
       last = kt == steps;
+    };
+    // Whole turns of the ring run without a test between their k-steps (a workgroup has one wave per SIMD,
+    // so every scalar branch, taken or not, is a bubble in its MFMA stream: one branch per five k-steps
+    // instead of one per k-step is worth 0.4-0.8 % on long K); the remaining k-steps go one by one.  The
+    // row-sliced kernels keep one test per k-step: with two loops around their 256 accumulator registers
+    // the register allocator carries one accumulator block through vector registers.
+    if constexpr (!kRowSliced)
+      for (uint32_t turns = steps / kSlots; turns > 0; --turns) static_for<kSlots>(k_step);
+    while (!last) static_for<kSlots>([&](auto phase) __attribute__((always_inline)) {
+      if (last) return;
+      k_step(phase);
     });
-    if (last) break;
-    }
     // The tail copies (past the end of K) must have landed, and every wave must be past its last
     // LDS read, before the ring is refilled for the next tile.
     wait_vmcnt<0>();
