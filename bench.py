@@ -43,7 +43,7 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs of this script
 # (FETCH_SIZE, then WRITE_SIZE, each with --copy-calibration and scaled by what the same counter
 # reads for the 1 GiB copy: x2.000 and x1.000).  Workloads without a counter run report null.
-MEASURED_TRAFFIC_BYTES = {"bf16_8192": 1.746e9, "fp8_8192": 0.944e9, "mxfp8_8192": 0.965e9, "bf16_4096": 2.352e8,
+MEASURED_TRAFFIC_BYTES = {"bf16_8192": 1.750e9, "fp8_8192": 0.943e9, "mxfp8_8192": 0.965e9, "bf16_4096": 2.352e8,
                           "skinny_16_14336_4096": 1.190e8, "skinny_64_14336_4096": 1.236e8, "skinny_64_4096_14336": 1.527e8,
                           "skinny_256_14336_4096": 1.561e8, "skinny_256_6144_4096": 1.209e8, "skinny_128_8192_4096": 1.130e8}
 TRAFFIC_PROFILE = {"bf16_8192": "profiles/gemm_tn_tile_ring__bf16_8192.md", "fp8_8192": "profiles/gemm_tn_tile_ring__fp8_8192.md",
@@ -59,9 +59,9 @@ SETTLE_MIN_MS, SETTLE_MAX_MS, SETTLE_BATCH_MS = 150.0, 2000.0, 10.0
 # run): the share of SIMD cycles with an MFMA in flight and the shader clock during the kernel
 # (busy CU cycles / CUs / traced duration).
 PROFILED = {
-    "bf16_8192": {"mfma_busy": 0.884, "shader_clock_ghz": 1.74, "lds_bank_conflict_cycles": 0,
+    "bf16_8192": {"mfma_busy": 0.903, "shader_clock_ghz": 1.66, "lds_bank_conflict_cycles": 0,
                   "source": "profiles/gemm_tn_tile_ring__bf16_8192.md"},
-    "fp8_8192": {"mfma_busy": 0.872, "shader_clock_ghz": 1.77, "lds_bank_conflict_cycles": 0,
+    "fp8_8192": {"mfma_busy": 0.875, "shader_clock_ghz": 1.71, "lds_bank_conflict_cycles": 0,
                  "source": "profiles/gemm_tn_tile_ring__fp8_8192.md"},
 }
 
@@ -393,6 +393,24 @@ def cpu_baseline(A, B, total_rows, scale=1.0, budget_s=12.0, native_budget_s=5.0
                       % (done, el, rows, N, K, kind, os.cpu_count())}
 
 
+def larger_shapes(steps, do_settle):
+    """Two larger bf16 problems (twice the K; twice the M and N with half the K), this library and the vendor
+    library one after the other on the same operands, same protocol.  {"M_N_K": {tflops, torch_mm_tflops, vs_torch_mm}}"""
+    import torch
+    out = {}
+    for (M, N, K) in ((8192, 8192, 16384), (16384, 16384, 4096)):
+        row, keep = measure("bf16_shape_%d_%d_%d" % (M, N, K), "auto", steps, steps, do_settle)
+        sets, C, fp8, flops, _ = keep
+        vendor = vendor_same_run(sets, C, fp8, flops, steps, steps, do_settle)
+        out["%d_%d_%d" % (M, N, K)] = {
+            "ms": row["ms"], "tflops": row["tflops"], "frac": round(row["tflops"] / PEAK_TFLOPS["bf16"], 4),
+            "torch_mm_tflops": vendor["value"],
+            "vs_torch_mm": round(row["tflops"] / vendor["value"], 4) if vendor["value"] else None}
+        del sets, C, keep
+        torch.cuda.empty_cache()
+    return out
+
+
 def other_configs(extras, mfma_ceiling, hbm_read):
     """The other configurations the baseline names (the nine small-M projection shapes, bf16 4096^3,
     fp16 512^3) in brief: time per launch, achieved rate, fraction of the published peak and of the
@@ -459,6 +477,9 @@ def flatten_into(roof, fp8_block):
             roof["fp8_profiled_shader_clock_ghz"] = r8["profiled"]["shader_clock_ghz"]
         if fp8_block.get("cpu_baseline"):
             roof["fp8_cpu_baseline_tflops"] = fp8_block["cpu_baseline"]["value"]
+    for shape, e in (roof.get("larger_shapes") or {}).items():
+        for key, v in e.items():
+            roof["bf16_%s_%s" % (shape, key)] = v
     for name, e in (roof.get("other_configs") or {}).items():
         unit = "tflops" if e["unit"] == "TFLOP/s" else "gbs"
         roof["cfg_%s_ms" % name] = e["ms"]
@@ -555,6 +576,9 @@ def main():
                 extras.append(row)
                 del keep
                 torch.cuda.empty_cache()
+
+    if a.workload == "bf16_8192" and a.variant == "auto" and not a.no_extras and not a.no_vendor:
+        roof["larger_shapes"] = larger_shapes(40, do_settle)
 
     # Last, so that the GPU does not idle (and drop its clocks) in the middle of the measurements.
     cpu = cpu_baseline(*cpu_operands) if cpu_operands else None

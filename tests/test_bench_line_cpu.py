@@ -44,6 +44,7 @@ def test_roofline_carries_every_yardstick_as_a_scalar_field():
     roof = {"bound": "mfma", "peak": 2500.0,
             "measured_mfma_ceiling": {"value": 2000.0, "value_zero_operands": 2400.0, "by_shape": {"16x16x32": 2000.0, "32x32x16": 1800.0}},
             "measured_hbm_read": {"value": 6800.0}, "torch_mm_same_run": {"value": 1660.0}, "profiled": b.PROFILED["bf16_8192"],
+            "larger_shapes": {"8192_8192_16384": {"ms": 1.42, "tflops": 1550.0, "frac": 0.62, "torch_mm_tflops": 1540.0, "vs_torch_mm": 1.0065}},
             "other_configs": b.other_configs([row("bf16_4096", 0.09, 1500.0, 1.0), row("skinny_64_6144_4096", 0.017, 1.0, 3000.0)],
                                              {"value": 2000.0}, {"value": 6800.0})}
     fp8 = {"value": 3200.0, "ms_per_step": 0.34, "cpu_baseline": {"value": 1.3},
@@ -59,11 +60,14 @@ def test_roofline_carries_every_yardstick_as_a_scalar_field():
                       ("fp8_value_tflops", 3200.0), ("fp8_frac", 0.64), ("fp8_mfma_ceiling_32_32_64_tflops", 4100.0),
                       ("fp8_torch_scaled_mm_same_run_tflops", 3230.0), ("fp8_vs_torch_scaled_mm_same_run", 0.99),
                       ("fp8_cpu_baseline_tflops", 1.3), ("cfg_bf16_4096_tflops", 1500.0), ("cfg_bf16_4096_frac", 0.6),
-                      ("cfg_skinny_64_6144_4096_gbs", 3000.0), ("cfg_skinny_64_6144_4096_frac", 0.375)]:
+                      ("cfg_skinny_64_6144_4096_gbs", 3000.0),
+                      ("bf16_8192_8192_16384_tflops", 1550.0), ("bf16_8192_8192_16384_torch_mm_tflops", 1540.0),
+                      ("bf16_8192_8192_16384_vs_torch_mm", 1.0065), ("cfg_skinny_64_6144_4096_frac", 0.375)]:
         assert flat[key] == want, key
     # an MFMA in every cycle at the profiled clock, and the issue share the 0.70 target would need at that clock
     assert flat["full_issue_at_profiled_clock_tflops"] == round(1048.576 * b.PROFILED["bf16_8192"]["shader_clock_ghz"], 1)
-    assert 0.9 < flat["mfma_busy_needed_for_target"] < 1.0
+    # (above 1 when the target is out of reach at that clock whatever the schedule)
+    assert 0.9 < flat["mfma_busy_needed_for_target"] < 1.1
     json.dumps(roof)                                     # everything stays serialisable
     assert all(len(v) <= 120 for v in flat.values() if isinstance(v, str))    # survives a reader that cuts long strings
 
