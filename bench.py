@@ -323,6 +323,63 @@ def calibrate(A, B, do_settle=True, read=True):
     return mfma_entry, read_entry
 
 
+def clock_under_load(sets, C, fp8, variant, flops, ms_hint, do_settle):
+    """The shader clock while this workload's launches run, without a profiler: the library's clock probe (single
+    waves that sleep and sample the cycle counter and the 100 MHz counter) runs on a second stream beside a train of
+    launches long enough to outlast it.  Returns the clock (mean over the probe's waves, and by XCD), the time per
+    launch meanwhile, and whether the probe really ended before the launches did."""
+    import ctypes
+    import torch
+    import gemm_kernels
+    lib = ctypes.CDLL(os.path.join(ROOT, "cute-examples_amd", "gemm_kernels", "libmi355gemm.so"))
+    vp, ci = ctypes.c_void_p, ctypes.c_int
+    lib.mi355_clock_probe_bytes.restype = ctypes.c_size_t
+    lib.mi355_clock_probe_bytes.argtypes = [ci, ci]
+    lib.mi355_clock_probe.argtypes = [ci, ci, ci, vp, vp]
+    A, B = sets[0][:2]
+    if fp8:
+        def call():
+            gemm_kernels.gemm_tn_fp8(A, B, fp8[0], fp8[1], C, variant)
+    else:
+        def call():
+            gemm_kernels.gemm_tn(A, B, C, variant)
+    waves, samples, pause = 32, 100, 8                      # 800 sleeps of 8128 cycles: 2.7 ms at 2.4 GHz, 6.5 ms at 1 GHz
+    launches = int(2 * 6.5 / max(ms_hint, 1e-3)) + 4        # twice the slowest probe
+    out = torch.zeros(lib.mi355_clock_probe_bytes(waves, samples) // 8, dtype=torch.int64, device=A.device)
+    side = torch.cuda.Stream()
+    started, ended, probe_ended = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+    # A stream's hardware queue is set up at its first launch, which disturbs whatever runs then: get that over with.
+    assert lib.mi355_clock_probe(1, 2, 1, out.data_ptr(), side.cuda_stream) == 0
+    torch.cuda.synchronize()
+    settle(call, do_settle)
+    for _ in range(3):
+        call()
+    started.record()
+    for _ in range(launches):
+        call()
+    ended.record()
+    side.wait_event(started)
+    rc = lib.mi355_clock_probe(waves, samples, pause, out.data_ptr(), side.cuda_stream)
+    assert rc == 0, rc
+    probe_ended.record(side)
+    torch.cuda.synchronize()
+    got = out.view(waves, 2, samples + 1).cpu()
+    cycles, ticks = got[:, 0, 1:].double(), got[:, 1, 1:].double()
+    ghz = (cycles[:, -1] - cycles[:, 0]) / (ticks[:, -1] - ticks[:, 0]) / 10.0     # a tick is 10 ns
+    by_xcd = {}
+    for w in range(waves):
+        by_xcd.setdefault(int(got[w, 0, 0]), []).append(float(ghz[w]))
+    by_xcd = {str(k): round(sum(v) / len(v), 3) for k, v in sorted(by_xcd.items())}
+    ms = started.elapsed_time(ended) / launches
+    return {"value": round(float(ghz.mean()), 3), "unit": "GHz", "by_xcd": by_xcd,
+            "min_xcd": min(by_xcd.values()), "max_xcd": max(by_xcd.values()),
+            "ms_per_launch_meanwhile": round(ms, 5), "tflops_meanwhile": round(flops / ms / 1e9, 1),
+            "launches": launches, "probe_ms": round(started.elapsed_time(probe_ended), 3),
+            "probe_inside_launches": started.elapsed_time(probe_ended) < started.elapsed_time(ended),
+            "what": "mi355_clock_probe: %d waves x %d samples of s_memtime (shader cycles) and s_memrealtime (100 MHz) on a "
+                    "second stream beside the launches" % (waves, samples)}
+
+
 def vendor_same_run(sets, C, fp8, flops, steps, warmup, do_settle):
     """The vendor library on the same operands, same protocol (settle, W warm-up, K timed launches):
     torch.mm (hipBLASLt) for the 16-bit types, torch._scaled_mm for e4m3 with per-tensor scales.
@@ -449,6 +506,16 @@ def flatten_into(roof, fp8_block):
         roof["measured_hbm_read_gbs"] = roof["measured_hbm_read"]["value"]
     if roof.get("torch_mm_same_run"):
         roof["torch_mm_same_run_tflops"] = roof["torch_mm_same_run"]["value"]
+    per_ghz = 256 * 4 * (2048 if roof["peak"] > 3000 else 1024) / 1e3     # TFLOP/s per GHz with an MFMA in every cycle
+    clk = roof.get("shader_clock")
+    if clk:
+        # Measured in this run: the clock under this workload, an MFMA in every cycle of every SIMD at that clock, and
+        # the share of that the launches beside the probe reached (= the share of cycles with an MFMA issued).
+        roof["shader_clock_ghz_live"], roof["shader_clock_ghz_live_min_xcd"] = clk["value"], clk["min_xcd"]
+        roof["shader_clock_ghz_live_max_xcd"], roof["shader_clock_probe_inside_launches"] = clk["max_xcd"], clk["probe_inside_launches"]
+        roof["full_issue_at_live_clock_tflops"] = round(per_ghz * clk["value"], 1)
+        roof["tflops_beside_clock_probe"] = clk["tflops_meanwhile"]
+        roof["mfma_issue_share_live"] = round(clk["tflops_meanwhile"] / (per_ghz * clk["value"]), 4)
     prof = roof.get("profiled")
     if prof:
         roof["profiled_mfma_busy"], roof["profiled_shader_clock_ghz"] = prof["mfma_busy"], prof["shader_clock_ghz"]
@@ -456,7 +523,6 @@ def flatten_into(roof, fp8_block):
         # An MFMA in every cycle of every SIMD at the clock the profile shows for this kernel (256 CUs x 4 SIMDs x
         # 1024 flop per cycle for the 16-bit types, twice that for fp8), and the share of cycles the 0.70 / 0.60
         # target of the published peak would therefore need MFMAs to be issued in.
-        per_ghz = 256 * 4 * (2048 if roof["peak"] > 3000 else 1024) / 1e3
         roof["full_issue_at_profiled_clock_tflops"] = round(per_ghz * prof["shader_clock_ghz"], 1)
         target = 0.60 if roof["peak"] > 3000 else 0.70
         roof["mfma_busy_needed_for_target"] = round(target * roof["peak"] / roof["full_issue_at_profiled_clock_tflops"], 3)
@@ -472,6 +538,11 @@ def flatten_into(roof, fp8_block):
         if r8.get("torch_mm_same_run"):
             roof["fp8_torch_scaled_mm_same_run_tflops"] = r8["torch_mm_same_run"]["value"]
             roof["fp8_vs_torch_scaled_mm_same_run"] = r8.get("vs_torch_mm_same_run")
+        if r8.get("shader_clock"):
+            c8k = r8["shader_clock"]
+            roof["fp8_shader_clock_ghz_live"] = c8k["value"]
+            roof["fp8_full_issue_at_live_clock_tflops"] = round(256 * 4 * 2048 / 1e3 * c8k["value"], 1)
+            roof["fp8_mfma_issue_share_live"] = round(c8k["tflops_meanwhile"] / (256 * 4 * 2048 / 1e3 * c8k["value"]), 4)
         if r8.get("profiled"):
             roof["fp8_profiled_mfma_busy"] = r8["profiled"]["mfma_busy"]
             roof["fp8_profiled_shader_clock_ghz"] = r8["profiled"]["shader_clock_ghz"]
@@ -522,6 +593,8 @@ def main():
         roof["torch_mm_same_run"] = vendor_same_run(sets, C, fp8, flops, a.steps, a.warmup, do_settle)
         if roof["torch_mm_same_run"]["value"]:
             roof["vs_torch_mm_same_run"] = round(head["tflops"] / roof["torch_mm_same_run"]["value"], 4)
+    if roof["bound"] == "mfma" and not a.no_calibrate:
+        roof["shader_clock"] = clock_under_load(sets, C, fp8, a.variant, flops, head["ms"], do_settle)
     if a.workload in PROFILED:
         roof["profiled"] = PROFILED[a.workload]
 
@@ -543,6 +616,8 @@ def main():
             roof8["torch_mm_same_run"] = vendor_same_run(sets8, C8, sc8, flops8, a.steps, a.warmup, do_settle)
             if roof8["torch_mm_same_run"]["value"]:
                 roof8["vs_torch_mm_same_run"] = round(row["tflops"] / roof8["torch_mm_same_run"]["value"], 4)
+        if not a.no_calibrate:
+            roof8["shader_clock"] = clock_under_load(sets8, C8, sc8, a.variant, flops8, row["ms"], do_settle)
         roof8["profiled"] = PROFILED["fp8_8192"]
         fp8_block = {"value": row["tflops"], "unit": "TFLOP/s", "ms_per_step": row["ms"], "steps": a.steps,
                      "warmup": a.warmup, "settle_launches": row["settle_launches"], "settle_ms": row["settle_ms"],

@@ -13,6 +13,10 @@
 //                  blocks: the same 128 x 128 outputs per wave), so that a benchmark can show what
 //                  the choice of shape is worth on the GPU and the data at hand.
 //   read_ceiling   16-byte loads, grid-stride over the buffer, xor-reduced so nothing is elided.
+//   clock_probe    single-wave workgroups that sleep and, every so often, read the shader-cycle counter
+//                  and the constant 100 MHz counter: launched on a second stream beside other work
+//                  (a wave of it needs 8 registers and no LDS, so it fits beside a workgroup of the
+//                  tile kernels), it tells the shader clock that work runs at without a profiler.
 //
 // Counterpart in the reference: none (its benchmark takes the peak from a table,
 // kernels/tests/gemm_bench.py:592-599).
@@ -93,6 +97,34 @@ __global__ __launch_bounds__(256) void read_ceiling(const u32x4* src, size_t chu
   sink[(size_t)blockIdx.x * 256 + threadIdx.x] = x[0] ^ x[1] ^ x[2] ^ x[3];
 }
 
+// out[w][0][0] = XCD of wave w, out[w][1][0] = 0; out[w][0][1 + s] = shader cycles and out[w][1][1 + s] = 10 ns ticks
+// at sample s (uint64 out[waves][2][samples + 1]).  s_memtime counts shader cycles on this GPU (a chain of
+// dependent MFMAs reads the same difference whatever the clock), s_memrealtime counts at 100 MHz.  Every loop is
+// bounded by the arguments.
+__global__ __launch_bounds__(64) void clock_probe(uint64_t* out, int samples, int pause) {
+  uint32_t xcc;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+  // One lane writes, in 4-byte pieces: nothing here is worth the care wider stores' data registers need.
+  volatile uint32_t* cycles_of = (volatile uint32_t*)(out + (size_t)blockIdx.x * 2 * (size_t)(samples + 1));
+  volatile uint32_t* ticks_of = cycles_of + 2 * (size_t)(samples + 1);
+  auto put = [](volatile uint32_t* at, uint64_t x) __attribute__((always_inline)) {
+    at[0] = (uint32_t)x;
+    at[1] = (uint32_t)(x >> 32);
+  };
+  if (threadIdx.x == 0) {
+    put(cycles_of, xcc & 15u);
+    put(ticks_of, 0);
+  }
+  for (int s = 0; s < samples; ++s) {
+    const uint64_t cycles = __builtin_readcyclecounter(), ticks = __builtin_amdgcn_s_memrealtime();
+    if (threadIdx.x == 0) {
+      put(cycles_of + 2 * (size_t)(1 + s), cycles);
+      put(ticks_of + 2 * (size_t)(1 + s), ticks);
+    }
+    for (int p = 0; p < pause; ++p) __builtin_amdgcn_s_sleep(127);
+  }
+}
+
 }  // namespace
 }  // namespace mi355
 
@@ -145,6 +177,21 @@ int mi355_calibrate_read(const void* src, size_t bytes, void* sink, void* stream
   const unsigned blocks = (unsigned)(cus * 16 < 4096 ? cus * 16 : 4096);
   hipLaunchKernelGGL(read_ceiling, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const u32x4*)src, bytes / 16,
                      (uint32_t*)sink);
+  return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ERR_LAUNCH;
+}
+
+size_t mi355_clock_probe_bytes(int waves, int samples) {
+  if (waves < 1 || waves > 1024 || samples < 2 || samples > 4096) return 0;
+  return (size_t)waves * (size_t)(samples + 1) * 2 * sizeof(uint64_t);
+}
+
+int mi355_clock_probe(int waves, int samples, int pause, void* out, void* stream) {
+  using namespace mi355;
+  if (!out) return MI355_ERR_NULL;
+  // at most 65536 sleeps of 127 x 64 cycles per wave: a quarter of a second at 2 GHz
+  if (mi355_clock_probe_bytes(waves, samples) == 0 || pause < 1 || (int64_t)samples * pause > 65536) return MI355_ERR_SHAPE;
+  if ((uintptr_t)out % 8 != 0) return MI355_ERR_ALIGN;
+  hipLaunchKernelGGL(clock_probe, dim3((unsigned)waves), dim3(64), 0, (hipStream_t)stream, (uint64_t*)out, samples, pause);
   return hipGetLastError() == hipSuccess ? MI355_OK : MI355_ERR_LAUNCH;
 }
 

@@ -282,6 +282,23 @@ int mi355_calibrate_mfma_shape(int in_dtype, int wide_blocks, const void *a, siz
                                void *stream);
 int mi355_calibrate_read(const void *src, size_t bytes, void *sink, void *stream);
 
+/*
+ * Shader clock under load, without a profiler.  No counterpart in the reference.
+ * mi355_clock_probe enqueues ONE launch of `waves` single-wave workgroups (1..1024) that do nothing
+ * but sleep and, `samples` times (2..4096) with `pause` sleeps of 127 x 64 cycles in between
+ * (samples * pause <= 65536), read the shader-cycle counter and the constant 100 MHz counter.
+ * Enqueued on a second stream while other work runs on the first (a wave of it needs 8 registers and
+ * no LDS, so it finds room beside the tile kernels' workgroups), it yields the clock that work runs at.
+ * (A stream's hardware queue is set up at its first launch, which disturbs whatever runs at that
+ * moment: launch something small on the second stream once before the measurement.)
+ * `out` is device memory of mi355_clock_probe_bytes(waves, samples) bytes, 8-byte aligned, read as
+ * uint64 out[waves][2][samples + 1]: out[w][0][0] = XCD the wave ran on, out[w][1][0] = 0,
+ * out[w][0][1 + s] = shader cycles and out[w][1][1 + s] = ticks of 10 ns at sample s; the clock
+ * between two samples is the ratio of the differences.  mi355_clock_probe_bytes returns 0 for counts outside the ranges above.
+ */
+size_t mi355_clock_probe_bytes(int waves, int samples);
+int mi355_clock_probe(int waves, int samples, int pause, void *out, void *stream);
+
 /* Human-readable text for a status code; never NULL.  Replaces the TORCH_CHECK messages of
  * gemm_test.cu:15-41 and the stderr print of :88-90. */
 const char *mi355_gemm_strerror(int status);

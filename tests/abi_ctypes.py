@@ -66,6 +66,10 @@ def load():
     L.mi355_calibrate_mfma_shape.restype = ci
     L.mi355_calibrate_read.argtypes = [vp, sz, vp, vp]
     L.mi355_calibrate_read.restype = ci
+    L.mi355_clock_probe_bytes.argtypes = [ci, ci]
+    L.mi355_clock_probe_bytes.restype = sz
+    L.mi355_clock_probe.argtypes = [ci, ci, ci, vp, vp]
+    L.mi355_clock_probe.restype = ci
     L.mi355_gemm_strerror.argtypes = [ci]
     L.mi355_gemm_strerror.restype = ctypes.c_char_p
     L.mi355_gemm_version.argtypes = []

@@ -77,3 +77,43 @@ def test_calibration_kernels_run_and_report_plausible_ceilings(abi):
         torch.cuda.synchronize()
     gbs = src.numel() / e0.elapsed_time(e1) / 1e6
     assert 1000.0 < gbs, gbs
+
+
+def test_clock_probe_reads_a_plausible_shader_clock_beside_a_gemm(abi):
+    """mi355_clock_probe on a second stream while GEMMs run on the first: every wave's cycle and 10 ns counters
+    rise from sample to sample, the clock they give lies between 0.5 and 2.6 GHz, the waves report XCDs 0..7,
+    and the GEMM's result is what it is without the probe.  Argument errors come back before any launch."""
+    import torch
+    from tests import abi_ctypes as ac
+    import gemm_kernels
+
+    assert abi.mi355_clock_probe_bytes(0, 10) == 0 and abi.mi355_clock_probe_bytes(8, 1) == 0
+    assert abi.mi355_clock_probe_bytes(8, 4097) == 0 and abi.mi355_clock_probe_bytes(1025, 10) == 0
+    waves, samples, pause = 16, 40, 4
+    assert abi.mi355_clock_probe_bytes(waves, samples) == waves * (samples + 1) * 16
+    out = torch.zeros((waves, 2, samples + 1), dtype=torch.int64, device="cuda")
+    assert abi.mi355_clock_probe(waves, samples, pause, None, None) == ac.ERR_NULL
+    assert abi.mi355_clock_probe(waves, samples, 0, out.data_ptr(), None) == ac.ERR_SHAPE
+    assert abi.mi355_clock_probe(waves, 4096, 17, out.data_ptr(), None) == ac.ERR_SHAPE
+    assert abi.mi355_clock_probe(waves, samples, pause, out.data_ptr() + 4, None) == ac.ERR_ALIGN
+    A = torch.randn(4096, 4096, device="cuda").to(torch.bfloat16)
+    B = torch.randn(4096, 4096, device="cuda").to(torch.bfloat16)
+    alone = gemm_kernels.gemm_tn(A, B, torch.empty(4096, 4096, dtype=torch.bfloat16, device="cuda"))
+    torch.cuda.synchronize()
+    C = torch.empty_like(alone)
+    side = torch.cuda.Stream()
+    started = torch.cuda.Event()
+    gemm_kernels.gemm_tn(A, B, C)
+    started.record()
+    for _ in range(12):
+        gemm_kernels.gemm_tn(A, B, C)
+    side.wait_event(started)
+    assert abi.mi355_clock_probe(waves, samples, pause, out.data_ptr(), side.cuda_stream) == ac.OK
+    torch.cuda.synchronize()
+    assert torch.equal(C, alone)
+    got = out.cpu()
+    assert set(got[:, 0, 0].tolist()) <= set(range(8)) and (got[:, 1, 0] == 0).all()
+    cycles, ticks = got[:, 0, 1:], got[:, 1, 1:]
+    assert (cycles[:, 1:] > cycles[:, :-1]).all() and (ticks[:, 1:] > ticks[:, :-1]).all()
+    ghz = (cycles[:, -1] - cycles[:, 0]).double() / (ticks[:, -1] - ticks[:, 0]).double() / 10.0
+    assert (ghz > 0.5).all() and (ghz < 2.6).all(), ghz

@@ -44,6 +44,7 @@ def test_roofline_carries_every_yardstick_as_a_scalar_field():
     roof = {"bound": "mfma", "peak": 2500.0,
             "measured_mfma_ceiling": {"value": 2000.0, "value_zero_operands": 2400.0, "by_shape": {"16x16x32": 2000.0, "32x32x16": 1800.0}},
             "measured_hbm_read": {"value": 6800.0}, "torch_mm_same_run": {"value": 1660.0}, "profiled": b.PROFILED["bf16_8192"],
+            "shader_clock": {"value": 1.7, "min_xcd": 1.66, "max_xcd": 1.73, "probe_inside_launches": True, "tflops_meanwhile": 1600.0},
             "larger_shapes": {"8192_8192_16384": {"ms": 1.42, "tflops": 1550.0, "frac": 0.62, "torch_mm_tflops": 1540.0, "vs_torch_mm": 1.0065}},
             "other_configs": b.other_configs([row("bf16_4096", 0.09, 1500.0, 1.0), row("skinny_64_6144_4096", 0.017, 1.0, 3000.0)],
                                              {"value": 2000.0}, {"value": 6800.0})}
@@ -61,6 +62,8 @@ def test_roofline_carries_every_yardstick_as_a_scalar_field():
                       ("fp8_torch_scaled_mm_same_run_tflops", 3230.0), ("fp8_vs_torch_scaled_mm_same_run", 0.99),
                       ("fp8_cpu_baseline_tflops", 1.3), ("cfg_bf16_4096_tflops", 1500.0), ("cfg_bf16_4096_frac", 0.6),
                       ("cfg_skinny_64_6144_4096_gbs", 3000.0),
+                      ("shader_clock_ghz_live", 1.7), ("shader_clock_ghz_live_min_xcd", 1.66), ("shader_clock_probe_inside_launches", True),
+                      ("full_issue_at_live_clock_tflops", round(1048.576 * 1.7, 1)), ("mfma_issue_share_live", round(1600.0 / (1048.576 * 1.7), 4)),
                       ("bf16_8192_8192_16384_tflops", 1550.0), ("bf16_8192_8192_16384_torch_mm_tflops", 1540.0),
                       ("bf16_8192_8192_16384_vs_torch_mm", 1.0065), ("cfg_skinny_64_6144_4096_frac", 0.375)]:
         assert flat[key] == want, key
