@@ -70,6 +70,16 @@ bool auto_alternates(int64_t M, int64_t N, int64_t K, int in_dtype) {
   const int64_t k_steps = (K * 2 + 127) / 128, tiles = ((M + 255) / 256) * ((N + 127) / 128);
   return k_steps >= 1 && k_steps <= 4 && tiles >= 1024;
 }
+// Whether the tile kernels write C with non-temporal stores (nt sc1) or keep it in the caches on its way out (sc1).
+// Kept when the output (16-bit) is at most 192 MiB and operands and output together at most 288 MiB, a little more
+// than the 256 MB Infinity Cache.  Measured, kept against streamed: fp8 8192^3 2-3 % faster, 8192^2 x 1024..2048 6 %,
+// bf16 8192^2 x 4096 1.6 %, the two-workgroup kernel at K <= 256 with outputs up to 192 MiB 9-16 %; bf16 8192^3
+// (384 MiB in all) 0-0.9 % slower, outputs of 256 MiB and more 0.6-5.7 % slower (that kernel: 22-34 %).
+int32_t c_streams(int64_t M, int64_t N, int64_t K, int elem_bytes) {
+  const double mib = 1024.0 * 1024.0, out = (double)M * (double)N * 2.0;
+  const double total = ((double)M + (double)N) * (double)K * elem_bytes + out;
+  return out <= 192.0 * mib && total <= 288.0 * mib ? 0 : 1;
+}
 bool skinny_ok(int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int in_dtype) {
   if (M > 256) return false;
   return tile256_ok(M, N, K, lda, ldb, ldc, in_dtype);
@@ -385,6 +395,7 @@ int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, in
   g.tail_splits = 1;
   g.scale_a = g.scale_b = nullptr;
   g.mx_a = g.mx_b = nullptr;
+  g.c_streams = c_streams(M, N, K, 1);
   if (K == 0) {  // an empty sum: zeros, written by the generic kernel
     g.tiles_m = g.tiles_n = 0;
     return mi355::launch_simple(g, MI355_E4M3, out_dtype, s) == 0 ? MI355_OK : MI355_ERR_LAUNCH;
@@ -491,6 +502,7 @@ int run_gemm(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_
   g.scale_a = scale_a;
   g.scale_b = scale_b;
   g.mx_a = g.mx_b = nullptr;
+  g.c_streams = c_streams(M, N, K, in_dtype == MI355_E4M3 ? 1 : 2);
   hipStream_t s = (hipStream_t)stream;
 
   if (v == MI355_VARIANT_BASIC || v == MI355_VARIANT_PINGPONG || v == MI355_VARIANT_SKINNY || v == MI355_VARIANT_ALTERNATE) {

@@ -28,6 +28,9 @@ struct GemmArgs {
   // kernel that writes C, so that per-tensor fp8 scales never have to visit the host.
   const float* scale_a;
   const float* scale_b;
+  // Non-zero when operands and output together exceed what the Infinity Cache holds: the tile kernels then write C
+  // with non-temporal stores (tile_store.h).
+  int32_t c_streams;
   // Block scales (MX) of A and of B in the shuffled layout, or null.
   const uint8_t* mx_a;
   const uint8_t* mx_b;

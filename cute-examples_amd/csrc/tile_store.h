@@ -40,11 +40,12 @@ __device__ __forceinline__ void store_output_tile(typename G::Acc (&acc)[kNbM][k
                                                   uint32_t wave_row, uint32_t wave_col, uint32_t lane, float scale) {
   typedef typename G::Acc Acc;
   constexpr int kBlk = G::kBlk;
-  // Non-temporal, write-through stores (nt + sc1) keep C out of L2: it is written once and would
-  // evict operand panels.  They only pay when a store instruction covers at least 64 contiguous
-  // bytes per row, which the 16-wide blocks do (two blocks side by side) and the 32-wide blocks do
-  // not (32 bytes: measured 3 % slower with sc1, 25 % with nt + sc1).
-  constexpr int kAux = kBlk == 16 ? 18 : 0;
+  // Cache policy of the stores.  Write-through (sc1) always: C is written once and read by nobody here.  Non-temporal
+  // on top of that (nt + sc1) when the host finds the output too large to pass through the Infinity Cache beside the
+  // operands (g.c_streams): then it would push operand panels out (16384^2 x 4096: 2-6 % faster with nt), while a
+  // smaller C is written faster without nt (8192^2 x 1024..2048: 6 %, fp8 8192^3: 2-3 %).  Either only pays when a
+  // store instruction covers at least 64 contiguous bytes per row, which the 16-wide blocks do (two blocks side by
+  // side) and the 32-wide blocks do not (32 bytes: measured 3 % slower with sc1, 25 % with nt + sc1).
   const uint32_t rblk = lane & (kBlk - 1), grp = lane / kBlk;
   const int64_t rows = g.M - m0 < tile_rows ? g.M - m0 : tile_rows;
   const uint32_t cols = (uint32_t)(g.N - n0 < tile_cols ? g.N - n0 : tile_cols);
@@ -57,8 +58,9 @@ __device__ __forceinline__ void store_output_tile(typename G::Acc (&acc)[kNbM][k
   const uint32_t v0 = (wave_row + rblk) * ldc_b + col0 * 2;
   const uint32_t block_step = __builtin_amdgcn_readfirstlane(kBlk * ldc_b);
 
+  float factor = scale;
   auto pack_quad = [&](const Acc& a, int q) __attribute__((always_inline)) -> u32x2 {
-    return Pack4<OutT>::run(a[4 * q] * scale, a[4 * q + 1] * scale, a[4 * q + 2] * scale, a[4 * q + 3] * scale);
+    return Pack4<OutT>::run(a[4 * q] * factor, a[4 * q + 1] * factor, a[4 * q + 2] * factor, a[4 * q + 3] * factor);
   };
   // emit(i, col, x, y): x = the lane's first four outputs, y = the last four, `col` columns right of
   // col0 in row block i (both compile-time values).
@@ -95,17 +97,28 @@ __device__ __forceinline__ void store_output_tile(typename G::Acc (&acc)[kNbM][k
     });
   };
   if (cols == (uint32_t)tile_cols) {
-    u32x4 previous = {0u, 0u, 0u, 0u}, before = {0u, 0u, 0u, 0u};
-    convert([&](auto ic, auto colc, u32x2 x, u32x2 y) __attribute__((always_inline)) {
-      constexpr int i = decltype(ic)::value, col = decltype(colc)::value;
-      u32x4 data = {x[0], x[1], y[0], y[1]};
-      hold_previous(data, previous, before);
-      __builtin_amdgcn_raw_buffer_store_b128(data, rc, v0 + col * 2, i * block_step, kAux);
-      MI355_FENCE();   // the next block's conversion stays behind this store
-      before = previous;
-      previous = data;
-    });
-    hold_last(previous);
+    auto whole_rows = [&](auto auxc) __attribute__((always_inline)) {
+      // The two forms of this phase differ in one bit of their stores.  Each takes the scale through a statement of
+      // its own, so that the compiler cannot lift the first conversions, which would otherwise be the same in both,
+      // in front of the choice between them: the distance between a store and the next write of its data registers
+      // rests on every conversion standing between the stores of its own form.
+      if constexpr (decltype(auxc)::value == 18) asm volatile("; C streamed" : "+v"(factor));
+      else asm volatile("; C kept" : "+v"(factor));
+      u32x4 previous = {0u, 0u, 0u, 0u}, before = {0u, 0u, 0u, 0u};
+      convert([&](auto ic, auto colc, u32x2 x, u32x2 y) __attribute__((always_inline)) {
+        constexpr int i = decltype(ic)::value, col = decltype(colc)::value;
+        u32x4 data = {x[0], x[1], y[0], y[1]};
+        hold_previous(data, previous, before);
+        __builtin_amdgcn_raw_buffer_store_b128(data, rc, v0 + col * 2, i * block_step, decltype(auxc)::value);
+        MI355_FENCE();   // the next block's conversion stays behind this store
+        before = previous;
+        previous = data;
+      });
+      hold_last(previous);
+    };
+    if constexpr (kBlk != 16) whole_rows(std::integral_constant<int, 0>{});
+    else if (g.c_streams) whole_rows(std::integral_constant<int, 18>{});
+    else whole_rows(std::integral_constant<int, 16>{});
   } else {
     // N is a multiple of 4 (host check), so each half of the 8 columns is in or out as a whole.
     u32x4 previous = {0u, 0u, 0u, 0u}, before = {0u, 0u, 0u, 0u};
