@@ -88,6 +88,16 @@ struct SmallTileCost {
   double pair, pair_slack, single, single_busy, few_rows, fixed, reduce_mb, reduce;
 };
 constexpr SmallTileCost kCost128 = {0.990, 0.498, 0.244, 0.352, 0.519, 5.53, 0.101, 1.71};
+// Tiles of fewer than 16 k-steps, which none of the problems above had (and which are never split): the k-step part of
+// the estimate scaled by k_part, and fixed costs per round and per launch in place of `fixed`.  Weighted least squares
+// over 330 bf16 and e4m3 problems of 1...14 k-steps, M, N = 512...16384 (residuals 4-9 % rms).  On 140 further problems
+// the shortest estimate costs 0.7 % of the best tile's time on average and more than 5 % on 4 of them, against 1.7 %
+// and 16 for the coefficients above with the 10 % preference for larger tiles they needed there.
+struct ShortTileCost {
+  double k_part, per_round, per_launch;
+};
+constexpr ShortTileCost kShort256 = {0.889, 5.38, 3.46}, kShort256x128 = {0.775, 3.38, 2.39}, kShort128 = {0.762, 3.36, 0.61};
+constexpr int64_t kShortSteps = 16;
 
 // k_loop_factor scales the k-step part of the small tile's estimate (not the fixed and reduction parts): see ring_tile_edge.
 double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes, double k_loop_factor = 1.0) {
@@ -108,6 +118,7 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes, do
     const double step_sum = c.pair * pair_rounds - c.pair_slack * slack +
                             (single ? c.single + c.single_busy * (double)rest / (double)kCuSlots : 0.0) +
                             c.few_rows * rounds / (double)tm;
+    if (steps < kShortSteps) return kShort128.k_part * item_steps * step_sum + kShort128.per_round * rounds + kShort128.per_launch;
     return k_loop_factor * item_steps * step_sum + c.fixed * rounds + (partial_mb > 0.0 ? c.reduce_mb * partial_mb + c.reduce : 0.0);
   }
   const TileCost& c = tile == 256 ? kCost256 : kCost256x128;
@@ -123,6 +134,10 @@ double estimate_us(int tile, int64_t M, int64_t N, int64_t K, int elem_bytes, do
     }
   }
   const double step_us = c.step + c.step_busy * occupancy + c.few_rows / (double)tm + c.few_cols / (double)tn;
+  if (steps < kShortSteps) {
+    const ShortTileCost& k = tile == 256 ? kShort256 : kShort256x128;
+    return k.k_part * rounds * item_steps * step_us + k.per_round * rounds + k.per_launch;
+  }
   return rounds * (item_steps * step_us + c.fixed) + (partial_mb > 0.0 ? c.reduce_mb * partial_mb + c.reduce : 0.0);
 }
 
@@ -194,10 +209,7 @@ int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_s
   // 256 x 128 tiles, 28.1 us against 29.5).
   const double e128 = estimate_us(128, M, N, K, elem_bytes, single_round ? 0.82 : 1.0);
   const double e2 = estimate_us(kRingTile256x128, M, N, K, elem_bytes);
-  // Under 16 k-steps, fewer than any fitted problem had, the estimates of the small tiles run low (e4m3,
-  // 14 k-steps, 1264 x 3240 and 11664 x 328: 128 x 128 tiles estimated 2 % ahead of 256 x 128, measured 8 and 15 %
-  // behind): a larger tile is preferred within 10 % there.
-  const double margin = k_steps_of(K, elem_bytes) < 16 ? 1.10 : 1.02;
+  const double margin = 1.02;
   const double best = margin * (e256 < e128 ? (e256 < e2 ? e256 : e2) : (e128 < e2 ? e128 : e2));
   return e256 <= best ? 256 : e2 <= best ? kRingTile256x128 : single_round ? kRingTile128DeepPlain : 128;
 }
