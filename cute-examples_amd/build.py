@@ -4,7 +4,9 @@
     python cute-examples_amd/build.py --lib-only  # libmi355gemm.so only (no torch headers needed)
 
 Outputs land in cute-examples_amd/gemm_kernels/: libmi355gemm.so (the C ABI of
-include/mi355_gemm.h) and _C.<abi>.so (the torch binding, linked against it via $ORIGIN).
+include/mi355_gemm.h), _C.<abi>.so (the torch binding, linked against it via $ORIGIN) and
+libmi355gemm_syncscales.so, the same library with the block-scaled kernel in its fallback form
+(MI355_MX_SYNC_SCALES), which the GPU tests run beside the default one.
 Counterpart in the reference: kernels/setup.py:8-28 + build.sh:1-7.
 """
 import os
@@ -16,6 +18,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "gemm_kernels")
 LIB = os.path.join(OUT, "libmi355gemm.so")
+LIB_SYNC_SCALES = os.path.join(OUT, "libmi355gemm_syncscales.so")
 
 HIP_SOURCES = ["gemm_api.hip", "gemm_tn_simple.hip", "gemm_tn_ring_bf16.hip", "gemm_tn_ring_f16.hip", "gemm_tn_ring_e4m3.hip", "gemm_tn_ring_mx.hip", "ring_plan.hip", "gemm_tn_pingpong.hip", "gemm_tn_alternate.hip", "gemm_tn_stream.hip", "quantize_e4m3.hip", "mx_scales.hip", "calibrate.hip"]
 
@@ -57,8 +60,9 @@ def build_lib():
 
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     with tempfile.TemporaryDirectory() as tmp:
-        def compile_one(src, defines=()):
-            obj = os.path.join(tmp, src.replace(".hip", ".o"))
+        def compile_one(src, defines=(), subdir=""):
+            os.makedirs(os.path.join(tmp, subdir), exist_ok=True)
+            obj = os.path.join(tmp, subdir, src.replace(".hip", ".o"))
             extra = ["-save-temps=obj"] if src in HAZARD_SOURCES else []
             _run([hipcc] + HIPCC_FLAGS + ["-c"] + extra + list(defines) + ["-o", obj, os.path.join(CSRC, src)])
             return obj
@@ -69,8 +73,11 @@ def build_lib():
         # themselves instead: slower, no assumption.
         sync_scales = ["-DMI355_MX_SYNC_SCALES"] if os.environ.get("MI355_MX_SYNC_SCALES") == "1" else []
 
-        with ThreadPoolExecutor(max_workers=min(len(HIP_SOURCES), os.cpu_count() or 1)) as pool:
+        with ThreadPoolExecutor(max_workers=min(len(HIP_SOURCES) + 1, os.cpu_count() or 1)) as pool:
+            # the fallback form of the block-scaled kernel, for the second library, beside everything else
+            fallback = pool.submit(compile_one, CHECKED_SOURCE, ["-DMI355_MX_SYNC_SCALES"], "sync_scales")
             objs = list(pool.map(lambda src: compile_one(src, sync_scales if src == CHECKED_SOURCE else ()), HIP_SOURCES))
+            fallback_obj = fallback.result()
         copies = 0
         for src in CHECKED_SOURCES:
             asm = glob.glob(os.path.join(tmp, src.replace(".hip", "") + "-hip-amdgcn-*gfx950.s"))
@@ -100,6 +107,15 @@ def build_lib():
               "results untouched for %d" % (stores, check_async_loads.STORE_DATA_WINDOW, mfmas,
                                              check_async_loads.MFMA_RESULT_WINDOW), flush=True)
         _run([hipcc] + HIPCC_FLAGS + ["-o", LIB] + objs)
+        # The same library around the fallback form of the block-scaled kernel, held to the same distances.
+        asm = glob.glob(os.path.join(tmp, "sync_scales", CHECKED_SOURCE.replace(".hip", "") + "-hip-amdgcn-*gfx950.s"))
+        if len(asm) != 1:
+            raise RuntimeError("expected one device assembly file for the fallback build, found %r" % (asm,))
+        check_async_loads.check_lds_base(asm[0])
+        check_async_loads.check_hazard_distances(asm[0])
+        check_async_loads.check_no_scratch(asm[0])
+        main_obj = os.path.join(tmp, CHECKED_SOURCE.replace(".hip", ".o"))
+        _run([hipcc] + HIPCC_FLAGS + ["-o", LIB_SYNC_SCALES] + [fallback_obj if o == main_obj else o for o in objs])
     return LIB
 
 

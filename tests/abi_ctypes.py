@@ -6,6 +6,7 @@ import re
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB = os.path.join(ROOT, "cute-examples_amd", "gemm_kernels", "libmi355gemm.so")
+LIB_SYNC_SCALES = os.path.join(ROOT, "cute-examples_amd", "gemm_kernels", "libmi355gemm_syncscales.so")
 HEADER = os.path.join(ROOT, "include", "mi355_gemm.h")
 
 BF16, F16, E4M3, F32 = 0, 1, 2, 3
@@ -21,10 +22,10 @@ def declared_symbols():
     return sorted(set(re.findall(r"\b(mi355_[a-z0-9_]+)\s*\(", text)))
 
 
-def load():
-    if not os.path.exists(LIB):
-        raise RuntimeError("libmi355gemm.so is not built; run python cute-examples_amd/build.py")
-    L = ctypes.CDLL(LIB)
+def load(path=LIB):
+    if not os.path.exists(path):
+        raise RuntimeError(os.path.basename(path) + " is not built; run python cute-examples_amd/build.py")
+    L = ctypes.CDLL(path)
     i64, vp, ci, f32, sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_size_t
     L.mi355_gemm_tn.argtypes = [vp, vp, vp, i64, i64, i64, i64, i64, i64, ci, ci, f32, ci, vp, sz, vp]
     L.mi355_gemm_tn.restype = ci

@@ -20,6 +20,15 @@ def test_exports_every_declared_symbol(abi):
         assert f" T {n}" in dyn, n
 
 
+def test_fallback_library_loads_and_exports_the_same_symbols():
+    """The second library of the build (the block-scaled kernel in its fallback form) is a full library."""
+    fallback = ac.load(ac.LIB_SYNC_SCALES)
+    dyn = subprocess.run(["nm", "-D", "--defined-only", ac.LIB_SYNC_SCALES], capture_output=True, text=True).stdout
+    for n in ac.declared_symbols():
+        assert hasattr(fallback, n) and f" T {n}" in dyn, n
+    assert fallback.mi355_gemm_mx_check(256, 256, 128, 128, 128, 256, ac.BF16) == ac.OK
+
+
 def test_version_and_strerror(abi):
     assert abi.mi355_gemm_version() >= 1
     for code in range(0, -8, -1):

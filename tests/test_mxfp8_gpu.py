@@ -403,3 +403,22 @@ def test_few_rows_without_room_for_the_k_split_fall_back_to_the_tile_kernel(abi)
     torch.cuda.synchronize()
     err, _ = check(C.cpu(), A, sa, B, sb)
     assert err < 5e-3
+
+
+@pytest.mark.parametrize("shuffled", [False, True])
+@pytest.mark.parametrize("shape", [(256, 256, 1024), (512, 768, 640), (257, 1020, 384), (768, 768, 8192), (4096, 6144, 4096),
+                                   (2048, 2048, 2048), (512, 6144, 4096), (33, 6144, 4096)])
+def test_fallback_build_of_the_block_scaled_kernel_gives_the_same_bits(abi, shape, shuffled):
+    """libmi355gemm_syncscales.so is the library with the block-scaled tile kernel built in its fallback form (scale
+    loads that wait for themselves, what the build switches to when the compiler copies the registers of the
+    asynchronous ones).  Same arithmetic in the same order: its results must pass the oracle check and equal the default
+    build's bit for bit, on every tile shape, with K and tail splits, ragged edges and few rows."""
+    fallback = ac.load(ac.LIB_SYNC_SCALES)
+    M, N, K = shape
+    A, sa = random_mx(M, K, 61)
+    B, sb = random_mx(N, K, 62)
+    want = run_mx(abi, A, sa, B, sb, shuffled=shuffled)
+    got = run_mx(fallback, A, sa, B, sb, shuffled=shuffled)
+    if M * N * K <= 768 * 768 * 8192:
+        check(got, A, sa, B, sb)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
