@@ -43,9 +43,9 @@ PEAK_HBM_GBS = 8000.0
 # HBM-side bytes per launch of the dominant kernel, from two rocprofv3 --pmc runs of this script
 # (FETCH_SIZE, then WRITE_SIZE, each with --copy-calibration and scaled by what the same counter
 # reads for the 1 GiB copy: x2.000 and x1.000).  Workloads without a counter run report null.
-MEASURED_TRAFFIC_BYTES = {"bf16_8192": 1.750e9, "fp8_8192": 0.943e9, "mxfp8_8192": 0.965e9, "bf16_4096": 2.352e8,
+MEASURED_TRAFFIC_BYTES = {"bf16_8192": 1.747e9, "fp8_8192": 0.941e9, "mxfp8_8192": 0.975e9, "bf16_4096": 2.354e8,
                           "skinny_16_14336_4096": 1.190e8, "skinny_64_14336_4096": 1.236e8, "skinny_64_4096_14336": 1.527e8,
-                          "skinny_256_14336_4096": 1.561e8, "skinny_256_6144_4096": 1.209e8, "skinny_128_8192_4096": 1.130e8}
+                          "skinny_256_14336_4096": 1.560e8, "skinny_256_6144_4096": 1.209e8, "skinny_128_8192_4096": 1.131e8}
 TRAFFIC_PROFILE = {"bf16_8192": "profiles/gemm_tn_tile_ring__bf16_8192.md", "fp8_8192": "profiles/gemm_tn_tile_ring__fp8_8192.md",
                    "mxfp8_8192": "profiles/gemm_tn_tile_ring__mxfp8_8192.md", "bf16_4096": "profiles/gemm_tn_tile_ring__bf16_4096.md",
                    "skinny_16_14336_4096": "profiles/gemm_tn_stream__skinny_16_14336_4096.md",
@@ -59,9 +59,9 @@ SETTLE_MIN_MS, SETTLE_MAX_MS, SETTLE_BATCH_MS = 150.0, 2000.0, 10.0
 # run): the share of SIMD cycles with an MFMA in flight and the shader clock during the kernel
 # (busy CU cycles / CUs / traced duration).
 PROFILED = {
-    "bf16_8192": {"mfma_busy": 0.903, "shader_clock_ghz": 1.66, "lds_bank_conflict_cycles": 0,
+    "bf16_8192": {"mfma_busy": 0.906, "shader_clock_ghz": 1.71, "lds_bank_conflict_cycles": 0,
                   "source": "profiles/gemm_tn_tile_ring__bf16_8192.md"},
-    "fp8_8192": {"mfma_busy": 0.875, "shader_clock_ghz": 1.71, "lds_bank_conflict_cycles": 0,
+    "fp8_8192": {"mfma_busy": 0.870, "shader_clock_ghz": 1.78, "lds_bank_conflict_cycles": 0,
                  "source": "profiles/gemm_tn_tile_ring__fp8_8192.md"},
 }
 
