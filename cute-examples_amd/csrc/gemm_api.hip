@@ -263,11 +263,17 @@ int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant, 
     rows = 256;
     cols = 128;
   } else if (v == MI355_VARIANT_BASIC) {
-    const int tile = mi355::ring_tile_edge(M, N, K, es);
+    int64_t pm = M, pn = N;   // of two launches (mi355_gemm_pieces) the first one's plan
+    if (variant == MI355_VARIANT_AUTO) {
+      bool along_m = false;
+      const int64_t first = mi355::ring_first_piece(M, N, K, es, &along_m);
+      if (first > 0) (along_m ? pm : pn) = first;
+    }
+    const int tile = mi355::ring_tile_edge(pm, pn, K, es);
     rows = mi355::ring_tile_rows(tile);
     cols = mi355::ring_tile_cols(tile);
-    splits = mi355::ring_splits(M, N, K, es);
-    if (splits == 1) mi355::ring_tail(M, N, K, es, &tt, &ts);
+    splits = mi355::ring_splits(pm, pn, K, es);
+    if (splits == 1) mi355::ring_tail(pm, pn, K, es, &tt, &ts);
   }
   if (tile_rows) *tile_rows = rows;
   if (tile_cols) *tile_cols = cols;
@@ -275,6 +281,20 @@ int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant, 
   if (tail_tiles) *tail_tiles = tt;
   if (tail_splits) *tail_splits = ts;
   return v;
+}
+
+int mi355_gemm_pieces(int64_t M, int64_t N, int64_t K, int in_dtype, int variant, int64_t* first_rows, int64_t* first_cols) {
+  if (first_rows) *first_rows = M;
+  if (first_cols) *first_cols = N;
+  if (!valid_in(in_dtype) || M <= 0 || N <= 0 || K <= 0 || !extents_ok(M, N, K, K, K, N)) return MI355_ERR_SHAPE;
+  if (variant < MI355_VARIANT_AUTO || variant > MI355_VARIANT_ALTERNATE) return MI355_ERR_VARIANT;
+  if (variant != MI355_VARIANT_AUTO || resolve(M, N, K, K, K, N, in_dtype, variant) != MI355_VARIANT_BASIC) return 1;
+  bool along_m = false;
+  const int64_t first = mi355::ring_first_piece(M, N, K, elem_bytes(in_dtype), &along_m);
+  if (first <= 0) return 1;
+  if (along_m && first_rows) *first_rows = first;
+  if (!along_m && first_cols) *first_cols = first;
+  return 2;
 }
 
 size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int in_dtype, int variant) {
@@ -287,6 +307,15 @@ size_t mi355_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int in_dtype,
     Repack r;
     if (!repack_plan(nullptr, nullptr, nullptr, M, N, K, K, K, N, in_dtype, &r)) return 0;
     return r.bytes_a + r.bytes_b + r.bytes_c + mi355_gemm_workspace_bytes(M, r.Np, r.Kp, in_dtype, MI355_VARIANT_AUTO);
+  }
+  if (v == MI355_VARIANT_BASIC && variant == MI355_VARIANT_AUTO) {   // two launches: what the hungrier piece wants
+    bool along_m = false;
+    const int64_t first = mi355::ring_first_piece(M, N, K, elem_bytes(in_dtype), &along_m);
+    if (first > 0) {
+      const size_t a = mi355_gemm_workspace_bytes(along_m ? first : M, along_m ? N : first, K, in_dtype, MI355_VARIANT_BASIC);
+      const size_t b = mi355_gemm_workspace_bytes(along_m ? M - first : M, along_m ? N : N - first, K, in_dtype, MI355_VARIANT_BASIC);
+      return a > b ? a : b;
+    }
   }
   int splits = 1;
   if (v == MI355_VARIANT_SKINNY) splits = mi355::stream_splits(M, N, K, elem_bytes(in_dtype));
@@ -539,6 +568,24 @@ int run_gemm(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_
         if (r.c && mi355::launch_copy_out(wc, M, N, r.ld_c, C, ldc, s) != 0) return MI355_ERR_LAUNCH;
         return MI355_OK;
       }
+    }
+  }
+  if (variant == MI355_VARIANT_AUTO && v == MI355_VARIANT_BASIC) {
+    // Two launches where the planner finds a cut that spares a partly filled last round (ring_first_piece): each
+    // piece is the single-group kernel's problem of its own, with its own tile, splits and store policy, one after
+    // the other on the stream and through the same workspace.
+    bool along_m = false;
+    const int64_t first = mi355::ring_first_piece(M, N, K, elem_bytes(in_dtype), &along_m);
+    if (first > 0) {
+      const int64_t es = elem_bytes(in_dtype);
+      st = run_gemm(A, B, C, along_m ? first : M, along_m ? N : first, K, lda, ldb, ldc, in_dtype, out_dtype, scale, scale_a,
+                    scale_b, MI355_VARIANT_BASIC, workspace, workspace_bytes, stream, mode);
+      if (st != MI355_OK) return st;
+      const uint8_t* a2 = (const uint8_t*)A + (along_m ? first * lda * es : 0);
+      const uint8_t* b2 = (const uint8_t*)B + (along_m ? 0 : first * ldb * es);
+      uint8_t* c2 = (uint8_t*)C + (along_m ? first * ldc : first) * 2;   // 16-bit output
+      return run_gemm(a2, b2, c2, along_m ? M - first : M, along_m ? N : N - first, K, lda, ldb, ldc, in_dtype, out_dtype, scale,
+                      scale_a, scale_b, MI355_VARIANT_BASIC, workspace, workspace_bytes, stream, mode);
     }
   }
   int rc;

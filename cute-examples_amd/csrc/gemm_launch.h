@@ -66,6 +66,9 @@ inline int ring_tile_cols(int tile) { return tile == 256 ? 256 : 128; }
 // block_scaled: for the kernel with block scales, which exists on the five-slot ring only.
 int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_scaled = false);
 int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_scaled = false);
+// Whether MI355_VARIANT_AUTO runs the problem as two launches of the single-group kernel: the first piece's extent
+// along N (along M with *along_m set), or 0 for one launch.  Pure host heuristic; plain operands only.
+int64_t ring_first_piece(int64_t M, int64_t N, int64_t K, int elem_bytes, bool* along_m);
 // C = rne(scale * sum_s partial[s]) for partial laid out [splits][M][N] in fp32.
 int launch_splitk_reduce(const float* partial, const GemmArgs& g, int out_dtype, hipStream_t stream);
 int launch_tile_ring(const GemmArgs& g, int in_dtype, int out_dtype, int tile, hipStream_t stream);

@@ -214,6 +214,49 @@ int ring_tile_edge(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_s
   return e256 <= best ? 256 : e2 <= best ? kRingTile256x128 : single_round ? kRingTile128DeepPlain : 128;
 }
 
+// Two launches instead of one.  A problem whose 256 x 256 tiles do not fill their last round of workgroups leaves CUs
+// idle in it (or pays partial sums for a tail split).  Cut along N (or M) so that the first piece is a whole number of
+// rounds, and the rest is a problem of its own, for which the planner may take another tile.  Decided on the estimates
+// above: the candidates are the (up to four) largest first pieces that are whole rounds; the best of them is taken
+// when it promises at least 2 % over the single launch, the second launch counted with 3 us.  Measured against the
+// single launch on 61 problems the estimates would cut (bf16 and e4m3, 1...9 rounds): up to 3.3 rounds all 22 gain,
+// 4-21 % (bf16 4096 x 6144 x 1728 72 -> 67 us, 12544 x 4096 x 7104 547 -> 482 us, e4m3 4096 x 6144 x 4096 90 -> 76 us);
+// at 3.5 rounds 2-4 % up to 64 k-steps (bf16 4096 x 14336 x 4096 329 -> 321 us) and from 3 % more to 4 % less beyond;
+// from 4 rounds on from 5 % less to 5 % more, 1 % on average.  So: at most 3.4 rounds, or 3.6 with at most 64 k-steps.
+// Returns the first piece's extent along N (or along M, *along_m set), 0 for a single launch.
+int64_t ring_first_piece(int64_t M, int64_t N, int64_t K, int elem_bytes, bool* along_m) {
+  *along_m = false;
+  if (std::getenv("MI355_ONE_PIECE")) return 0;   // for measurements: never cut
+  const int64_t tm = (M + 255) / 256, tn = (N + 255) / 256;
+  const int64_t steps = k_steps_of(K, elem_bytes);
+  if (tm * tn <= kCuSlots || (tm * tn) % kCuSlots == 0 || steps < kShortSteps) return 0;
+  if (10 * tm * tn > 36 * kCuSlots || (10 * tm * tn > 34 * kCuSlots && steps > 64)) return 0;
+  const auto best_of = [&](int64_t m, int64_t n) {
+    const double a = estimate_us(256, m, n, K, elem_bytes), b = estimate_us(kRingTile256x128, m, n, K, elem_bytes),
+                 c = estimate_us(128, m, n, K, elem_bytes);
+    return a < b ? (a < c ? a : c) : (b < c ? b : c);
+  };
+  const double whole = best_of(M, N), second_launch_us = 3.0;
+  double best = 0.98 * whole;
+  int64_t extent = 0;
+  for (int axis = 0; axis < 2; ++axis) {
+    const int64_t across = axis == 0 ? tm : tn, along = axis == 0 ? tn : tm;   // axis 0: cut N, axis 1: cut M
+    int64_t g = across, h = kCuSlots;                                         // gcd(across, 256)
+    while (h) { const int64_t r = g % h; g = h; h = r; }
+    const int64_t step = kCuSlots / g;                                        // tile columns (rows) per whole number of rounds
+    int64_t c = (along - 1) / step * step;
+    for (int tries = 0; tries < 4 && c >= step; ++tries, c -= step) {
+      const double e = axis == 0 ? best_of(M, c * 256) + best_of(M, N - c * 256) : best_of(c * 256, N) + best_of(M - c * 256, N);
+      if (e + second_launch_us < best) {
+        best = e + second_launch_us;
+        extent = c * 256;
+        *along_m = axis == 1;
+      }
+    }
+  }
+  return extent;
+}
+
 // K splits for the single-group kernel on the tile ring_tile_edge picks.
 int ring_splits(int64_t M, int64_t N, int64_t K, int elem_bytes, bool block_scaled) {
   return uniform_splits(tiles_of(M, N, ring_tile_edge(M, N, K, elem_bytes, block_scaled)), k_steps_of(K, elem_bytes));

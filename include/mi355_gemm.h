@@ -235,6 +235,16 @@ int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant,
                     int *tile_rows, int *tile_cols, int *k_splits,
                     int *tail_tiles, int *tail_splits);
 
+/* How many launches of the GEMM kernel a call makes for this problem: 1, or 2 where MI355_VARIANT_AUTO cuts a
+ * problem of the tiled kernel along N or M so that the first piece fills a whole number of rounds of workgroups and
+ * the rest runs as a problem of its own (mi355_gemm_plan then describes the first piece; the second is what
+ * MI355_VARIANT_BASIC plans for its shape).  *first_rows x *first_cols receive the first piece's extent (M x N for one
+ * launch); either may be NULL.  Explicit variants never cut.  Returns a negative mi355_status for bad arguments.
+ * Pure host function.  Counterpart in the reference: none (its Scheduler walks one tile grid per launch,
+ * kernels/gemm_kernels/sm90a/gemm.cuh:168-212). */
+int mi355_gemm_pieces(int64_t M, int64_t N, int64_t K, int in_dtype, int variant,
+                      int64_t *first_rows, int64_t *first_cols);
+
 /* The variant MI355_VARIANT_AUTO resolves to for this problem (an enum mi355_variant value),
  * or a negative mi355_status.  Replaces the compile-time choice of kernel header at
  * kernels/gemm_kernels/sm90a/gemm_test.cu:7 / kernels/setup.py:12-15. */

@@ -53,6 +53,8 @@ def load(path=LIB):
     ip = ctypes.POINTER(ctypes.c_int)
     L.mi355_gemm_plan.argtypes = [i64, i64, i64, ci, ci, ip, ip, ip, ip, ip]
     L.mi355_gemm_plan.restype = ci
+    L.mi355_gemm_pieces.argtypes = [i64, i64, i64, ci, ci, ctypes.POINTER(i64), ctypes.POINTER(i64)]
+    L.mi355_gemm_pieces.restype = ci
     L.mi355_gemm_select_variant.argtypes = [i64, i64, i64, ci]
     L.mi355_gemm_select_variant.restype = ci
     L.mi355_gemm_check.argtypes = [i64, i64, i64, i64, i64, i64, ci, ci, ci]

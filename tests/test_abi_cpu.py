@@ -342,6 +342,7 @@ def test_plan_invariants_over_random_shapes(abi):
     import random
     rng = random.Random(7)
     seen = set()
+    seen_pieces = set()
     seen_alternate = False
     for dt, es in ((ac.BF16, 2), (ac.F16, 2), (ac.E4M3, 1)):
         for _ in range(3000):
@@ -364,6 +365,20 @@ def test_plan_invariants_over_random_shapes(abi):
             assert (v == ac.SKINNY) == (M <= 64 or (not deep and M <= 128 and -(-N // 64) <= 256 and M * K * es <= 2200000))
             if deep and M > 64:
                 assert (v, rows, cols) == (ac.BASIC, 128, 128), (M, N, K)
+            # Two launches: the plan describes the first piece, a whole number of rounds of 256 x 256 tiles cut off
+            # along one axis; the workspace is what the hungrier piece wants on the tile kernel.
+            first_rows, first_cols = ctypes.c_int64(), ctypes.c_int64()
+            pieces = abi.mi355_gemm_pieces(M, N, K, dt, ac.AUTO, ctypes.byref(first_rows), ctypes.byref(first_cols))
+            Mp, Np = first_rows.value, first_cols.value
+            assert pieces in (1, 2) and (pieces == 2) == ((Mp, Np) != (M, N))
+            if pieces == 2:
+                seen_pieces.add(Mp != M)
+                assert v == ac.BASIC and steps >= 16 and (Mp == M) != (Np == N) and 0 < Mp <= M and 0 < Np <= N
+                assert (Mp if Mp != M else Np) % 256 == 0 and (-(-Mp // 256) * -(-Np // 256)) % 256 == 0
+                assert (-(-M // 256) * -(-N // 256)) % 256 != 0
+                rest = (M - Mp, N) if Mp != M else (M, N - Np)
+                assert abi.mi355_gemm_pieces(Mp, Np, K, dt, ac.BASIC, None, None) == 1      # explicit variants never cut
+            M_all, N_all, M, N = M, N, Mp, Np
             tiles = -(-M // rows) * -(-N // cols)
             assert splits >= 1 and tail_splits >= 1 and tail_tiles >= 0
             if splits > 1:
@@ -380,8 +395,11 @@ def test_plan_invariants_over_random_shapes(abi):
                     assert tail_tiles * tail_splits <= 256 and steps // tail_splits >= 16      # uneven cuts allowed
                     want = tail_tiles * tail_splits * 256 * 256 * 4
                 seen.add((rows, cols, splits > 1, tail_tiles > 0))
-            assert abi.mi355_gemm_workspace_bytes(M, N, K, dt, ac.AUTO) == want, (M, N, K)
-    assert len(seen) >= 7 and seen_alternate, seen
+            if pieces == 2:
+                assert abi.mi355_gemm_workspace_bytes(M, N, K, dt, ac.BASIC) == want, (M, N, K)
+                want = max(want, abi.mi355_gemm_workspace_bytes(rest[0], rest[1], K, dt, ac.BASIC))
+            assert abi.mi355_gemm_workspace_bytes(M_all, N_all, K, dt, ac.AUTO) == want, (M_all, N_all, K)
+    assert len(seen) >= 7 and seen_alternate and seen_pieces == {False, True}, (seen, seen_pieces)
 
 
 def test_noalloc_entry_point_decides_before_any_hip_call(abi):

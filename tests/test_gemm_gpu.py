@@ -5,6 +5,8 @@ the dtypes, ragged shapes and full sizes of the benchmark configurations.
 
 Tolerances: relative Frobenius error <= 1e-2 for bf16/fp16 and <= 3e-2 for fp8 (against the fp32
 product of the dequantised operands); closed-form and permutation cases are bit-exact."""
+import ctypes
+
 import pytest
 import torch
 
@@ -344,7 +346,10 @@ def test_tail_split(abi, dt, M, N, K):
     bad = d > 2e-2 * S.cpu().float().abs() + 2e-2 * (K ** 0.5) * scale
     assert int(bad.sum()) == 0, (int(bad.sum()), float(d.max()))
     C2 = run_abi(abi, A, B, ac.AUTO, scale)
-    assert torch.equal(C.view(torch.int16), C2.view(torch.int16))
+    if abi.mi355_gemm_pieces(M, N, K, ac.torch_code(dt), ac.AUTO, None, None) == 1:
+        assert torch.equal(C.view(torch.int16), C2.view(torch.int16))
+    else:       # two launches instead of a tail split: other summation order inside the tiles that were cut
+        check(C2, A, B, scale)
     # no workspace: same tiles, no split; differs from C only by the summation order inside the tail tiles
     C3 = torch.full((M, N), float("nan"), dtype=out_dtype_of(dt), device="cuda")
     rc = abi.mi355_gemm_tn(Ad.data_ptr(), Bd.data_ptr(), C3.data_ptr(), M, N, K, K, K, N, ac.torch_code(dt),
@@ -985,3 +990,47 @@ def test_fp8_gemm_with_device_resident_scales(abi):
         assert rc == 0
         torch.cuda.synchronize()
         assert oracle.rel_frobenius(C3, ref) < 4e-3, variant
+
+
+@pytest.mark.parametrize("dt,M,N,K,along_m", [
+    (torch.bfloat16, 4096, 14336, 4096, False),       # 3.5 rounds of 256 x 256 tiles: 12288 + 2048 columns
+    (torch.bfloat16, 14336, 4096, 4096, True),        # the same cut along M
+    (torch.float8_e4m3fn, 4096, 6144, 4096, False),   # 1.5 rounds: 4096 + 2048 columns instead of a tail split
+    (torch.float16, 4000, 14300, 2056, False),        # ragged rows, columns and last k-step
+    (torch.bfloat16, 14300, 4000, 2056, True),
+    (torch.float8_e4m3fn, 2048, 10240, 2048, False),
+])
+def test_two_launches_where_the_last_round_would_be_partly_filled(abi, dt, M, N, K, along_m):
+    """MI355_VARIANT_AUTO cuts such a problem into a first piece of whole rounds and a rest (mi355_gemm_pieces says
+    where): the result must pass the oracle on sampled rows, agree element by element with the one-thread-per-output
+    kernel, leave everything outside C alone (padded rows of C, guard rows), come out the same twice, and be what the
+    two pieces give when the caller runs them as problems of their own."""
+    code = ac.torch_code(dt)
+    rows, cols = ctypes.c_int64(), ctypes.c_int64()
+    assert abi.mi355_gemm_pieces(M, N, K, code, ac.AUTO, ctypes.byref(rows), ctypes.byref(cols)) == 2
+    assert (rows.value != M) == along_m and (cols.value != N) == (not along_m)
+    first = rows.value if along_m else cols.value
+    assert first % 256 == 0 and 0 < first < (M if along_m else N)
+    A = rand((M, K), M + 1, torch.float32).clamp_(-50, 50).to(dt)
+    B = rand((N, K), N + 2, torch.float32).clamp_(-50, 50).to(dt)
+    scale = 2.0 ** -3
+    C = run_abi(abi, A, B, ac.AUTO, scale, ldc=N + 24)
+    _sampled_rows_check(C, A, B, scale, TOL[dt])
+    Ad, Bd = A.cuda(), B.cuda()
+    S = torch.empty((M, N), dtype=out_dtype_of(dt), device="cuda")
+    assert ac.gemm_tn(abi, Ad, Bd, S, scale, ac.SIMPLE) == 0
+    torch.cuda.synchronize()
+    d = (C.float() - S.cpu().float()).abs()
+    bad = d > 2e-2 * S.cpu().float().abs() + 2e-2 * (K ** 0.5) * scale * 50
+    assert int(bad.sum()) == 0, (int(bad.sum()), float(d.max()))
+    assert torch.equal(run_abi(abi, A, B, ac.AUTO, scale).view(torch.int16), C.contiguous().view(torch.int16))
+    # the caller's own two calls on the pieces (explicit variants never cut)
+    P = torch.full((M, N), float("nan"), dtype=out_dtype_of(dt), device="cuda")
+    if along_m:
+        assert ac.gemm_tn(abi, Ad[:first], Bd, P[:first], scale, ac.BASIC) == 0
+        assert ac.gemm_tn(abi, Ad[first:], Bd, P[first:], scale, ac.BASIC) == 0
+    else:
+        assert ac.gemm_tn(abi, Ad, Bd[:first], P[:, :first], scale, ac.BASIC) == 0
+        assert ac.gemm_tn(abi, Ad, Bd[first:], P[:, first:], scale, ac.BASIC) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(P.cpu().view(torch.int16), C.contiguous().view(torch.int16))
