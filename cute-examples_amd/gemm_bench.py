@@ -12,7 +12,7 @@ cross-checked (relative Frobenius distance between the two results on the same o
 run ends with the reference's summary table (:635-672) and, with --out, one JSON file.
 
     PYTHONPATH=cute-examples_amd python cute-examples_amd/gemm_bench.py [--dtype bf16|fp16] [--runs 100]
-                                        [--shapes 1024x1024,8192x16384] [--out sweep.json]
+                                        [--shapes 1024x1024,8192x16384,4096x14336x4096] [--out sweep.json]
 """
 import argparse
 import json
@@ -97,7 +97,7 @@ def summary_table(rows, peak):
            f"{'':12} {'(ms / TFLOPS)':<18} {'(ms / TFLOPS)':<20} {'(speedup)':<12} {'(custom)':<10} {'(Frobenius)':<10}",
            "-" * 100]
     for r in rows:
-        shape = f"{r['M']}x{r['K']}"
+        shape = f"{r['M']}x{r['K']}" if r['M'] == r['N'] else f"{r['M']}x{r['N']}x{r['K']}"
         custom = f"{r['ours_wall_ms']:.3f} / {r['ours_wall_tflops']:.1f}"
         torch_s = f"{r['blas_wall_ms']:.3f} / {r['blas_wall_tflops']:.1f}"
         out.append(f"{shape:<12} {custom:<18} {torch_s:<20} {r['blas_wall_ms'] / r['ours_wall_ms']:<12.2f} "
@@ -109,7 +109,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp16"])
     ap.add_argument("--runs", type=int, default=100)
-    ap.add_argument("--shapes", default=None, help="comma-separated s0xs1 (M = N = s0, K = s1); default: the reference's six")
+    ap.add_argument("--shapes", default=None, help="comma-separated s0xs1 (M = N = s0, K = s1, the reference's notation) or "
+                                                   "MxNxK; default: the reference's six")
     ap.add_argument("--json", action="store_true", help="also print one JSON line per shape")
     ap.add_argument("--out", default=None, help="write all rows and the run's parameters to this JSON file")
     a = ap.parse_args()
@@ -126,9 +127,10 @@ def main():
     hdr = f"{'M=N':>6} {'K':>6} | {'ours ms':>8} {'TF':>7} {'%pk':>5} | {'blas ms':>8} {'TF':>7} {'%pk':>5} | {'ours/blas':>9} || {'ours ev-ms':>10} {'TF':>7} | {'blas ev-ms':>10} {'TF':>7}"
     print(hdr)
     print("-" * len(hdr))
-    for s0, s1 in shapes:
-        M = N = s0
-        K = s1
+    for shape in shapes:
+        if len(shape) not in (2, 3):
+            raise SystemExit("a shape is s0xs1 or MxNxK, not %r" % (shape,))
+        M, N, K = (shape[0], shape[0], shape[1]) if len(shape) == 2 else shape
         flops = 2.0 * M * N * K
         for fn in (ours, blas):                              # warm-up, as gemm_bench.py:473-481
             A, B, C = fresh_operands(M, N, K, dtype, flush)
@@ -140,7 +142,8 @@ def main():
         e_ours = events_back_to_back(ours, M, N, K, dtype, a.runs)
         e_blas = events_back_to_back(blas, M, N, K, dtype, a.runs)
         tf = lambda t: flops / t / 1e12
-        print(f"{M:>6} {K:>6} | {t_ours*1e3:8.4f} {tf(t_ours):7.1f} {100*tf(t_ours)/peak:5.1f} | "
+        label = f"{M:>6}" if M == N else f"{M}x{N}"
+        print(f"{label} {K:>6} | {t_ours*1e3:8.4f} {tf(t_ours):7.1f} {100*tf(t_ours)/peak:5.1f} | "
               f"{t_blas*1e3:8.4f} {tf(t_blas):7.1f} {100*tf(t_blas)/peak:5.1f} | {t_blas/t_ours:9.3f} || "
               f"{e_ours*1e3:10.4f} {tf(e_ours):7.1f} | {e_blas*1e3:10.4f} {tf(e_blas):7.1f}", flush=True)
         rows.append({"M": M, "N": N, "K": K, "dtype": a.dtype, "rel_diff": rel,

@@ -18,12 +18,14 @@ def test_gemm_bench_two_smallest_shapes(tmp_path):
     out = tmp_path / "sweep.json"
     env = dict(os.environ, PYTHONPATH=os.path.join(ROOT, "cute-examples_amd"))
     proc = subprocess.run([sys.executable, os.path.join(ROOT, "cute-examples_amd", "gemm_bench.py"), "--runs", "3",
-                           "--shapes", "1024x1024,2048x2048", "--out", str(out)],
+                           "--shapes", "1024x1024,2048x2048,512x1536x1024", "--out", str(out)],
                           capture_output=True, text=True, env=env, timeout=300)
     assert proc.returncode == 0, proc.stdout + proc.stderr
     assert "PERFORMANCE SUMMARY" in proc.stdout and "1024x1024" in proc.stdout and "2048x2048" in proc.stdout
+    assert "512x1536x1024" in proc.stdout       # a shape with M != N, which the reference's notation cannot name
     data = json.loads(out.read_text())
-    assert data["comparator"].startswith("torch.mm") and len(data["rows"]) == 2
+    assert data["comparator"].startswith("torch.mm") and len(data["rows"]) == 3
+    assert (data["rows"][2]["M"], data["rows"][2]["N"], data["rows"][2]["K"]) == (512, 1536, 1024)
     for row in data["rows"]:
         assert row["rel_diff"] <= 1e-2, row                     # ours and torch.mm on the same operands
         for key in ("ours_wall_ms", "blas_wall_ms", "ours_event_ms", "blas_event_ms"):
