@@ -45,6 +45,7 @@ ROWS = {
     "tile kernel, uniform K split": [(256, 6144, 4096, torch.bfloat16), (256, 4096, 2048, torch.bfloat16),
                                      (130, 1024, 4096, torch.float16)],
     "tile kernel, tail split": [(4096, 6144, 4096, torch.bfloat16), (4352, 4352, 2048, torch.bfloat16)],
+    "tile kernel, two launches, the second with a K split": [(8704, 4096, 2496, torch.bfloat16), (2048, 8448, 6912, torch.float16)],
     "fp8": [(256, 14336, 4096, torch.float8_e4m3fn), (16, 4096, 14336, torch.float8_e4m3fn)],
     "repacked misaligned problem": [(1001, 1003, 1001, torch.bfloat16), (515, 1003, 777, torch.bfloat16)],
 }
