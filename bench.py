@@ -200,6 +200,21 @@ def build_case(name, variant, device="cuda", seed=0):
             else:
                 sets.append((X.to(torch.float8_e4m3fn), (W * 50.0).to(torch.float8_e4m3fn)))
         tag, fp8 = "e4m3", (("mxsets",) if name.startswith("skinnymx_") else (1.0, 1.0))
+    elif name.startswith("quant_e4m3_") or name.startswith("quant_mxfp8_"):
+        # the quantisers in front of the fp8 GEMMs: bf16 (rows, K) -> e4m3 with one scale per tensor (two passes over
+        # x: maximum, then cast) or with one E8M0 scale per 32 elements in the GEMM's layout (one pass)
+        rows, K = (int(x) for x in name.split("_")[2:])
+        x = torch.randn(rows, K, device=device, generator=torch.Generator(device=device).manual_seed(seed)).to(torch.bfloat16)
+        per_tensor = name.startswith("quant_e4m3_")
+
+        def call():
+            if per_tensor:
+                gemm_kernels.quantize_e4m3(x)
+            else:
+                gemm_kernels.quantize_mxfp8(x, shuffled=True)
+        n = rows * K
+        nbytes = (2 * 2 * n + n) if per_tensor else (2 * n + n + n // 32)
+        return call, 0.0, nbytes, "bf16", (rows, 0, K), [(x, x)], None, None
     else:
         raise SystemExit("unknown workload " + name)
     M, K = sets[0][0].shape
@@ -635,7 +650,8 @@ def main():
     if not a.no_extras:
         names = ["bf16_8192", "fp8_8192", "mxfp8_8192", "bf16_4096", "fp16_512"] + \
                 ["skinny_%d_%d_%d" % (m, n, k) for (n, k) in ((14336, 4096), (4096, 14336), (6144, 4096))
-                 for m in (16, 64, 256)] + ["skinny_128_8192_4096", "skinnyfp8_16_14336_4096", "skinnymx_16_14336_4096"]
+                 for m in (16, 64, 256)] + ["skinny_128_8192_4096", "skinnyfp8_16_14336_4096", "skinnymx_16_14336_4096",
+                                            "quant_e4m3_8192_8192", "quant_mxfp8_8192_8192"]
         for n in names:
             if n == a.workload or (n == "fp8_8192" and fp8_block):
                 continue

@@ -94,11 +94,7 @@ __global__ __launch_bounds__(256) void mx_quantize_kernel(const void* __restrict
   const float inv = __builtin_bit_cast(float, (254u - byte) << 23);  // 2^(127 - byte), exact
   uint32_t w[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    w[i] = 0;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) w[i] |= to_e4m3(v[4 * i + k] * inv) << (8 * k);
-  }
+  for (int i = 0; i < 8; ++i) w[i] = to_e4m3x4(v[4 * i] * inv, v[4 * i + 1] * inv, v[4 * i + 2] * inv, v[4 * i + 3] * inv);
   u32x4* dst = (u32x4*)(q + row * blocks_per_row * kMxBlock + blk * kMxBlock);
   dst[0] = (u32x4){w[0], w[1], w[2], w[3]};
   dst[1] = (u32x4){w[4], w[5], w[6], w[7]};

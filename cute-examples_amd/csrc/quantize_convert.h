@@ -50,4 +50,20 @@ __device__ __forceinline__ uint32_t to_e4m3(float f) {
   return sign | code;
 }
 
+// Four fp32 -> four e4m3 codes in one word (a in the lowest byte), bit for bit what to_e4m3 gives: the hardware
+// conversion (v_cvt_pk_fp8_f32, OCP e4m3 on this GPU, round to nearest even) behind an explicit clamp to +-448.  A NaN
+// is carried around the clamp, which would turn it into a number, and comes out of the conversion as a code whose
+// low seven bits are all ones, as no number does; the sign of such codes is cleared afterwards.
+__device__ __forceinline__ uint32_t to_e4m3x4(float a, float b, float c, float d) {
+  const auto clamped = [](float f) __attribute__((always_inline)) {
+    const float inside = __builtin_amdgcn_fmed3f(f, -448.0f, 448.0f);
+    return f != f ? f : inside;
+  };
+  int w = __builtin_amdgcn_cvt_pk_fp8_f32(clamped(a), clamped(b), 0, false);
+  w = __builtin_amdgcn_cvt_pk_fp8_f32(clamped(c), clamped(d), w, true);
+  const uint32_t u = (uint32_t)w;
+  const uint32_t nan_sign = ((u & 0x7f7f7f7fu) + 0x01010101u) & 0x80808080u;   // bit 7 of the bytes that hold 0x7f or 0xff
+  return u & ~nan_sign;
+}
+
 }  // namespace mi355
