@@ -224,6 +224,33 @@ def test_quantizer_is_bit_exact(abi, dtype):
     assert torch.equal(q.cpu(), want_q.view(torch.uint8))
 
 
+def test_quantizer_conversion_on_a_dense_sweep_of_fp32_patterns(abi):
+    """The kernels convert fp32 to e4m3 with the hardware instruction; the oracle does it in integer arithmetic.
+    Blocks whose first element is 256 have the scale 1, so their other 31 elements come out as the conversion of the
+    raw fp32 pattern: 4.2 million patterns spread evenly over [0, 448] (and a few beyond, which must saturate), both
+    signs, every binade down to the fp32 subnormals, must give the oracle's code."""
+    import numpy as np
+    rows, K = 4096, 1024
+    i = np.arange(rows * K, dtype=np.uint64)
+    bits = ((i * 1021 * 268) % 0x43f00000).astype(np.uint32)          # magnitudes up to 480
+    bits |= ((i >> 3) & 1).astype(np.uint32) << 31                     # both signs
+    x = torch.from_numpy(bits.view(np.float32).copy()).reshape(rows, K)
+    x[:, ::32] = 256.0
+    assert float(x.abs().max()) < 512.0 and bool(torch.isfinite(x).all())
+    q = torch.empty(x.shape, dtype=torch.uint8, device="cuda")
+    sc = torch.empty(rows, K // 32, dtype=torch.uint8, device="cuda")
+    xd = x.cuda()
+    rc = abi.mi355_quantize_mxfp8(xd.data_ptr(), ac.F32, rows, K, xd.stride(0), q.data_ptr(), sc.data_ptr(), 0,
+                                  torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert bool((sc.cpu() == 127).all())                               # every block: scale 2^0
+    want_q, want_s = oracle.quantize_mxfp8(x)
+    assert torch.equal(sc.cpu(), want_s) and torch.equal(q.cpu(), want_q.view(torch.uint8))
+    codes = q.cpu()
+    assert len(torch.unique(codes)) >= 250                             # the sweep reaches (nearly) every code
+
+
 @pytest.mark.parametrize("rows", [300, 256, 1])
 def test_quantizer_writes_shuffled_scales_directly(abi, rows):
     """The quantiser's shuffled output is byte for byte what mi355_mx_shuffle_scales makes of its
