@@ -360,6 +360,7 @@ int mi355_quantize_mxfp8(const void* x, int x_dtype, int64_t rows, int64_t K, in
   if (!x || !x_q || !scales) return MI355_ERR_NULL;
   const int64_t es = x_dtype == MI355_F32 ? 4 : 2;
   if ((uintptr_t)x % 16 != 0 || (ldx * es) % 16 != 0 || (uintptr_t)x_q % 16 != 0) return MI355_ERR_ALIGN;
+  if (scales_shuffled && (uintptr_t)scales % 8 != 0) return MI355_ERR_ALIGN;   // as mi355_mx_shuffle_scales wants its output
   return mi355::launch_quantize_mxfp8(x, x_dtype, rows, K, ldx, x_q, scales, scales_shuffled != 0, (hipStream_t)stream) == 0
              ? MI355_OK : MI355_ERR_LAUNCH;
 }

@@ -101,6 +101,49 @@ __global__ __launch_bounds__(256) void mx_quantize_kernel(const void* __restrict
   scales[kShuffled ? shuffled_index(row, blk, blocks_per_row) : id] = (uint8_t)byte;
 }
 
+// The quantiser that writes the shuffled layout, by patches of 128 rows x 8 blocks (two 512-byte units of scales):
+// eight neighbouring threads read 512 contiguous bytes of a row, the 1024 scale bytes of the patch are put in place
+// in LDS, and 256 threads write them out four bytes each, instead of every thread writing one byte to a line of its own
+// (bf16 8192 x 8192: 35.8 -> 30 us, what the natural layout takes).  Rows past the end get the scale 1.
+template <class In>
+__global__ __launch_bounds__(1024) void mx_quantize_shuffled_kernel(const void* __restrict__ x, int64_t rows,
+                                                                    int64_t blocks_per_row, int64_t ldx,
+                                                                    uint8_t* __restrict__ q, uint8_t* __restrict__ scales) {
+  __shared__ uint32_t patch[256];
+  const int t = threadIdx.x;
+  const int64_t row = (int64_t)blockIdx.y * 128 + t / 8, blk = (int64_t)blockIdx.x * 8 + t % 8;
+  uint32_t byte = 127u;
+  if (row < rows && blk < blocks_per_row) {
+    const int64_t at = row * ldx + blk * kMxBlock;
+    float v[kMxBlock];
+#pragma unroll
+    for (int i = 0; i < kMxBlock; i += 8) Load8<In>::run(x, at + i, v + i);
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < kMxBlock; ++i) amax = __builtin_fmaxf(amax, __builtin_fabsf(v[i]));
+    const uint32_t field = __builtin_bit_cast(uint32_t, amax) >> 23;     // as in mx_quantize_kernel
+    byte = amax == 0.f ? 127u : (field > 8u ? field - 8u : 0u);
+    const float inv = __builtin_bit_cast(float, (254u - byte) << 23);
+    uint32_t w[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = to_e4m3x4(v[4 * i] * inv, v[4 * i + 1] * inv, v[4 * i + 2] * inv, v[4 * i + 3] * inv);
+    u32x4* dst = (u32x4*)(q + row * blocks_per_row * kMxBlock + blk * kMxBlock);
+    dst[0] = (u32x4){w[0], w[1], w[2], w[3]};
+    dst[1] = (u32x4){w[4], w[5], w[6], w[7]};
+  }
+  // Byte of (row, block) inside its unit: lane (row % 16 + 16 * (block % 4)) x 8 + (row % 128) / 16 (shuffled_index).
+  const int r = t / 8, b = t % 8;
+  ((uint8_t*)patch)[(b / 4) * 512 + (r % 16 + 16 * (b % 4)) * 8 + r / 16] = (uint8_t)byte;
+  __syncthreads();
+  if (t < 256) {
+    const int64_t unit_blk = (int64_t)blockIdx.x * 8 + (t / 128) * 4;      // first block of the unit this thread writes to
+    if (unit_blk < blocks_per_row) {
+      const int64_t unit = (int64_t)blockIdx.y * (blocks_per_row / 4) + unit_blk / 4;
+      ((uint32_t*)(scales + unit * 512))[t % 128] = patch[t];
+    }
+  }
+}
+
 template <class In>
 int run_quantize(const void* x, int64_t rows, int64_t K, int64_t ldx, void* q, uint8_t* scales, bool shuffled,
                  hipStream_t stream) {
@@ -108,10 +151,15 @@ int run_quantize(const void* x, int64_t rows, int64_t K, int64_t ldx, void* q, u
   if (n == 0) return 0;
   const int64_t blocks = (n + 255) / 256;
   if (blocks >= ((int64_t)1 << 31)) return -1;
-  if (shuffled)
-    hipLaunchKernelGGL((mx_quantize_kernel<In, true>), dim3((unsigned)blocks), dim3(256), 0, stream, x, rows,
-                       K / kMxBlock, ldx, (uint8_t*)q, scales);
-  else
+  if (shuffled) {
+    const int64_t bpr = K / kMxBlock, gx = (bpr + 7) / 8, gy = (rows + 255) / 256 * 2;   // rows padded to 256: whole patches
+    if (gy > 65535 || gx >= ((int64_t)1 << 31))      // more than 8 million rows: the one-byte stores
+      hipLaunchKernelGGL((mx_quantize_kernel<In, true>), dim3((unsigned)blocks), dim3(256), 0, stream, x, rows, bpr, ldx,
+                         (uint8_t*)q, scales);
+    else
+      hipLaunchKernelGGL((mx_quantize_shuffled_kernel<In>), dim3((unsigned)gx, (unsigned)gy), dim3(1024), 0, stream, x, rows,
+                         bpr, ldx, (uint8_t*)q, scales);
+  } else
     hipLaunchKernelGGL((mx_quantize_kernel<In, false>), dim3((unsigned)blocks), dim3(256), 0, stream, x, rows,
                        K / kMxBlock, ldx, (uint8_t*)q, scales);
   return hipGetLastError() == hipSuccess ? 0 : -1;

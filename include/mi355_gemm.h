@@ -212,7 +212,7 @@ size_t mi355_mx_shuffled_bytes(int64_t rows, int64_t K);
  * layout, or, with scales_shuffled != 0 (K % 128 == 0), mi355_mx_shuffled_bytes(rows, K) bytes in the
  * layout mi355_gemm_tn_mxfp8 takes with scales_shuffled == 1 (no shuffle launch then).  Per block: scale = 2^(floor(log2(amax)) - 8) (1 for a block of zeros), elements
  * x/scale rounded to nearest even, saturated at +-448.  x 16-byte aligned with ldx*elem_bytes
- * % 16 == 0, x_q 16-byte aligned.  NaN and infinity are not supported.
+ * % 16 == 0, x_q 16-byte aligned, shuffled scales 8-byte aligned.  NaN and infinity are not supported.
  * Counterpart in the reference: none; OCP MX specification v1.0, section 6.3.
  */
 int mi355_quantize_mxfp8(const void *x, int x_dtype, int64_t rows, int64_t K, int64_t ldx,
