@@ -400,8 +400,16 @@ size_t mx_partial_bytes(int64_t M, int64_t N, int64_t K, int* splits, int* tail_
 size_t mi355_gemm_mx_workspace_bytes(int64_t M, int64_t N, int64_t K, int scales_shuffled) {
   if (M <= 0 || N <= 0 || K <= 0 || K % 128 != 0 || !extents_ok(M, N, K, K, K, N)) return 0;
   const int ss = mx_stream_splits(M, N, K, K, K, N);
-  const size_t partial = ss ? (ss > 1 ? (size_t)ss * (size_t)M * (size_t)N * sizeof(float) : 0)
-                            : mx_partial_bytes(M, N, K, nullptr, nullptr, nullptr);
+  size_t partial = ss ? (ss > 1 ? (size_t)ss * (size_t)M * (size_t)N * sizeof(float) : 0)
+                      : mx_partial_bytes(M, N, K, nullptr, nullptr, nullptr);
+  if (!ss) {   // two launches (as for plain operands): what the hungrier piece wants
+    bool along_m = false;
+    if (const int64_t first = mi355::ring_first_piece(M, N, K, 1, &along_m)) {
+      const size_t a = mx_partial_bytes(along_m ? first : M, along_m ? N : first, K, nullptr, nullptr, nullptr);
+      const size_t b = mx_partial_bytes(along_m ? M - first : M, along_m ? N : N - first, K, nullptr, nullptr, nullptr);
+      partial = a > b ? a : b;
+    }
+  }
   return partial + (scales_shuffled ? 0 : mi355::mx_shuffled_bytes(M, K) + mi355::mx_shuffled_bytes(N, K));
 }
 
@@ -458,20 +466,39 @@ int mi355_gemm_tn_mxfp8(const void* A_q, const void* B_q, void* C, int64_t M, in
       return mi355::launch_stream_mx(g, out_dtype, ss, (uint8_t*)workspace + used, s) == 0 ? MI355_OK : MI355_ERR_LAUNCH;
     }
   }
+  // The tile kernel on rows [m0, m0 + m) of A and rows [n0, n0 + n) of B (multiples of 256 but for the last).
   // K split or tail split when the rest of the workspace holds the partial results (optional, as
   // for the other tiled kernels: without it the tiles run unsplit).
-  int splits, tail_tiles, tail_splits;
-  const size_t partial = mx_partial_bytes(M, N, K, &splits, &tail_tiles, &tail_splits);
-  if (partial && workspace && (uintptr_t)workspace % 16 == 0 && workspace_bytes >= used + partial) {
-    g.partial = (float*)((uint8_t*)workspace + used);  // used is a multiple of 1024
-    g.splits = splits;
-    g.tail_tiles = tail_tiles;
-    g.tail_splits = tail_splits;
-  }
-  const int tile = mi355::ring_tile_edge(M, N, K, 1, true);
-  g.tiles_m = (M + mi355::ring_tile_rows(tile) - 1) / mi355::ring_tile_rows(tile);
-  g.tiles_n = (N + mi355::ring_tile_cols(tile) - 1) / mi355::ring_tile_cols(tile);
-  return mi355::launch_tile_ring_mx(g, out_dtype, tile, s) == 0 ? MI355_OK : MI355_ERR_LAUNCH;
+  const auto tiles_of_piece = [&](int64_t m0, int64_t m, int64_t n0, int64_t n) {
+    mi355::GemmArgs p = g;
+    p.A = (const uint8_t*)A_q + m0 * lda;
+    p.B = (const uint8_t*)B_q + n0 * ldb;
+    p.C = (uint8_t*)C + (m0 * ldc + n0) * 2;                              // 16-bit output
+    p.mx_a = g.mx_a + (m0 / 128) * (K / 128) * 512;                       // one 512-byte unit per 128 rows and k-step
+    p.mx_b = g.mx_b + (n0 / 128) * (K / 128) * 512;
+    p.M = m;
+    p.N = n;
+    p.c_streams = c_streams(m, n, K, 1);
+    int splits, tail_tiles, tail_splits;
+    const size_t partial = mx_partial_bytes(m, n, K, &splits, &tail_tiles, &tail_splits);
+    if (partial && workspace && (uintptr_t)workspace % 16 == 0 && workspace_bytes >= used + partial) {
+      p.partial = (float*)((uint8_t*)workspace + used);  // used is a multiple of 1024
+      p.splits = splits;
+      p.tail_tiles = tail_tiles;
+      p.tail_splits = tail_splits;
+    }
+    const int tile = mi355::ring_tile_edge(m, n, K, 1, true);
+    p.tiles_m = (m + mi355::ring_tile_rows(tile) - 1) / mi355::ring_tile_rows(tile);
+    p.tiles_n = (n + mi355::ring_tile_cols(tile) - 1) / mi355::ring_tile_cols(tile);
+    return mi355::launch_tile_ring_mx(p, out_dtype, tile, s) == 0 ? MI355_OK : MI355_ERR_LAUNCH;
+  };
+  // Two launches where a cut spares a partly filled last round of workgroups, as for plain operands (ring_first_piece).
+  bool along_m = false;
+  const int64_t first = mi355::ring_first_piece(M, N, K, 1, &along_m);
+  if (first <= 0) return tiles_of_piece(0, M, 0, N);
+  st = along_m ? tiles_of_piece(0, first, 0, N) : tiles_of_piece(0, M, 0, first);
+  if (st != MI355_OK) return st;
+  return along_m ? tiles_of_piece(first, M - first, 0, N) : tiles_of_piece(0, M, first, N - first);
 }
 
 int mi355_gemm_tn(const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,

@@ -239,7 +239,8 @@ int mi355_gemm_plan(int64_t M, int64_t N, int64_t K, int in_dtype, int variant,
  * problem of the tiled kernel along N or M so that the first piece fills a whole number of rounds of workgroups and
  * the rest runs as a problem of its own (mi355_gemm_plan then describes the first piece; the second is what
  * MI355_VARIANT_BASIC plans for its shape).  *first_rows x *first_cols receive the first piece's extent (M x N for one
- * launch); either may be NULL.  Explicit variants never cut.  Returns a negative mi355_status for bad arguments.
+ * launch); either may be NULL.  Explicit variants never cut; mi355_gemm_tn_mxfp8 cuts where this function says so for
+ * MI355_E4M3 operands (and M > 64).  Returns a negative mi355_status for bad arguments.
  * Pure host function.  Counterpart in the reference: none (its Scheduler walks one tile grid per launch,
  * kernels/gemm_kernels/sm90a/gemm.cuh:168-212). */
 int mi355_gemm_pieces(int64_t M, int64_t N, int64_t K, int in_dtype, int variant,

@@ -135,7 +135,8 @@ def test_mx_sizes_and_rejections_before_any_device_access(abi):
     assert ac.plan(abi, 256, 4096, 14336, ac.E4M3)[1:4] == (128, 128, 4)
     assert abi.mi355_gemm_mx_workspace_bytes(256, 4096, 14336, 1) == 7 * 256 * 4096 * 4
     assert abi.mi355_gemm_mx_workspace_bytes(256, 4096, 14336, 0) == 7 * 256 * 4096 * 4 + (256 + 4096) * 448
-    assert abi.mi355_gemm_mx_workspace_bytes(4096, 6144, 4096, 1) == 2 * 128 * 256 * 256 * 4
+    assert abi.mi355_gemm_mx_workspace_bytes(6144, 4096, 4096, 1) == 2 * 128 * 256 * 256 * 4      # tail split: 128 tiles cut in two
+    assert abi.mi355_gemm_mx_workspace_bytes(4096, 6144, 4096, 1) == 0                              # two launches instead
     assert abi.mi355_gemm_mx_workspace_bytes(512, 6144, 4096, 1) == 0      # 192 tiles of 128x128, unsplit
     f = abi.mi355_gemm_tn_mxfp8
     assert f(None, None, None, 256, 256, 128, 128, 128, 256, None, 4, None, 4, 0, ac.BF16, None, 0, None) == ac.ERR_NULL

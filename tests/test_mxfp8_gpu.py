@@ -6,6 +6,8 @@ Tolerance: relative Frobenius error <= 3e-2 against the fp32 product of the dequ
 the bf16/fp16 output rounding differ); the quantiser, the power-of-two cases and the permutation
 case are bit-exact."""
 import numpy as np
+import ctypes
+
 import pytest
 import torch
 
@@ -71,7 +73,7 @@ def test_ragged_tiles(abi, shape):
 
 
 @pytest.mark.parametrize("shuffled", [False, True])
-@pytest.mark.parametrize("shape", [(768, 768, 8192), (256, 4096, 14336), (4096, 6144, 4096), (300, 1000, 8192)])
+@pytest.mark.parametrize("shape", [(768, 768, 8192), (256, 4096, 14336), (6144, 4096, 4096), (300, 1000, 8192)])
 def test_k_split_and_tail_split(abi, shape, shuffled):
     """Few tiles: K split 4 ways on 128x128 tiles, 7 ways on 256x128 tiles; 384 tiles of 256x256: the
     last round cut in two.  Same result as without the workspace for the partial results (unsplit),
@@ -449,3 +451,31 @@ def test_fallback_build_of_the_block_scaled_kernel_gives_the_same_bits(abi, shap
     if M * N * K <= 768 * 768 * 8192:
         check(got, A, sa, B, sb)
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("shuffled", [False, True])
+@pytest.mark.parametrize("shape,along_m", [((4096, 6144, 4096), False), ((5120, 4096, 5120), True), ((2048, 10100, 2048), False)])
+def test_two_launches_where_the_last_round_would_be_partly_filled(abi, shape, along_m, shuffled):
+    """Block-scaled problems are cut like plain ones (mi355_gemm_pieces for e4m3 operands says where): the result must
+    pass the oracle on sampled rows and be, bit for bit, what the caller gets by running the two pieces as problems of
+    their own, each with its own rows of the operands and of the scales."""
+    M, N, K = shape
+    rows, cols = ctypes.c_int64(), ctypes.c_int64()
+    assert abi.mi355_gemm_pieces(M, N, K, ac.E4M3, ac.AUTO, ctypes.byref(rows), ctypes.byref(cols)) == 2
+    first = rows.value if along_m else cols.value
+    assert (rows.value != M) == along_m and (cols.value != N) == (not along_m) and first % 256 == 0
+    A, sa = random_mx(M, K, 71)
+    B, sb = random_mx(N, K, 72)
+    C = run_mx(abi, A, sa, B, sb, shuffled=shuffled, ldc=N + 16)
+    idx = torch.arange(0, M, max(1, M // 24))
+    ref = oracle.gemm_tn_mxfp8_fp32(A[idx], sa[idx], B, sb)
+    assert oracle.no_nan_left(C) and oracle.rel_frobenius(C[idx], ref) <= TOL
+    if along_m:
+        top = run_mx(abi, A[:first], sa[:first], B, sb, shuffled=shuffled)
+        bottom = run_mx(abi, A[first:], sa[first:], B, sb, shuffled=shuffled)
+        pieces = torch.cat([top, bottom], dim=0)
+    else:
+        left = run_mx(abi, A, sa, B[:first], sb[:first], shuffled=shuffled)
+        right = run_mx(abi, A, sa, B[first:], sb[first:], shuffled=shuffled)
+        pieces = torch.cat([left, right], dim=1)
+    assert torch.equal(pieces.view(torch.int16), C.contiguous().view(torch.int16))
