@@ -395,6 +395,15 @@ def clock_under_load(sets, C, fp8, variant, flops, ms_hint, do_settle):
                     "second stream beside the launches" % (waves, samples)}
 
 
+def guarded(yardstick, *args):
+    """A yardstick beside the measurement must not cost the measurement: None (and a line on stderr) if it fails."""
+    try:
+        return yardstick(*args)
+    except Exception as e:   # noqa: BLE001
+        print("bench.py: %s not available: %s: %s" % (yardstick.__name__, type(e).__name__, str(e)[:200]), file=sys.stderr)
+        return None
+
+
 def vendor_same_run(sets, C, fp8, flops, steps, warmup, do_settle):
     """The vendor library on the same operands, same protocol (settle, W warm-up, K timed launches):
     torch.mm (hipBLASLt) for the 16-bit types, torch._scaled_mm for e4m3 with per-tensor scales.
@@ -609,7 +618,7 @@ def main():
         if roof["torch_mm_same_run"]["value"]:
             roof["vs_torch_mm_same_run"] = round(head["tflops"] / roof["torch_mm_same_run"]["value"], 4)
     if roof["bound"] == "mfma" and not a.no_calibrate:
-        roof["shader_clock"] = clock_under_load(sets, C, fp8, a.variant, flops, head["ms"], do_settle)
+        roof["shader_clock"] = guarded(clock_under_load, sets, C, fp8, a.variant, flops, head["ms"], do_settle)
     if a.workload in PROFILED:
         roof["profiled"] = PROFILED[a.workload]
 
@@ -632,7 +641,7 @@ def main():
             if roof8["torch_mm_same_run"]["value"]:
                 roof8["vs_torch_mm_same_run"] = round(row["tflops"] / roof8["torch_mm_same_run"]["value"], 4)
         if not a.no_calibrate:
-            roof8["shader_clock"] = clock_under_load(sets8, C8, sc8, a.variant, flops8, row["ms"], do_settle)
+            roof8["shader_clock"] = guarded(clock_under_load, sets8, C8, sc8, a.variant, flops8, row["ms"], do_settle)
         roof8["profiled"] = PROFILED["fp8_8192"]
         fp8_block = {"value": row["tflops"], "unit": "TFLOP/s", "ms_per_step": row["ms"], "steps": a.steps,
                      "warmup": a.warmup, "settle_launches": row["settle_launches"], "settle_ms": row["settle_ms"],
@@ -669,7 +678,7 @@ def main():
                 torch.cuda.empty_cache()
 
     if a.workload == "bf16_8192" and a.variant == "auto" and not a.no_extras and not a.no_vendor:
-        roof["larger_shapes"] = larger_shapes(40, do_settle)
+        roof["larger_shapes"] = guarded(larger_shapes, 40, do_settle)
 
     # Last, so that the GPU does not idle (and drop its clocks) in the middle of the measurements.
     cpu = cpu_baseline(*cpu_operands) if cpu_operands else None
