@@ -261,7 +261,7 @@ def roofline_of(row, workload, variant, sets, flops, nbytes):
     """The roofline object of one measured workload (the dominant kernel is its only GEMM kernel)."""
     import gemm_kernels
     traffic = MEASURED_TRAFFIC_BYTES.get(workload)
-    if not workload.startswith("skinny"):
+    if not workload.startswith(("skinny", "quant_")):
         roof = {"bound": "mfma", "achieved": row["tflops"], "peak": PEAK_TFLOPS[row["dtype"]],
                 "unit": "TFLOP/s", "frac": round(row["tflops"] / PEAK_TFLOPS[row["dtype"]], 4), "traffic": traffic}
     else:
@@ -269,8 +269,11 @@ def roofline_of(row, workload, variant, sets, flops, nbytes):
                 "frac": round(row["gbs"] / PEAK_HBM_GBS, 4), "traffic": traffic}
     # the counters are not read in this run: the figure is the one of the committed profile of this command
     roof["traffic_source"] = (TRAFFIC_PROFILE[workload] + " (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE of this script; not re-measured)") if traffic else None
-    roof["kernel"] = gemm_kernels.select_variant(row["M"], row["N"], row["K"], sets[0][0].dtype) \
-        if variant == "auto" else variant
+    if workload.startswith("quant_"):
+        roof["kernel"] = "amax_kernel + quantize_kernel" if workload.startswith("quant_e4m3") else "mx_quantize_shuffled_kernel"
+    else:
+        roof["kernel"] = gemm_kernels.select_variant(row["M"], row["N"], row["K"], sets[0][0].dtype) \
+            if variant == "auto" else variant
     roof["flops_per_launch"] = flops
     roof["algorithmic_bytes_per_launch"] = nbytes
     roof["avg_launch_ms"] = row["ms"]
@@ -604,6 +607,8 @@ def main():
         torch.cuda.empty_cache()
 
     do_settle = not a.no_settle
+    if a.workload.startswith("quant_"):      # no GEMM: no CPU GEMM baseline, no second configuration
+        a.no_cpu = a.no_fp8 = True
     head, keep = measure(a.workload, a.variant, a.steps, a.warmup, do_settle)
     sets, C, fp8, flops, nbytes = keep
     roof = roofline_of(head, a.workload, a.variant, sets, flops, nbytes)

@@ -26,6 +26,15 @@ __global__ __launch_bounds__(256) void amax_kernel(const void* x, int64_t n, flo
   float m = 0.f;
   const int64_t stride = (int64_t)gridDim.x * 256 * 8;
   int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  for (; i + 3 * stride + 8 <= n; i += 4 * stride) {   // four loads in flight per thread: few workgroups run this
+    float v[4][8];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) Load8<In>::run(x, i + u * stride, v[u]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) m = __builtin_fmaxf(m, __builtin_fabsf(v[u][k]));
+  }
   for (; i + 8 <= n; i += stride) {
     float v[8];
     Load8<In>::run(x, i, v);
