@@ -24,9 +24,10 @@ def _capture(fn):
     return g
 
 
-@pytest.mark.parametrize("shape", [(512, 768, 1024), (16, 4096, 4096), (512, 6144, 4096), (4096, 6144, 4096)])
+@pytest.mark.parametrize("shape", [(512, 768, 1024), (16, 4096, 4096), (512, 6144, 4096), (4096, 6144, 4096), (8704, 4096, 2496)])
 def test_bf16_gemm_replays(shape):
-    """Tile kernel, streaming kernel with its K split, tile kernel with K split and with tail split."""
+    """Tile kernel, streaming kernel with its K split, tile kernel with K split and with tail split, and a problem that
+    runs as two launches, the second with a K split."""
     M, N, K = shape
     A = torch.randn(M, K, device="cuda").bfloat16()
     B = torch.randn(N, K, device="cuda").bfloat16()
